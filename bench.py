@@ -1,0 +1,212 @@
+"""Benchmark of the compressed-expert hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one pass of the grouped expert launch over one batch of synthetic
+tokens.  The default workload is the Switch-c-2048 MoE layer swept with one
+token per expert (2048 experts, wi 6144x2080 and wo 2080x6144 each, about
+4.6 GB of compressed weights: larger than every cache, so the rate is an HBM
+rate).  Prints ONE JSON line: microseconds per layer, the achieved rate on
+algorithmic (compressed) bytes against the 8 TB/s HBM peak, and the CPU
+oracle timed on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (shape key, experts, p_zero, description)
+    'c2048-sweep': ('c2048', 2048, 0.90,
+                    'Switch-c-2048 MoE layer, 2048 experts, 1 token per expert (sweep)'),
+    'large128': ('large', 128, 0.88, 'Switch-large-128 MoE layer, 1 token per expert'),
+    'base128': ('base', 128, 0.90, 'Switch-base-128 MoE layer, 1 token per expert'),
+}
+
+
+def algorithmic_bytes(stack, experts_used):
+    """Bytes the products of one launch have to read and write (per product:
+    2*codes + 4*(H+1) row offsets + 4*H min/max + 2*W input + 2*H output), plus
+    the 256 KiB slot table once per launch."""
+    total = 256 * 1024
+    for e in experts_used:
+        total += 2 * int(stack.wi_codes[e]) + 2 * int(stack.wo_codes[e])
+        for h, w in ((stack.d_ff, stack.d_model), (stack.d_model, stack.d_ff)):
+            total += 4 * (h + 1) + 4 * h + 2 * w + 2 * h
+    return total
+
+
+def time_launches(fn, steps, warmup, stream_ptr):
+    """(wall seconds for `steps` calls, average microseconds per call from HIP
+    events recorded on the launch stream)."""
+    import ctypes
+    import torch
+    from qmoe_amd import _lib
+    lib = _lib.load()
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    tick = time.perf_counter()
+    _lib.check(lib.sub1_timing_begin(stream_ptr))
+    for _ in range(steps):
+        fn()
+    us = ctypes.c_double()
+    _lib.check(lib.sub1_timing_end(stream_ptr, ctypes.byref(us)))
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - tick
+    return wall, us.value / steps
+
+
+def cpu_baseline(stack, x, sample_experts, budget_s=12.0):
+    """The CPU oracle's reference-order decode+matvec (a scalar C port of the
+    reference kernel's arithmetic, one core) on the first experts of the same
+    stack, extrapolated to the whole layer."""
+    import numpy as np
+    import torch
+    from oracle import sub1_oracle as so
+    from qmoe_amd import synthetic
+    o = so.COracle()
+    o.tables()
+    done, spent = 0, 0.0
+    for e in range(sample_experts):
+        wi, wo = synthetic.expert_layers(stack, e)
+        host = [tuple(t.view(torch.int16).cpu().numpy().view(np.uint16) if t.dtype != torch.int32
+                      else t.cpu().numpy() for t in l) for l in (wi, wo)]
+        xe = x[e].view(torch.int16).cpu().numpy().view(np.uint16)
+        tick = time.perf_counter()
+        o.expert_ffn(host[0], host[1], xe, order=0)
+        spent += time.perf_counter() - tick
+        done += 1
+        if spent > budget_s:
+            break
+    return done, spent
+
+
+def dense_gemv_us(stack, x, experts):
+    """Dense bf16 batched GEMV (torch.bmm -> hipBLASLt/rocBLAS) on the decoded
+    weights of the first `experts` experts, microseconds per expert FFN."""
+    import torch
+    from qmoe_amd import sub1_hip, synthetic
+    wis, wos = [], []
+    for e in range(experts):
+        wi, wo = synthetic.expert_layers(stack, e)
+        wis.append(sub1_hip.sub1decode(stack.dec, wi[0], wi[1], wi[2], stack.d_model,
+                                       want_tern=False)[1])
+        wos.append(sub1_hip.sub1decode(stack.dec, wo[0], wo[1], wo[2], stack.d_ff,
+                                       want_tern=False)[1])
+    wi = torch.stack(wis)
+    wo = torch.stack(wos)
+    del wis, wos
+    xv = x[:experts].unsqueeze(2).contiguous()
+
+    def run():
+        h = torch.relu(torch.bmm(wi, xv))
+        return torch.bmm(wo, h)
+
+    for _ in range(3):
+        run()
+    torch.cuda.synchronize()
+    tick = time.perf_counter()
+    reps = 10
+    for _ in range(reps):
+        run()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - tick) / reps / experts * 1e6
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--warmup', type=int, default=3)
+    ap.add_argument('--workload', default='c2048-sweep', choices=sorted(WORKLOADS))
+    ap.add_argument('--experts', type=int, default=0, help='override the expert count (debugging)')
+    ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline')
+    ap.add_argument('--no-dense', action='store_true', help='skip the dense bf16 comparison')
+    ap.add_argument('--seed', type=int, default=20231116)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit('bench.py measures one GPU: this build has no multi-GPU path (--gpus 1 only)')
+
+    import ctypes
+    import torch
+    from qmoe_amd import synthetic
+
+    shape, experts, p_zero, desc = WORKLOADS[args.workload]
+    if args.experts:
+        experts = args.experts
+        desc += ' [reduced to %d experts]' % experts
+    d_model, d_ff = synthetic.SHAPES[shape]
+    torch.cuda.set_device(0)
+    tick = time.perf_counter()
+    stack = synthetic.build_stack(experts, d_model, d_ff, p_zero, args.seed)
+    torch.cuda.synchronize()
+    print('built %d experts in %.1f s, %.3f GB compressed' %
+          (experts, time.perf_counter() - tick, stack.compressed_bytes() / 1e9), file=sys.stderr)
+
+    x = synthetic.activations(experts, d_model, args.seed + 1)
+    route = torch.arange(experts, dtype=torch.int32, device='cuda')
+    y = torch.empty_like(x)
+    stream_ptr = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    wall, us_launch = time_launches(lambda: stack.forward(x, route, y), args.steps,
+                                    args.warmup, stream_ptr)
+    assert stack.launch_faults(experts) == (0, 0)
+    ms_per_step = wall / args.steps * 1e3
+    abytes = algorithmic_bytes(stack, range(experts))
+    achieved = abytes / (us_launch * 1e-6) / 1e9
+
+    out = {
+        'metric': 'us per compressed MoE layer (batch-1) + achieved HBM GB/s vs roofline',
+        'value': round(ms_per_step * 1e3, 2),
+        'unit': 'us/layer',
+        'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': round(ms_per_step, 4),
+        'higher_is_better': False, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'bf16 in/out, fp32 accumulate, u16 codes',
+        'data': 'synthetic (seeded iid ternary experts, N(0,1) bf16 tokens)',
+        'config': {'workload': desc, 'experts': experts, 'd_model': d_model, 'd_ff': d_ff,
+                   'p_zero': p_zero, 'tokens': experts,
+                   'compressed_bytes': stack.compressed_bytes(),
+                   'bits_per_weight': round(16.0 * stack.w_comp.numel()
+                                            / (2.0 * experts * d_model * d_ff), 4)},
+        'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS,
+                     'unit': 'GB/s', 'frac': round(achieved / HBM_PEAK_GBS, 4),
+                     'traffic': None, 'kernel': 'moe_kernel',
+                     'algorithmic_bytes': abytes, 'us_per_launch': round(us_launch, 2)},
+    }
+
+    also = {}
+    # batch-1: one token routed to one seeded uniform expert (launch-latency bound)
+    g = torch.Generator().manual_seed(args.seed + 2)
+    one = torch.randint(0, experts, (1,), generator=g).to(torch.int32).cuda()
+    _, us1 = time_launches(lambda: stack.forward(x[:1], one, y[:1]), 200, 20, stream_ptr)
+    also['single_token_us'] = round(us1, 2)
+    if not args.no_dense:
+        n = min(experts, 128)
+        d_us = dense_gemv_us(stack, x, n)
+        also['dense_bf16_gemv'] = {'us_per_expert_ffn': round(d_us, 2), 'experts_timed': n,
+                                   'us_per_layer_extrapolated': round(d_us * experts, 1),
+                                   'sub1_us_per_expert_ffn': round(us_launch / experts, 2)}
+    out['also'] = also
+
+    if not args.no_cpu:
+        done, spent = cpu_baseline(stack, x, min(experts, 64))
+        out['cpu_baseline'] = {
+            'value': round(spent / done * experts * 1e6, 1), 'unit': 'us/layer', 'cores': 1,
+            'kind': 'port',
+            'sample': '%d of %d expert FFNs of the same stack through the scalar C oracle in '
+                      'the reference kernel\'s lane order, %.1f s, extrapolated to the layer'
+                      % (done, experts, spent)}
+    print(json.dumps(out))
+
+
+if __name__ == '__main__':
+    main()

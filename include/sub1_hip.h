@@ -1,0 +1,164 @@
+/*
+ * libsub1_hip - C ABI of the gfx950 (MI355X) implementation of QMoE's
+ * compressed-expert operator: dictionary decode fused with matrix-vector
+ * product over ternary expert weights coded as 16-bit dictionary indices.
+ *
+ * The entry points are what a binding for the reference's `sub1_cuda`
+ * extension (reference sub1_cuda.cpp:35-59) would call: plain pointers and
+ * sizes, no torch types.  All device pointers must belong to the device that
+ * is current when the function is called; `stream` is a hipStream_t passed as
+ * void* (NULL = the null stream).  Functions return SUB1_OK or a negative
+ * status; sub1_last_error() gives the message for the calling thread.  No
+ * function synchronises the device unless stated.
+ *
+ * Data layout (reference sub1.py:114-130, identical here):
+ *   dec         int32 [131072]   decode table, entry e = words 2e, 2e+1
+ *   trie        int32 [65537*9]  encode trie, root at row 65536
+ *   w_comp      int16 [C]        codeword stream, rows back to back
+ *   row_off     int32 [H+1]      cumulative codeword count, row_off[0] = 0
+ *   ter_minmax  bf16  [2H]       (min, max) of row r at 2r, 2r+1
+ *   x           bf16  [W]        activations
+ *   y           bf16  [H]        output, ACCUMULATED INTO (y += W x)
+ */
+#ifndef SUB1_HIP_H_
+#define SUB1_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SUB1_OK 0
+#define SUB1_ERR_NULL (-1)       /* a required pointer is NULL */
+#define SUB1_ERR_SHAPE (-2)      /* height/width/count out of the supported range */
+#define SUB1_ERR_ALIGN (-3)      /* a pointer is not aligned for its element type */
+#define SUB1_ERR_HIP (-4)        /* a HIP runtime call failed */
+#define SUB1_ERR_INTERNAL (-5)
+
+#define SUB1_DICT_ENTRIES 65536              /* reference sub1.py:30 */
+#define SUB1_DEC_WORDS (2 * SUB1_DICT_ENTRIES)
+#define SUB1_TRIE_ROWS (SUB1_DICT_ENTRIES + 1)
+#define SUB1_TRIE_WORDS (9 * SUB1_TRIE_ROWS)
+#define SUB1_MAX_WIDTH 12288                 /* x is staged in LDS */
+
+/* Message of the last failure on this thread ("" if none). */
+const char *sub1_last_error(void);
+
+/* ABI version, bumped on any signature change. */
+int sub1_abi_version(void);
+
+/*
+ * Build the fixed dictionary on the HOST: dec_host[131072], trie_host[65537*9].
+ * Either may be NULL.  Replaces the Python `setup()` of reference
+ * sub1.py:29-102 (same table bytes).  Deterministic, no GPU needed.
+ */
+int sub1_build_tables(int32_t *dec_host, int32_t *trie_host);
+
+/*
+ * y[r] += bf16( sum_k deq(w[r,k]) * x[k] ),  fp32 accumulation, for any
+ * height >= 1 and 1 <= width <= SUB1_MAX_WIDTH.  Replaces `sub1matvec`
+ * (reference sub1_cuda.cpp:35-45, sub1_cuda_kernel.cu:70-88,129-202), which
+ * handled six hard-coded shapes and silently did nothing for others.
+ * The first call with a given `dec` pointer derives a compact device table
+ * from it (one small kernel and one allocation, cached for the process; the
+ * contents of `dec` must not change afterwards).
+ */
+int sub1_matvec(const int32_t *dec, const int16_t *w_comp, const int32_t *row_off,
+                const void *ter_minmax, const void *x, void *y, int height,
+                int width, void *stream);
+
+/*
+ * T products with one matrix: y[t, :] += W x[t, :], x row stride `ldx`, y row
+ * stride `ldy` (elements).  One launch; what the token loop of reference
+ * sub1.py:139-142 does with T launches.
+ */
+int sub1_matvec_tokens(const int32_t *dec, const int16_t *w_comp,
+                       const int32_t *row_off, const void *ter_minmax,
+                       const void *x, void *y, int height, int width,
+                       int tokens, int64_t ldx, int64_t ldy, void *stream);
+
+/*
+ * Encoder, phase 1.  Replaces `Sub1PreparePack` plus the cumulative sum of
+ * reference sub1_cuda_kernel.cu:103-112,211-239: greedy longest-match parse
+ * of every row of w_tern (int32 [H, W], symbols 0/1/2).  w_tern is
+ * OVERWRITTEN with the row's codes (row r's codes at w_tern[r*W ...]) and
+ * row_off [H+1] receives the cumulative counts.  The caller then reads
+ * row_off[H] (a device-to-host copy, as the reference does at
+ * sub1_cuda_kernel.cu:115) to size w_comp.
+ */
+int sub1_pack_count(const int32_t *trie, int32_t *w_tern, int32_t *row_off,
+                    int height, int width, void *stream);
+
+/*
+ * Encoder, phase 2.  Replaces `Sub1Pack` (reference
+ * sub1_cuda_kernel.cu:241-250): compacts the codes left in w_tern by
+ * sub1_pack_count into w_comp[row_off[r] + i].
+ */
+int sub1_pack_emit(const int32_t *w_tern, const int32_t *row_off, int16_t *w_comp,
+                   int height, int width, void *stream);
+
+/*
+ * Decoder without the product, for checking: out_tern (uint8 [H, W], symbols)
+ * and/or out_w (bf16 [H, W], dequantised weights) may each be NULL.  What the
+ * Python `decompress` of reference test.py:103-115 computes.
+ * bad_rows (int32 [1], device, may be NULL) is incremented for every row whose
+ * codes do not cover exactly the row width.
+ */
+int sub1_decode(const int32_t *dec, const int16_t *w_comp, const int32_t *row_off,
+                const void *ter_minmax, uint8_t *out_tern, void *out_w,
+                int32_t *bad_rows, int height, int width, void *stream);
+
+/*
+ * One MoE layer's expert FFNs in ONE persistent launch: for every token t
+ * with expert e = token_expert[t] >= 0,
+ *     y[t] = wo_e( relu( wi_e( x[t] ) ) )      (h is rounded to bf16 between)
+ * and y[t] = x[t] for tokens with token_expert[t] < 0 (tokens the router
+ * dropped keep their input, reference sub1.py:312).  Replaces the per-expert
+ * Python loop of reference sub1.py:315-317 and the two launches per token
+ * inside it.  Unlike sub1_matvec, y is OVERWRITTEN.
+ *
+ * The stack is the experts' Sub1Linear buffers back to back:
+ *   w_comp            int16, all streams in one buffer
+ *   wi_code_base[e]   int64 [E]  first codeword of expert e's wi stream
+ *   wo_code_base[e]   int64 [E]  likewise for wo
+ *   wi_row_off        int32 [E, d_ff+1]     each row starts at 0
+ *   wo_row_off        int32 [E, d_model+1]
+ *   wi_minmax         bf16  [E, 2*d_ff]
+ *   wo_minmax         bf16  [E, 2*d_model]
+ * workspace: sub1_moe_workspace_bytes(tokens, d_ff) bytes of device memory,
+ * 256-byte aligned, contents irrelevant on entry.
+ */
+typedef struct sub1_moe_stack {
+  const int32_t *dec;
+  const int16_t *w_comp;
+  const int64_t *wi_code_base;
+  const int64_t *wo_code_base;
+  const int32_t *wi_row_off;
+  const int32_t *wo_row_off;
+  const void *wi_minmax;
+  const void *wo_minmax;
+  int32_t experts;
+  int32_t d_model;
+  int32_t d_ff;
+} sub1_moe_stack;
+
+int64_t sub1_moe_workspace_bytes(int tokens, int d_ff);
+
+int sub1_moe_grouped(const sub1_moe_stack *stack, const int32_t *token_expert,
+                     const void *x, void *y, int tokens, void *workspace,
+                     int64_t workspace_bytes, void *stream);
+
+/*
+ * Average duration in microseconds of the most recent launches, measured with
+ * HIP events on the launch stream: call sub1_timing_begin(stream) before and
+ * sub1_timing_end(stream, &us) after a run of launches (end synchronises).
+ * For benchmarks; not thread safe.
+ */
+int sub1_timing_begin(void *stream);
+int sub1_timing_end(void *stream, double *elapsed_us);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SUB1_HIP_H_ */

@@ -1,0 +1,72 @@
+"""ctypes binding of libsub1_hip.so (the C ABI declared in include/sub1_hip.h)."""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, 'libsub1_hip.so')
+
+SUB1_OK = 0
+DICT_ENTRIES = 65536
+DEC_WORDS = 2 * DICT_ENTRIES
+TRIE_ROWS = DICT_ENTRIES + 1
+MAX_WIDTH = 12288
+
+_vp = ctypes.c_void_p
+_int = ctypes.c_int
+_i64 = ctypes.c_int64
+
+
+class MoeStack(ctypes.Structure):
+    """struct sub1_moe_stack"""
+    _fields_ = [('dec', _vp), ('w_comp', _vp), ('wi_code_base', _vp),
+                ('wo_code_base', _vp), ('wi_row_off', _vp), ('wo_row_off', _vp),
+                ('wi_minmax', _vp), ('wo_minmax', _vp), ('experts', ctypes.c_int32),
+                ('d_model', ctypes.c_int32), ('d_ff', ctypes.c_int32)]
+
+
+# every symbol include/sub1_hip.h declares, with its prototype
+PROTOTYPES = {
+    'sub1_last_error': (ctypes.c_char_p, []),
+    'sub1_abi_version': (_int, []),
+    'sub1_build_tables': (_int, [_vp, _vp]),
+    'sub1_matvec': (_int, [_vp] * 6 + [_int, _int, _vp]),
+    'sub1_matvec_tokens': (_int, [_vp] * 6 + [_int, _int, _int, _i64, _i64, _vp]),
+    'sub1_pack_count': (_int, [_vp, _vp, _vp, _int, _int, _vp]),
+    'sub1_pack_emit': (_int, [_vp, _vp, _vp, _int, _int, _vp]),
+    'sub1_decode': (_int, [_vp] * 7 + [_int, _int, _vp]),
+    'sub1_moe_workspace_bytes': (_i64, [_int, _int]),
+    'sub1_moe_grouped': (_int, [ctypes.POINTER(MoeStack), _vp, _vp, _vp, _int, _vp,
+                                _i64, _vp]),
+    'sub1_timing_begin': (_int, [_vp]),
+    'sub1_timing_end': (_int, [_vp, ctypes.POINTER(ctypes.c_double)]),
+}
+
+_lib = None
+
+
+class Sub1Error(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__('libsub1_hip status %d: %s' % (status, message))
+        self.status = status
+
+
+def load():
+    """The loaded library.  There is no fallback: a missing library is an error."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                '%s is missing: build it with `python -m qmoe_amd.build` '
+                '(hipcc, gfx950); there is no CPU fallback' % LIB_PATH)
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in PROTOTYPES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = lib
+    return _lib
+
+
+def check(status):
+    if status != SUB1_OK:
+        raise Sub1Error(status, load().sub1_last_error().decode())

@@ -1,0 +1,710 @@
+// gfx950 kernels and C ABI of libsub1_hip: decode-fused matrix-vector product
+// over dictionary-coded ternary weights, the encoder, a plain decoder and the
+// grouped expert-FFN launch.  Written for 64-wide wavefronts: one LANE walks
+// one ROW of the matrix, so a wavefront advances 64 independent code streams,
+// there is no cross-lane reduction, and work per codeword is proportional to
+// the non-zero weights in it (at most three for the fixed dictionary).
+//
+// Reference behaviour being reproduced (not its implementation):
+//   sub1_cuda_kernel.cu:129-202  Sub1MatVec       -> matvec_kernel / moe_kernel
+//   sub1_cuda_kernel.cu:211-239  Sub1PreparePack  -> pack_count_kernel
+//   sub1_cuda_kernel.cu:241-250  Sub1Pack         -> pack_emit_kernel
+//   test.py:103-115              decompress       -> decode_kernel
+//   sub1.py:306-321              expert loop      -> moe_kernel
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "sub1_hip.h"
+
+namespace {
+
+// ------------------------------------------------------------ host errors --
+
+thread_local std::string g_err;
+
+int fail(int code, const char *fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_err = buf;
+  return code;
+}
+
+#define HIP_TRY(expr)                                                          \
+  do {                                                                         \
+    hipError_t e_ = (expr);                                                    \
+    if (e_ != hipSuccess)                                                      \
+      return fail(SUB1_ERR_HIP, "%s: %s", #expr, hipGetErrorString(e_));       \
+  } while (0)
+
+// ---------------------------------------------------------- device helpers --
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) {
+  return __uint_as_float(static_cast<uint32_t>(h) << 16);
+}
+
+// round-to-nearest-even (what __float2bfloat16 in the reference kernel does)
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<uint16_t>(u >> 16);
+}
+
+// ------------------------------------------------------------ slot table ---
+//
+// The reference table spends two 32-bit words per entry on 28 two-bit digits
+// of which at most three are non-zero.  The kernels use a derived one-word
+// form that lists the non-zeros:
+//   bits 0-3          pair count L (the entry spans 2L weights)
+//   bits 4+7j..10+7j  slot j = 3*pos + sym  (pos 0..27, sym 1 = row min,
+//                     2 = row max), 0 = no further non-zero
+// 3*pos+sym is directly an offset into the tripled activation array below.
+constexpr int kSlots = 3;
+constexpr int kSlotBits = 7;
+constexpr uint32_t kSlotMask = (1u << kSlotBits) - 1;
+
+__global__ void derive_slot_table_kernel(const int32_t *__restrict__ dec,
+                                         uint32_t *__restrict__ tab,
+                                         int32_t *__restrict__ unsupported) {
+  int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= SUB1_DICT_ENTRIES) return;
+  uint32_t w0 = static_cast<uint32_t>(dec[2 * e]);
+  uint32_t w1 = static_cast<uint32_t>(dec[2 * e + 1]);
+  uint32_t out = w0 & 0xfu;
+  int n = 0;
+  bool bad = false;
+  for (int d = 0; d < 28; d++) {
+    uint32_t w = d < 14 ? w0 : w1;
+    uint32_t t = (w >> (4 + 2 * (d % 14))) & 3u;
+    if (t == 0) continue;
+    if (t == 3 || n == kSlots) {
+      bad = true;
+      break;
+    }
+    out |= static_cast<uint32_t>(3 * d + t) << (4 + kSlotBits * n);
+    n++;
+  }
+  tab[e] = out;
+  if (bad) atomicOr(unsupported, 1);
+}
+
+// ----------------------------------------------- activations in LDS --------
+//
+// x is kept in LDS as fp32, tripled:  M[3k] = 0, M[3k+1] = x[k], M[3k+2] = 0.
+// Reading the pair (M[i], M[i-1]) at i = 3k+sym gives (x,0) for sym 1, (0,x)
+// for sym 2 and (0,0) for an empty slot (i = 3k), so a slot costs two adds and
+// no select; the pair is one ds_read2_b32.  One spare dword in front makes
+// M[-1] readable, and 28 zero columns behind the row cover the digits of a
+// last codeword that hang over the row end (the reference pads the same way,
+// sub1_cuda_kernel.cu:147-151).
+__host__ __device__ constexpr int lds_dwords_for_width(int width) {
+  return 1 + 3 * (width + 28) + 3;
+}
+
+template <int kThreads>
+__device__ __forceinline__ void stage_activations(float *lds, const uint16_t *x,
+                                                  int width) {
+  const int n = width + 29;
+  if (threadIdx.x == 0) lds[0] = 0.f;
+  for (int k = threadIdx.x; k < n; k += kThreads) {
+    float v = k < width ? bf16_to_f32(x[k]) : 0.f;
+    float *m = lds + 1 + 3 * k;
+    m[0] = 0.f;
+    m[1] = v;
+    m[2] = 0.f;
+  }
+}
+
+// One codeword: three slots, then advance the column (in dwords of M).
+__device__ __forceinline__ void add_codeword(uint32_t e, const float *M, int &colw,
+                                             float &s1, float &s2) {
+#pragma unroll
+  for (int j = 0; j < kSlots; j++) {
+    int idx = colw + static_cast<int>((e >> (4 + kSlotBits * j)) & kSlotMask);
+    s1 += M[idx];
+    s2 += M[idx - 1];
+  }
+  colw += static_cast<int>(e & 0xfu) * 6;
+}
+
+__device__ __forceinline__ void load_codes8(const uint16_t *p, uint32_t (&w)[4]) {
+  // the stream is only 2-byte aligned; gfx950 global loads take any alignment
+  __builtin_memcpy(w, p, 16);
+}
+
+// Sum of activations under the symbol-1 and symbol-2 weights of one row, each
+// in fp32 in column order.
+__device__ __forceinline__ void row_sums(const uint32_t *__restrict__ tab,
+                                         const uint16_t *__restrict__ codes, int len,
+                                         const float *M, float &s1, float &s2) {
+  s1 = 0.f;
+  s2 = 0.f;
+  int colw = 0;
+  int i = 0;
+  uint32_t w[4];
+  if (len >= 8) load_codes8(codes, w);
+  for (; i + 8 <= len; i += 8) {
+    uint32_t cur[4] = {w[0], w[1], w[2], w[3]};
+    if (i + 16 <= len) load_codes8(codes + i + 8, w);
+    uint32_t e[8];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      e[2 * j] = tab[cur[j] & 0xffffu];
+      e[2 * j + 1] = tab[cur[j] >> 16];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++) add_codeword(e[j], M, colw, s1, s2);
+  }
+  int rem = len - i;
+  if (rem > 0) {
+    if (len >= 8) {
+      // the row's last eight codes; the first 8-rem of them are already done
+      load_codes8(codes + len - 8, w);
+      int skip = 8 - rem;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        uint32_t code = (j & 1) ? (w[j / 2] >> 16) : (w[j / 2] & 0xffffu);
+        uint32_t e = tab[code];
+        if (j < skip) e = 0u;  // entry 0 of the slot form: nothing, no advance
+        add_codeword(e, M, colw, s1, s2);
+      }
+    } else {
+      for (int j = 0; j < rem; j++) add_codeword(tab[codes[j]], M, colw, s1, s2);
+    }
+  }
+}
+
+__device__ __forceinline__ float row_result(uint32_t minmax, float s1, float s2) {
+  float mn = __uint_as_float(minmax << 16);
+  float mx = __uint_as_float(minmax & 0xffff0000u);
+  return __fmaf_rn(mn, s1, __fmul_rn(mx, s2));
+}
+
+// ------------------------------------------------------------- matvec ------
+
+template <int kThreads>
+__global__ __launch_bounds__(kThreads) void matvec_kernel(
+    const uint32_t *__restrict__ tab, const uint16_t *__restrict__ w_comp,
+    const int32_t *__restrict__ row_off, const uint32_t *__restrict__ minmax,
+    const uint16_t *__restrict__ x, uint16_t *__restrict__ y, int height, int width,
+    int64_t ldx, int64_t ldy) {
+  extern __shared__ float lds[];
+  x += static_cast<int64_t>(blockIdx.y) * ldx;
+  y += static_cast<int64_t>(blockIdx.y) * ldy;
+  stage_activations<kThreads>(lds, x, width);
+  __syncthreads();
+  const int row = blockIdx.x * kThreads + threadIdx.x;
+  if (row >= height) return;
+  const int off = row_off[row];
+  const int len = row_off[row + 1] - off;
+  float s1, s2;
+  row_sums(tab, w_comp + off, len, lds + 1, s1, s2);
+  float res = row_result(minmax[row], s1, s2);
+  // reference sub1_cuda_kernel.cu:200: y[row] += bf16(res), the sum in bf16
+  float acc = bf16_to_f32(y[row]) + bf16_to_f32(f32_to_bf16(res));
+  y[row] = f32_to_bf16(acc);
+}
+
+// ------------------------------------------------------------- decode ------
+
+__global__ void decode_kernel(const int32_t *__restrict__ dec,
+                              const uint16_t *__restrict__ w_comp,
+                              const int32_t *__restrict__ row_off,
+                              const uint32_t *__restrict__ minmax,
+                              uint8_t *__restrict__ out_tern,
+                              uint16_t *__restrict__ out_w,
+                              int32_t *__restrict__ bad_rows, int height, int width) {
+  int row = blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= height) return;
+  uint16_t deq[3] = {0, 0, 0};
+  if (minmax) {
+    uint32_t mm = minmax[row];
+    deq[1] = static_cast<uint16_t>(mm & 0xffffu);
+    deq[2] = static_cast<uint16_t>(mm >> 16);
+  }
+  int64_t base = static_cast<int64_t>(row) * width;
+  int idx = 0;
+  for (int c = row_off[row]; c < row_off[row + 1]; c++) {
+    int e = w_comp[c];
+    uint32_t w0 = static_cast<uint32_t>(dec[2 * e]);
+    uint32_t w1 = static_cast<uint32_t>(dec[2 * e + 1]);
+    int n = 2 * static_cast<int>(w0 & 0xfu);
+    for (int d = 0; d < n; d++) {
+      if (idx + d >= width) break;
+      uint32_t w = d < 14 ? w0 : w1;
+      uint32_t t = (w >> (4 + 2 * (d % 14))) & 3u;
+      if (out_tern) out_tern[base + idx + d] = static_cast<uint8_t>(t);
+      if (out_w) out_w[base + idx + d] = t < 3 ? deq[t] : 0;
+    }
+    idx += n;
+  }
+  if (idx != ((width + 1) & ~1) && bad_rows) atomicAdd(bad_rows, 1);
+}
+
+// --------------------------------------------------------------- pack ------
+
+constexpr int kTrieRoot = SUB1_DICT_ENTRIES;
+
+__global__ void pack_count_kernel(const int32_t *__restrict__ trie,
+                                  int32_t *__restrict__ w_tern,
+                                  int32_t *__restrict__ row_cnt, int height,
+                                  int width) {
+  int row = blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= height) return;
+  int32_t *w = w_tern + static_cast<int64_t>(row) * width;
+  int node = kTrieRoot;
+  int n = 0;
+  for (int i = 0; i < width; i += 2) {
+    int lo = w[i];
+    int hi = i + 1 < width ? w[i + 1] : 0;
+    int sym = 3 * hi + lo;
+    int child = trie[9 * node + sym];
+    if (child < 0) {
+      // n <= i/2 < i: the slot written was already consumed
+      w[n++] = node;
+      child = trie[9 * kTrieRoot + sym];
+    }
+    node = child;
+  }
+  w[n++] = node;
+  row_cnt[row + 1] = n;
+}
+
+// Inclusive prefix sum over cnt[1..height] in place, cnt[0] = 0.  One
+// workgroup; each thread owns a contiguous segment.
+constexpr int kScanThreads = 1024;
+
+__global__ __launch_bounds__(kScanThreads) void row_offset_scan_kernel(
+    int32_t *__restrict__ cnt, int height) {
+  __shared__ int32_t part[kScanThreads];
+  const int tid = threadIdx.x;
+  const int seg = (height + kScanThreads - 1) / kScanThreads;
+  const int lo = 1 + tid * seg;
+  const int hi = min(height + 1, lo + seg);
+  int32_t s = 0;
+  for (int i = lo; i < hi; i++) s += cnt[i];
+  part[tid] = s;
+  __syncthreads();
+  for (int d = 1; d < kScanThreads; d *= 2) {
+    int32_t v = tid >= d ? part[tid - d] : 0;
+    __syncthreads();
+    part[tid] += v;
+    __syncthreads();
+  }
+  int32_t run = tid ? part[tid - 1] : 0;
+  if (tid == 0) cnt[0] = 0;
+  for (int i = lo; i < hi; i++) {
+    run += cnt[i];
+    cnt[i] = run;
+  }
+}
+
+__global__ void pack_emit_kernel(const int32_t *__restrict__ w_codes,
+                                 const int32_t *__restrict__ row_off,
+                                 uint16_t *__restrict__ w_comp, int height,
+                                 int width) {
+  // one wavefront per row, lanes stride over the row's codes
+  int row = blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64;
+  if (row >= height) return;
+  int lane = threadIdx.x % 64;
+  int off = row_off[row];
+  int n = row_off[row + 1] - off;
+  const int32_t *src = w_codes + static_cast<int64_t>(row) * width;
+  for (int i = lane; i < n; i += 64)
+    w_comp[off + i] = static_cast<uint16_t>(src[i]);
+}
+
+// ------------------------------------------------------ grouped experts ----
+//
+// Persistent grid.  Work is cut into tiles (token, projection, block of
+// kThreads rows), numbered with all wi tiles before all wo tiles, and handed
+// out by an atomic ticket.  A wo tile of token t needs all of h[t], so it
+// waits until the wi tiles of t have signalled; those have smaller tickets,
+// were therefore taken by workgroups that are already running, and never wait
+// themselves, so the wait always ends.
+struct MoeArgs {
+  const uint32_t *tab;
+  const uint16_t *w_comp;
+  const int64_t *wi_code_base;
+  const int64_t *wo_code_base;
+  const int32_t *wi_row_off;
+  const int32_t *wo_row_off;
+  const uint32_t *wi_minmax;
+  const uint32_t *wo_minmax;
+  const int32_t *token_expert;
+  const uint16_t *x;
+  uint16_t *y;
+  uint16_t *h;
+  int32_t *ctrl;  // [0] ticket, [1] wait-limit hits, [2] tokens with an expert
+                  // id >= experts (treated as dropped), [4+t] wi tiles done for t
+  int tokens, d_model, d_ff, experts;
+  int wi_tiles, wo_tiles;  // per token
+  int spin_limit;
+};
+
+constexpr int kCtrlHeader = 4;
+
+template <int kThreads>
+__global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
+  extern __shared__ float lds[];
+  __shared__ int s_ticket;
+  const int n_wi = a.tokens * a.wi_tiles;
+  const int n_all = n_wi + a.tokens * a.wo_tiles;
+  for (;;) {
+    __syncthreads();  // previous tile's readers of lds and s_ticket are done
+    if (threadIdx.x == 0)
+      s_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const int ticket = s_ticket;
+    if (ticket >= n_all) break;
+
+    if (ticket < n_wi) {
+      const int t = ticket / a.wi_tiles;
+      const int blk = ticket - t * a.wi_tiles;
+      int e = a.token_expert[t];
+      if (e >= a.experts) e = -1;
+      if (e >= 0) {
+        stage_activations<kThreads>(lds, a.x + static_cast<int64_t>(t) * a.d_model,
+                                    a.d_model);
+        __syncthreads();
+        const int row = blk * kThreads + threadIdx.x;
+        if (row < a.d_ff) {
+          const int32_t *ro = a.wi_row_off + static_cast<int64_t>(e) * (a.d_ff + 1);
+          const int off = ro[row];
+          const int len = ro[row + 1] - off;
+          float s1, s2;
+          row_sums(a.tab, a.w_comp + a.wi_code_base[e] + off, len, lds + 1, s1, s2);
+          float res = row_result(
+              a.wi_minmax[static_cast<int64_t>(e) * a.d_ff + row], s1, s2);
+          uint16_t hb = f32_to_bf16(res);
+          if (hb & 0x8000u) hb = 0;  // relu
+          a.h[static_cast<int64_t>(t) * a.d_ff + row] = hb;
+        }
+        __threadfence();
+      }
+      __syncthreads();
+      if (threadIdx.x == 0)
+        __hip_atomic_fetch_add(&a.ctrl[kCtrlHeader + t], 1, __ATOMIC_RELEASE,
+                               __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+      const int j = ticket - n_wi;
+      const int t = j / a.wo_tiles;
+      const int blk = j - t * a.wo_tiles;
+      int e = a.token_expert[t];
+      if (e >= a.experts) {
+        if (blk == 0 && threadIdx.x == 0)
+          __hip_atomic_fetch_add(&a.ctrl[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        e = -1;
+      }
+      const int row = blk * kThreads + threadIdx.x;
+      if (e < 0) {
+        if (row < a.d_model) {
+          int64_t i = static_cast<int64_t>(t) * a.d_model + row;
+          a.y[i] = a.x[i];
+        }
+        continue;
+      }
+      if (threadIdx.x == 0) {
+        int spins = 0;
+        while (__hip_atomic_load(&a.ctrl[kCtrlHeader + t], __ATOMIC_ACQUIRE,
+                                 __HIP_MEMORY_SCOPE_AGENT) < a.wi_tiles) {
+          if (++spins > a.spin_limit) {
+            __hip_atomic_fetch_add(&a.ctrl[1], 1, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            break;
+          }
+          __builtin_amdgcn_s_sleep(8);
+        }
+      }
+      __syncthreads();
+      __threadfence();
+      stage_activations<kThreads>(lds, a.h + static_cast<int64_t>(t) * a.d_ff, a.d_ff);
+      __syncthreads();
+      if (row < a.d_model) {
+        const int32_t *ro = a.wo_row_off + static_cast<int64_t>(e) * (a.d_model + 1);
+        const int off = ro[row];
+        const int len = ro[row + 1] - off;
+        float s1, s2;
+        row_sums(a.tab, a.w_comp + a.wo_code_base[e] + off, len, lds + 1, s1, s2);
+        float res = row_result(
+            a.wo_minmax[static_cast<int64_t>(e) * a.d_model + row], s1, s2);
+        a.y[static_cast<int64_t>(t) * a.d_model + row] = f32_to_bf16(res);
+      }
+    }
+  }
+}
+
+__global__ void zero_i32_kernel(int32_t *p, int n) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// ------------------------------------------------- derived-table cache -----
+
+struct TableSlot {
+  int device;
+  const int32_t *dec;
+  uint32_t *tab;
+};
+
+std::mutex g_tab_mutex;
+std::vector<TableSlot> g_tabs;
+
+int slot_table_for(const int32_t *dec, hipStream_t stream, const uint32_t **out) {
+  int device = 0;
+  HIP_TRY(hipGetDevice(&device));
+  std::lock_guard<std::mutex> lock(g_tab_mutex);
+  for (const TableSlot &s : g_tabs)
+    if (s.device == device && s.dec == dec) {
+      *out = s.tab;
+      return SUB1_OK;
+    }
+  uint32_t *tab = nullptr;
+  HIP_TRY(hipMalloc(&tab, (SUB1_DICT_ENTRIES + 1) * sizeof(uint32_t)));
+  int32_t *flag = reinterpret_cast<int32_t *>(tab + SUB1_DICT_ENTRIES);
+  zero_i32_kernel<<<1, 64, 0, stream>>>(flag, 1);
+  derive_slot_table_kernel<<<SUB1_DICT_ENTRIES / 256, 256, 0, stream>>>(dec, tab, flag);
+  HIP_TRY(hipGetLastError());
+  int32_t bad = 0;
+  HIP_TRY(hipMemcpyAsync(&bad, flag, sizeof bad, hipMemcpyDeviceToHost, stream));
+  HIP_TRY(hipStreamSynchronize(stream));
+  if (bad) {
+    (void)hipFree(tab);
+    return fail(SUB1_ERR_SHAPE,
+                "dec holds an entry with a digit 3 or more than %d non-zero weights",
+                kSlots);
+  }
+  g_tabs.push_back({device, dec, tab});
+  *out = tab;
+  return SUB1_OK;
+}
+
+bool misaligned(const void *p, size_t a) {
+  return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0;
+}
+
+constexpr int kMatvecThreads = 256;
+constexpr int kMoeThreads = 256;
+
+template <typename K>
+int allow_lds(K kernel, size_t bytes) {
+  if (bytes > 48 * 1024)
+    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(bytes)));
+  return SUB1_OK;
+}
+
+hipEvent_t g_ev_begin = nullptr, g_ev_end = nullptr;
+
+}  // namespace
+
+// ================================================================ C ABI =====
+
+extern "C" const char *sub1_last_error(void) { return g_err.c_str(); }
+
+extern "C" int sub1_abi_version(void) { return 1; }
+
+extern "C" int sub1_matvec_tokens(const int32_t *dec, const int16_t *w_comp,
+                                  const int32_t *row_off, const void *ter_minmax,
+                                  const void *x, void *y, int height, int width,
+                                  int tokens, int64_t ldx, int64_t ldy, void *stream) {
+  if (!dec || !row_off || !ter_minmax || !x || !y)
+    return fail(SUB1_ERR_NULL, "sub1_matvec: NULL argument");
+  if (height < 1 || width < 1 || width > SUB1_MAX_WIDTH)
+    return fail(SUB1_ERR_SHAPE, "sub1_matvec: height %d width %d unsupported (width 1..%d)",
+                height, width, SUB1_MAX_WIDTH);
+  if (tokens < 0 || tokens > 65535)
+    return fail(SUB1_ERR_SHAPE, "sub1_matvec: tokens %d outside 0..65535", tokens);
+  if (tokens > 1 && (ldx < width || ldy < height))
+    return fail(SUB1_ERR_SHAPE, "sub1_matvec: row strides smaller than the rows");
+  if (!w_comp) return fail(SUB1_ERR_NULL, "sub1_matvec: NULL w_comp");
+  if (misaligned(dec, 4) || misaligned(row_off, 4) || misaligned(ter_minmax, 4) ||
+      misaligned(w_comp, 2) || misaligned(x, 2) || misaligned(y, 2))
+    return fail(SUB1_ERR_ALIGN, "sub1_matvec: misaligned pointer");
+  if (tokens == 0) return SUB1_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint32_t *tab = nullptr;
+  int rc = slot_table_for(dec, s, &tab);
+  if (rc) return rc;
+  size_t lds = lds_dwords_for_width(width) * sizeof(float);
+  rc = allow_lds(matvec_kernel<kMatvecThreads>, lds);
+  if (rc) return rc;
+  dim3 grid((height + kMatvecThreads - 1) / kMatvecThreads, tokens);
+  matvec_kernel<kMatvecThreads><<<grid, kMatvecThreads, lds, s>>>(
+      tab, reinterpret_cast<const uint16_t *>(w_comp), row_off,
+      static_cast<const uint32_t *>(ter_minmax), static_cast<const uint16_t *>(x),
+      static_cast<uint16_t *>(y), height, width, ldx, ldy);
+  HIP_TRY(hipGetLastError());
+  return SUB1_OK;
+}
+
+extern "C" int sub1_matvec(const int32_t *dec, const int16_t *w_comp,
+                           const int32_t *row_off, const void *ter_minmax,
+                           const void *x, void *y, int height, int width,
+                           void *stream) {
+  return sub1_matvec_tokens(dec, w_comp, row_off, ter_minmax, x, y, height, width, 1,
+                            width, height, stream);
+}
+
+extern "C" int sub1_pack_count(const int32_t *trie, int32_t *w_tern, int32_t *row_off,
+                               int height, int width, void *stream) {
+  if (!trie || !w_tern || !row_off) return fail(SUB1_ERR_NULL, "sub1_pack_count: NULL argument");
+  if (height < 1 || width < 1)
+    return fail(SUB1_ERR_SHAPE, "sub1_pack_count: height %d width %d", height, width);
+  if (misaligned(trie, 4) || misaligned(w_tern, 4) || misaligned(row_off, 4))
+    return fail(SUB1_ERR_ALIGN, "sub1_pack_count: misaligned pointer");
+  // the cumulative count is kept in int32 like the reference's row_off
+  if (static_cast<int64_t>(height) * ((width + 1) / 2) > INT32_MAX)
+    return fail(SUB1_ERR_SHAPE, "sub1_pack_count: more than 2^31 pairs in one call");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  pack_count_kernel<<<(height + 63) / 64, 64, 0, s>>>(trie, w_tern, row_off, height, width);
+  row_offset_scan_kernel<<<1, kScanThreads, 0, s>>>(row_off, height);
+  HIP_TRY(hipGetLastError());
+  return SUB1_OK;
+}
+
+extern "C" int sub1_pack_emit(const int32_t *w_tern, const int32_t *row_off,
+                              int16_t *w_comp, int height, int width, void *stream) {
+  if (!w_tern || !row_off || !w_comp) return fail(SUB1_ERR_NULL, "sub1_pack_emit: NULL argument");
+  if (height < 1 || width < 1)
+    return fail(SUB1_ERR_SHAPE, "sub1_pack_emit: height %d width %d", height, width);
+  if (misaligned(w_tern, 4) || misaligned(row_off, 4) || misaligned(w_comp, 2))
+    return fail(SUB1_ERR_ALIGN, "sub1_pack_emit: misaligned pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  pack_emit_kernel<<<(height + 3) / 4, 256, 0, s>>>(
+      w_tern, row_off, reinterpret_cast<uint16_t *>(w_comp), height, width);
+  HIP_TRY(hipGetLastError());
+  return SUB1_OK;
+}
+
+extern "C" int sub1_decode(const int32_t *dec, const int16_t *w_comp,
+                           const int32_t *row_off, const void *ter_minmax,
+                           uint8_t *out_tern, void *out_w, int32_t *bad_rows, int height,
+                           int width, void *stream) {
+  if (!dec || !w_comp || !row_off) return fail(SUB1_ERR_NULL, "sub1_decode: NULL argument");
+  if (out_w && !ter_minmax) return fail(SUB1_ERR_NULL, "sub1_decode: out_w needs ter_minmax");
+  if (height < 1 || width < 1)
+    return fail(SUB1_ERR_SHAPE, "sub1_decode: height %d width %d", height, width);
+  if (misaligned(dec, 4) || misaligned(row_off, 4) || misaligned(w_comp, 2) ||
+      misaligned(ter_minmax, 4) || misaligned(out_w, 2) || misaligned(bad_rows, 4))
+    return fail(SUB1_ERR_ALIGN, "sub1_decode: misaligned pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  decode_kernel<<<(height + 63) / 64, 64, 0, s>>>(
+      dec, reinterpret_cast<const uint16_t *>(w_comp), row_off,
+      static_cast<const uint32_t *>(ter_minmax), out_tern,
+      static_cast<uint16_t *>(out_w), bad_rows, height, width);
+  HIP_TRY(hipGetLastError());
+  return SUB1_OK;
+}
+
+extern "C" int64_t sub1_moe_workspace_bytes(int tokens, int d_ff) {
+  if (tokens < 0 || d_ff < 0) return 0;
+  int64_t ctrl = (static_cast<int64_t>(kCtrlHeader + tokens) * 4 + 255) / 256 * 256;
+  return ctrl + static_cast<int64_t>(tokens) * d_ff * 2;
+}
+
+extern "C" int sub1_moe_grouped(const sub1_moe_stack *st, const int32_t *token_expert,
+                                const void *x, void *y, int tokens, void *workspace,
+                                int64_t workspace_bytes, void *stream) {
+  if (!st || !token_expert || !x || !y)
+    return fail(SUB1_ERR_NULL, "sub1_moe_grouped: NULL argument");
+  if (!st->dec || !st->w_comp || !st->wi_code_base || !st->wo_code_base ||
+      !st->wi_row_off || !st->wo_row_off || !st->wi_minmax || !st->wo_minmax)
+    return fail(SUB1_ERR_NULL, "sub1_moe_grouped: NULL pointer in the stack");
+  if (st->experts < 1 || st->d_model < 1 || st->d_ff < 1 ||
+      st->d_model > SUB1_MAX_WIDTH || st->d_ff > SUB1_MAX_WIDTH)
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped: experts %d d_model %d d_ff %d (sizes 1..%d)",
+                st->experts, st->d_model, st->d_ff, SUB1_MAX_WIDTH);
+  if (tokens < 0 || tokens > (1 << 20))
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped: tokens %d outside 0..2^20", tokens);
+  if (tokens == 0) return SUB1_OK;
+  if (!workspace || workspace_bytes < sub1_moe_workspace_bytes(tokens, st->d_ff))
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped: workspace of %lld bytes needed",
+                static_cast<long long>(sub1_moe_workspace_bytes(tokens, st->d_ff)));
+  if (misaligned(workspace, 256) || misaligned(st->dec, 4) || misaligned(st->w_comp, 2) ||
+      misaligned(st->wi_code_base, 8) || misaligned(st->wo_code_base, 8) ||
+      misaligned(st->wi_row_off, 4) || misaligned(st->wo_row_off, 4) ||
+      misaligned(st->wi_minmax, 4) || misaligned(st->wo_minmax, 4) ||
+      misaligned(token_expert, 4) || misaligned(x, 2) || misaligned(y, 2))
+    return fail(SUB1_ERR_ALIGN, "sub1_moe_grouped: misaligned pointer");
+
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint32_t *tab = nullptr;
+  int rc = slot_table_for(st->dec, s, &tab);
+  if (rc) return rc;
+
+  MoeArgs a;
+  a.tab = tab;
+  a.w_comp = reinterpret_cast<const uint16_t *>(st->w_comp);
+  a.wi_code_base = st->wi_code_base;
+  a.wo_code_base = st->wo_code_base;
+  a.wi_row_off = st->wi_row_off;
+  a.wo_row_off = st->wo_row_off;
+  a.wi_minmax = static_cast<const uint32_t *>(st->wi_minmax);
+  a.wo_minmax = static_cast<const uint32_t *>(st->wo_minmax);
+  a.token_expert = token_expert;
+  a.x = static_cast<const uint16_t *>(x);
+  a.y = static_cast<uint16_t *>(y);
+  a.ctrl = static_cast<int32_t *>(workspace);
+  int64_t ctrl_bytes = (static_cast<int64_t>(kCtrlHeader + tokens) * 4 + 255) / 256 * 256;
+  a.h = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + ctrl_bytes);
+  a.tokens = tokens;
+  a.d_model = st->d_model;
+  a.d_ff = st->d_ff;
+  a.experts = st->experts;
+  a.wi_tiles = (st->d_ff + kMoeThreads - 1) / kMoeThreads;
+  a.wo_tiles = (st->d_model + kMoeThreads - 1) / kMoeThreads;
+  a.spin_limit = 1 << 24;
+  int64_t tiles = static_cast<int64_t>(tokens) * (a.wi_tiles + a.wo_tiles);
+  if (tiles > INT32_MAX - (1 << 20))
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped: too many tiles");
+
+  int wmax = st->d_model > st->d_ff ? st->d_model : st->d_ff;
+  size_t lds = lds_dwords_for_width(wmax) * sizeof(float);
+  rc = allow_lds(moe_kernel<kMoeThreads>, lds);
+  if (rc) return rc;
+  int device = 0, cus = 0, per_cu = 0;
+  HIP_TRY(hipGetDevice(&device));
+  HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, moe_kernel<kMoeThreads>,
+                                                       kMoeThreads, lds));
+  if (per_cu < 1) return fail(SUB1_ERR_INTERNAL, "sub1_moe_grouped: kernel does not fit a CU");
+  int64_t grid = static_cast<int64_t>(cus) * per_cu;
+  if (grid > tiles) grid = tiles;
+
+  int nctrl = kCtrlHeader + tokens;
+  zero_i32_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl);
+  moe_kernel<kMoeThreads><<<static_cast<unsigned>(grid), kMoeThreads, lds, s>>>(a);
+  HIP_TRY(hipGetLastError());
+  return SUB1_OK;
+}
+
+extern "C" int sub1_timing_begin(void *stream) {
+  if (!g_ev_begin) {
+    HIP_TRY(hipEventCreate(&g_ev_begin));
+    HIP_TRY(hipEventCreate(&g_ev_end));
+  }
+  HIP_TRY(hipEventRecord(g_ev_begin, static_cast<hipStream_t>(stream)));
+  return SUB1_OK;
+}
+
+extern "C" int sub1_timing_end(void *stream, double *elapsed_us) {
+  if (!g_ev_begin) return fail(SUB1_ERR_INTERNAL, "sub1_timing_end without sub1_timing_begin");
+  if (!elapsed_us) return fail(SUB1_ERR_NULL, "sub1_timing_end: NULL argument");
+  HIP_TRY(hipEventRecord(g_ev_end, static_cast<hipStream_t>(stream)));
+  HIP_TRY(hipEventSynchronize(g_ev_end));
+  float ms = 0.f;
+  HIP_TRY(hipEventElapsedTime(&ms, g_ev_begin, g_ev_end));
+  *elapsed_us = 1e3 * static_cast<double>(ms);
+  return SUB1_OK;
+}

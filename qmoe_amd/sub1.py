@@ -1,0 +1,106 @@
+"""Module surface of the reference's `sub1.py` for the compressed-layer path:
+`setup`, the tables `dec`/`trie`, `GPUS`/`DEV`/`DEC`/`TRIE`, `Sub1Linear`
+(same buffers, `forward(x)`, static `make(w)`), plus `Sub1Experts`, the
+one-launch form of the expert loop in `FasterMLP.forward`.
+
+Differences from the reference that a caller can observe:
+  * importing works without a GPU (the reference indexes GPUS[-1] at import,
+    sub1.py:107-111); the device tables are then empty until a GPU exists;
+  * `Sub1Linear.forward` runs all tokens in one launch (the reference loops
+    over tokens, sub1.py:137-142);
+  * any (height, width) works, not only the six Switch shapes.
+"""
+import torch
+import torch.nn as nn
+
+from . import sub1_hip
+
+
+def setup():
+    """(dec int32 [131072], trie int32 [65537, 9]) CPU tensors: the fixed
+    dictionary, byte-identical to what reference sub1.py:29-102 builds."""
+    return sub1_hip.build_tables()
+
+
+dec, trie = setup()
+
+# reference sub1.py:107-111; the last GPU is the default one there
+GPUS = [torch.device('cuda:%d' % i) for i in range(torch.cuda.device_count())] \
+    if torch.cuda.is_available() else []
+DEV = GPUS[-1] if GPUS else None
+DEC = [dec.to(gpu) for gpu in GPUS]
+TRIE = trie.to(DEV) if DEV is not None else None
+
+
+def device_tables(device):
+    """(DEC for that device, TRIE moved to that device)."""
+    device = torch.device(device)
+    if device.type != 'cuda' or not GPUS:
+        raise RuntimeError('the compressed-expert kernels need a GPU; got %s' % device)
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    t = TRIE if TRIE.device.index == idx else TRIE.to(device)
+    return DEC[idx], t
+
+
+class Sub1Linear(nn.Module):
+    """Compressed linear layer (reference sub1.py:114-166): buffers `w_comp`
+    int16 [comp_size], `row_off` int32 [height+1], `ter_minmax` bf16
+    [2*height], and an empty bf16 `weight` that HuggingFace's Switch expert
+    reads the dtype of."""
+
+    def __init__(self, height, comp_size):
+        super().__init__()
+        self.register_buffer('w_comp', torch.zeros(comp_size, dtype=torch.int16))
+        self.register_buffer('row_off', torch.zeros(height + 1, dtype=torch.int32))
+        self.register_buffer('ter_minmax', torch.zeros(2 * height, dtype=torch.bfloat16))
+        self.register_buffer('weight', torch.zeros(0, dtype=torch.bfloat16))
+
+    def forward(self, x):
+        """x bf16 [T, width] -> bf16 [T, height] (reference sub1.py:132-143)."""
+        height = self.row_off.shape[0] - 1
+        y = torch.zeros((x.shape[0], height), dtype=torch.bfloat16, device=x.device)
+        if x.shape[0] == 0:
+            return y
+        table = DEC[self.w_comp.device.index]
+        sub1_hip.sub1matvec_tokens(table, self.w_comp, self.row_off, self.ter_minmax,
+                                   x.contiguous(), y)
+        return y
+
+    @staticmethod
+    def make(w):
+        """Ternarise and pack a dense matrix whose rows take the values
+        {row min, 0, row max} (reference sub1.py:145-166; ties go to max)."""
+        w = w.bfloat16()
+        ter_minmax = torch.column_stack((w.min(1)[0], w.max(1)[0])).flatten()
+        row_off = torch.zeros(w.shape[0] + 1, dtype=torch.int32, device=w.device)
+        w_tern = torch.zeros(w.shape, dtype=torch.int32, device=w.device)
+        w_tern[w == ter_minmax[0::2].reshape((-1, 1))] = 1
+        w_tern[w == ter_minmax[1::2].reshape((-1, 1))] = 2
+        _, table = device_tables(w.device)
+        w_comp = sub1_hip.sub1pack(table, w_tern, row_off)
+
+        linear = Sub1Linear(w.shape[0], w_comp.shape[0])
+        linear.w_comp.data = w_comp
+        linear.row_off.data = row_off
+        linear.ter_minmax = ter_minmax
+        return linear
+
+
+class Sub1Experts(nn.Module):
+    """All experts of one MoE layer behind one launch.
+
+    Built from per-expert (wi, wo) `Sub1Linear` pairs; `forward(x, expert)`
+    returns wo_e(relu(wi_e(x[t]))) per token and passes through tokens whose
+    expert index is negative, which is what the loop at reference
+    sub1.py:312-317 produces for routed and for dropped tokens."""
+
+    def __init__(self, wi_layers, wo_layers):
+        super().__init__()
+        dev = wi_layers[0].w_comp.device
+        self.stack = sub1_hip.ExpertStack.from_layers(
+            DEC[dev.index],
+            [(l.w_comp, l.row_off, l.ter_minmax) for l in wi_layers],
+            [(l.w_comp, l.row_off, l.ter_minmax) for l in wo_layers])
+
+    def forward(self, x, expert_index):
+        return self.stack.forward(x.contiguous(), expert_index.to(torch.int32).contiguous())

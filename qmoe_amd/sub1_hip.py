@@ -1,0 +1,211 @@
+"""Operator module with the surface of the reference's `sub1_cuda` extension
+(reference sub1_cuda.cpp:56-59): `sub1matvec` and `sub1pack`, same positional
+arguments, tensors in, launched on torch's current stream.  Underneath is the C
+ABI of libsub1_hip.so; torch only supplies device memory and the stream.
+
+    import qmoe_amd.sub1_hip as sub1_cuda      # drop-in for `import sub1_cuda`
+
+Additions the reference does not have: argument checking (the reference casts
+raw pointers unchecked and silently ignores unsupported shapes,
+sub1_cuda_kernel.cu:78-87), `sub1matvec_tokens`, `sub1decode`, and the grouped
+expert launch `ExpertStack.forward`.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+DICT_ENTRIES = _lib.DICT_ENTRIES
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(t, dtype, name, device=None, numel=None, dim=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError('%s must be a torch.Tensor' % name)
+    if t.dtype != dtype:
+        raise TypeError('%s must be %s, got %s' % (name, dtype, t.dtype))
+    if not t.is_cuda:
+        raise ValueError('%s must live on the GPU' % name)
+    if device is not None and t.device != device:
+        raise ValueError('%s is on %s, expected %s' % (name, t.device, device))
+    if not t.is_contiguous():
+        raise ValueError('%s must be contiguous' % name)
+    if numel is not None and t.numel() != numel:
+        raise ValueError('%s must hold %d elements, got %d' % (name, numel, t.numel()))
+    if dim is not None and t.dim() != dim:
+        raise ValueError('%s must be %d-D' % (name, dim))
+    return t.data_ptr()
+
+
+def build_tables():
+    """(dec int32 [131072], trie int32 [65537, 9]) on the CPU: the fixed
+    dictionary of reference sub1.py:29-102, built by the library (C++)."""
+    dec = torch.empty(_lib.DEC_WORDS, dtype=torch.int32)
+    trie = torch.empty((_lib.TRIE_ROWS, 9), dtype=torch.int32)
+    _lib.check(_lib.load().sub1_build_tables(dec.data_ptr(), trie.data_ptr()))
+    return dec, trie
+
+
+def sub1matvec(dec, w_comp, row_off, ter_minmax, x, y):
+    """y += W x for one compressed matrix; height = y.numel(), width =
+    x.numel() (reference sub1_cuda_kernel.cu:78-79).  Any shape, in place."""
+    dev = dec.device if isinstance(dec, torch.Tensor) else None
+    height, width = y.numel(), x.numel()
+    args = [
+        _need(dec, torch.int32, 'dec', numel=_lib.DEC_WORDS),
+        _need(w_comp, torch.int16, 'w_comp', dev),
+        _need(row_off, torch.int32, 'row_off', dev, numel=height + 1),
+        _need(ter_minmax, torch.bfloat16, 'ter_minmax', dev, numel=2 * height),
+        _need(x, torch.bfloat16, 'x', dev),
+        _need(y, torch.bfloat16, 'y', dev),
+    ]
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().sub1_matvec(*args, height, width, _stream()))
+
+
+def sub1matvec_tokens(dec, w_comp, row_off, ter_minmax, x, y):
+    """y[t] += W x[t] for x [T, W], y [T, H] in one launch."""
+    dev = dec.device if isinstance(dec, torch.Tensor) else None
+    args = [
+        _need(dec, torch.int32, 'dec', numel=_lib.DEC_WORDS),
+        _need(w_comp, torch.int16, 'w_comp', dev),
+        _need(row_off, torch.int32, 'row_off', dev),
+        _need(ter_minmax, torch.bfloat16, 'ter_minmax', dev),
+        _need(x, torch.bfloat16, 'x', dev, dim=2),
+        _need(y, torch.bfloat16, 'y', dev, dim=2),
+    ]
+    tokens, width = x.shape
+    height = row_off.numel() - 1
+    if y.shape != (tokens, height) or ter_minmax.numel() != 2 * height:
+        raise ValueError('y must be [%d, %d] and ter_minmax [%d]' % (tokens, height, 2 * height))
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().sub1_matvec_tokens(*args, height, width, tokens,
+                                                  width, height, _stream()))
+
+
+def sub1pack(trie, w_tern, row_off):
+    """Greedy dictionary encode of w_tern (int32 [H, W] symbols, CLOBBERED);
+    row_off (int32 [H+1]) is overwritten with the cumulative code counts and
+    the int16 code stream is returned (reference sub1_cuda_kernel.cu:92-126)."""
+    dev = trie.device if isinstance(trie, torch.Tensor) else None
+    p_trie = _need(trie, torch.int32, 'trie', numel=_lib.TRIE_ROWS * 9)
+    p_w = _need(w_tern, torch.int32, 'w_tern', dev, dim=2)
+    height, width = w_tern.shape
+    p_ro = _need(row_off, torch.int32, 'row_off', dev, numel=height + 1)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(lib.sub1_pack_count(p_trie, p_w, p_ro, height, width, _stream()))
+        total = int(row_off[height].item())      # the one host sync, as in the reference
+        w_comp = torch.empty(total, dtype=torch.int16, device=dev)
+        _lib.check(lib.sub1_pack_emit(p_w, p_ro, w_comp.data_ptr(), height, width, _stream()))
+    return w_comp
+
+
+def sub1decode(dec, w_comp, row_off, ter_minmax, width, want_tern=True, want_w=True):
+    """Decode without multiplying: (symbols uint8 [H, W] or None, weights bf16
+    [H, W] or None, number of rows whose codes do not cover the width)."""
+    dev = dec.device if isinstance(dec, torch.Tensor) else None
+    height = row_off.numel() - 1
+    p_dec = _need(dec, torch.int32, 'dec', numel=_lib.DEC_WORDS)
+    p_wc = _need(w_comp, torch.int16, 'w_comp', dev)
+    p_ro = _need(row_off, torch.int32, 'row_off', dev)
+    p_mm = _need(ter_minmax, torch.bfloat16, 'ter_minmax', dev, numel=2 * height) \
+        if ter_minmax is not None else None
+    tern = torch.zeros((height, width), dtype=torch.uint8, device=dev) if want_tern else None
+    w = torch.zeros((height, width), dtype=torch.bfloat16, device=dev) if want_w else None
+    bad = torch.zeros(1, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().sub1_decode(
+            p_dec, p_wc, p_ro, p_mm, tern.data_ptr() if want_tern else None,
+            w.data_ptr() if want_w else None, bad.data_ptr(), height, width, _stream()))
+    return tern, w, int(bad.item())
+
+
+class ExpertStack:
+    """The Sub1Linear buffers of all experts of one MoE layer, back to back in
+    one set of tensors, and the one-launch forward over them.
+
+    wi[e], wo[e] are (w_comp int16 [C], row_off int32 [H+1], ter_minmax bf16
+    [2H]) triples as Sub1Linear holds them; wi has H = d_ff, wo has H = d_model.
+    """
+
+    def __init__(self, dec, w_comp, wi_code_base, wo_code_base, wi_row_off, wo_row_off,
+                 wi_minmax, wo_minmax, d_model, d_ff):
+        dev = dec.device
+        experts = wi_code_base.numel()
+        self.dec, self.w_comp = dec, w_comp
+        self.wi_code_base, self.wo_code_base = wi_code_base, wo_code_base
+        self.wi_row_off, self.wo_row_off = wi_row_off, wo_row_off
+        self.wi_minmax, self.wo_minmax = wi_minmax, wo_minmax
+        self.experts, self.d_model, self.d_ff = experts, d_model, d_ff
+        self.device = dev
+        self._c = _lib.MoeStack(
+            _need(dec, torch.int32, 'dec', numel=_lib.DEC_WORDS),
+            _need(w_comp, torch.int16, 'w_comp', dev),
+            _need(wi_code_base, torch.int64, 'wi_code_base', dev, numel=experts),
+            _need(wo_code_base, torch.int64, 'wo_code_base', dev, numel=experts),
+            _need(wi_row_off, torch.int32, 'wi_row_off', dev, numel=experts * (d_ff + 1)),
+            _need(wo_row_off, torch.int32, 'wo_row_off', dev, numel=experts * (d_model + 1)),
+            _need(wi_minmax, torch.bfloat16, 'wi_minmax', dev, numel=experts * 2 * d_ff),
+            _need(wo_minmax, torch.bfloat16, 'wo_minmax', dev, numel=experts * 2 * d_model),
+            experts, d_model, d_ff)
+        self._ws = None
+
+    @classmethod
+    def from_layers(cls, dec, wi_layers, wo_layers):
+        """Stack per-expert (w_comp, row_off, ter_minmax) triples."""
+        dev = dec.device
+        d_ff = wi_layers[0][1].numel() - 1
+        d_model = wo_layers[0][1].numel() - 1
+        sizes = [t[0].numel() for t in wi_layers] + [t[0].numel() for t in wo_layers]
+        bases = torch.zeros(len(sizes) + 1, dtype=torch.int64)
+        bases[1:] = torch.tensor(sizes, dtype=torch.int64).cumsum(0)
+        n = len(wi_layers)
+        w_comp = torch.cat([t[0] for t in wi_layers] + [t[0] for t in wo_layers])
+        return cls(dec, w_comp, bases[:n].to(dev), bases[n:2 * n].to(dev),
+                   torch.cat([t[1] for t in wi_layers]), torch.cat([t[1] for t in wo_layers]),
+                   torch.cat([t[2] for t in wi_layers]), torch.cat([t[2] for t in wo_layers]),
+                   d_model, d_ff)
+
+    def compressed_bytes(self):
+        """Bytes of the stack a full sweep reads: codes, row offsets, min/max."""
+        return (2 * self.w_comp.numel() + 4 * self.wi_row_off.numel()
+                + 4 * self.wo_row_off.numel() + 2 * self.wi_minmax.numel()
+                + 2 * self.wo_minmax.numel())
+
+    def workspace(self, tokens):
+        need = _lib.load().sub1_moe_workspace_bytes(tokens, self.d_ff)
+        if self._ws is None or self._ws.numel() < need:
+            self._ws = torch.empty(need, dtype=torch.uint8, device=self.device)
+        return self._ws
+
+    def forward(self, x, token_expert, y=None):
+        """y[t] = wo_e(relu(wi_e(x[t]))), e = token_expert[t]; tokens with a
+        negative expert keep their input.  x bf16 [T, d_model], token_expert
+        int32 [T]."""
+        dev = self.device
+        p_x = _need(x, torch.bfloat16, 'x', dev, dim=2)
+        tokens = x.shape[0]
+        if x.shape[1] != self.d_model:
+            raise ValueError('x must be [T, %d]' % self.d_model)
+        p_te = _need(token_expert, torch.int32, 'token_expert', dev, numel=tokens)
+        if y is None:
+            y = torch.empty_like(x)
+        p_y = _need(y, torch.bfloat16, 'y', dev, numel=x.numel())
+        ws = self.workspace(tokens)
+        with torch.cuda.device(dev):
+            _lib.check(_lib.load().sub1_moe_grouped(
+                ctypes.byref(self._c), p_te, p_x, p_y, tokens, ws.data_ptr(),
+                ws.numel(), _stream()))
+        return y
+
+    def launch_faults(self, tokens):
+        """(waits inside the last forward that gave up, tokens whose expert id
+        was >= experts and were passed through); both 0 when all is well.
+        Reads the control words of the workspace, synchronising."""
+        ctrl = self.workspace(tokens)[:16].view(torch.int32).tolist()
+        return ctrl[1], ctrl[2]

@@ -1,0 +1,262 @@
+"""GPU parity tests: the HIP library, called through its C ABI (via the ctypes
+binding), against the CPU oracle on the same seeded inputs.
+
+Bars:
+  * decode, pack: bit-exact against the oracle (integer/byte work);
+  * products: the output must equal the oracle's per-symbol stream-order result
+    bit for bit (the kernels add activations in that order), must lie within
+        2^-8 |exact| + 64 * 2^-24 * sum|w x|
+    of the double-precision product, and must agree with the reference kernel's
+    lane-order arithmetic to 1e-2 relative (normwise), the tolerance the task
+    states for bf16 outputs with fp32 accumulation.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import sub1_oracle as so
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2          # stated tolerance for outputs
+
+SWITCH_SHAPES = [(3072, 768, 0.90), (768, 3072, 0.90), (4096, 1024, 0.88),
+                 (1024, 4096, 0.88), (6144, 2080, 0.90), (2080, 6144, 0.90)]
+ODD_SHAPES = [(77, 333, 0.7), (5, 1, 0.5), (9, 2, 0.5), (33, 29, 0.3), (64, 56, 0.0),
+              (130, 15, 0.9), (1, 4000, 0.95), (300, 12288, 0.99)]
+
+
+@pytest.fixture(scope='module')
+def gpu():
+    from qmoe_amd import sub1, sub1_hip
+    assert torch.cuda.is_available(), 'these tests need the GPU'
+    assert sub1.DEC, 'device tables missing'
+    return sub1, sub1_hip
+
+
+def bf16_dev(bits):
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).cuda().view(torch.bfloat16)
+
+
+def bits_host(t):
+    return t.detach().contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def dev_case(oracle, height, width, p0, seed):
+    t, mm = so.synthetic_ternary(height, width, p0, seed)
+    codes, row_off = oracle.encode(t)
+    x = so.synthetic_activation(width, seed + 1000)
+    d = dict(t=t, mm=mm, codes=codes, row_off=row_off, x=x,
+             w_comp=torch.from_numpy(codes.view(np.int16)).cuda(),
+             row_off_d=torch.from_numpy(row_off).cuda(), mm_d=bf16_dev(mm), x_d=bf16_dev(x))
+    return d
+
+
+def check_product(oracle, c, y_bits):
+    exact, sum_abs = oracle.matvec_f64(c['t'].astype(np.uint8), c['mm'], c['x'])
+    y = so.bf16_bits_to_f32(y_bits).astype(np.float64)
+    bound = 2.0 ** -8 * np.abs(exact) + 64 * 2.0 ** -24 * sum_abs + 1e-30
+    assert np.all(np.abs(y - exact) <= bound)
+    lanes = so.bf16_bits_to_f32(oracle.matvec_lanes(c['codes'], c['row_off'], c['mm'], c['x']))
+    denom = max(np.linalg.norm(lanes), 1e-30)
+    assert np.linalg.norm(y - lanes) / denom <= REL_TOL
+    seq = oracle.matvec_seq(c['codes'], c['row_off'], c['mm'], c['x'])
+    assert np.array_equal(y_bits, seq)
+
+
+def test_device_tables_equal_oracle(gpu, oracle):
+    sub1, _ = gpu
+    dec, trie = oracle.tables()
+    assert np.array_equal(sub1.DEC[0].cpu().numpy(), dec)
+    assert np.array_equal(sub1.TRIE.cpu().numpy(), trie)
+
+
+@pytest.mark.parametrize('height,width,p0', SWITCH_SHAPES + ODD_SHAPES)
+def test_decode_bit_exact(gpu, oracle, height, width, p0):
+    sub1, op = gpu
+    c = dev_case(oracle, height, width, p0, seed=height + width)
+    tern, w, bad = op.sub1decode(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], width)
+    assert bad == 0
+    assert np.array_equal(tern.cpu().numpy(), c['t'].astype(np.uint8))
+    assert np.array_equal(bits_host(w), oracle.dequant(c['t'].astype(np.uint8), c['mm']))
+
+
+def test_decode_counts_bad_rows(gpu, oracle):
+    sub1, op = gpu
+    c = dev_case(oracle, 8, 64, 0.9, seed=1)
+    ro = c['row_off'].copy()
+    ro[3] -= 1                                   # row 2 loses a code, row 3 gains one
+    _, _, bad = op.sub1decode(sub1.DEC[0], c['w_comp'], torch.from_numpy(ro).cuda(),
+                              c['mm_d'], 64, want_w=False)
+    assert bad == 2
+
+
+@pytest.mark.parametrize('height,width,p0', SWITCH_SHAPES + ODD_SHAPES)
+def test_pack_bit_exact(gpu, oracle, height, width, p0):
+    sub1, op = gpu
+    t, _ = so.synthetic_ternary(height, width, p0, seed=3 * height + width)
+    codes, row_off = oracle.encode(t)
+    w_tern = torch.from_numpy(t).cuda()
+    ro = torch.full((height + 1,), -7, dtype=torch.int32, device='cuda')
+    w_comp = op.sub1pack(sub1.TRIE, w_tern, ro)
+    assert w_comp.dtype == torch.int16
+    assert np.array_equal(ro.cpu().numpy(), row_off)
+    assert np.array_equal(w_comp.cpu().numpy().view(np.uint16), codes)
+
+
+@pytest.mark.parametrize('height,width,p0', SWITCH_SHAPES + ODD_SHAPES)
+def test_matvec_against_oracle(gpu, oracle, height, width, p0):
+    sub1, op = gpu
+    c = dev_case(oracle, height, width, p0, seed=7 * height + width)
+    y = torch.zeros(height, dtype=torch.bfloat16, device='cuda')
+    op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], c['x_d'], y)
+    check_product(oracle, c, bits_host(y))
+
+
+def test_matvec_accumulates_into_y(gpu, oracle):
+    sub1, op = gpu
+    c = dev_case(oracle, 200, 512, 0.9, seed=5)
+    pre = so.f32_to_bf16_bits(np.random.default_rng(0).standard_normal(200).astype(np.float32))
+    y = bf16_dev(pre).clone()
+    op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], c['x_d'], y)
+    want = oracle.matvec_seq(c['codes'], c['row_off'], c['mm'], c['x'], y=pre)
+    assert np.array_equal(bits_host(y), want)
+    # twice more: the reference's benchmark loop keeps adding onto y (test.py:175)
+    op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], c['x_d'], y)
+    want = oracle.matvec_seq(c['codes'], c['row_off'], c['mm'], c['x'], y=want)
+    assert np.array_equal(bits_host(y), want)
+
+
+def test_matvec_closed_forms(gpu, oracle):
+    sub1, op = gpu
+    c = dev_case(oracle, 96, 300, 0.6, seed=9)
+    w = so.bf16_bits_to_f32(oracle.dequant(c['t'].astype(np.uint8), c['mm']))
+    for k in (0, 1, 27, 28, 150, 299):
+        x = torch.zeros(300, dtype=torch.bfloat16, device='cuda')
+        x[k] = 1.0
+        y = torch.zeros(96, dtype=torch.bfloat16, device='cuda')
+        op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], x, y)
+        assert np.array_equal(y.float().cpu().numpy(), w[:, k])
+    x = torch.ones(300, dtype=torch.bfloat16, device='cuda')
+    y = torch.zeros(96, dtype=torch.bfloat16, device='cuda')
+    op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], x, y)
+    f = so.bf16_bits_to_f32(c['mm'])
+    n1, n2 = (c['t'] == 1).sum(1), (c['t'] == 2).sum(1)
+    want = so.f32_to_bf16_bits((f[0::2] * n1 + f[1::2] * n2).astype(np.float32))
+    assert np.array_equal(bits_host(y), want)
+
+
+def test_matvec_on_unaligned_views(gpu, oracle):
+    """x[i] / y[i] row views and a code stream that starts at an odd element,
+    as the callers at reference sub1.py:141 and an expert stack produce."""
+    sub1, op = gpu
+    c = dev_case(oracle, 130, 333, 0.8, seed=12)
+    pad = torch.zeros(3, dtype=torch.int16, device='cuda')
+    stream = torch.cat((pad, c['w_comp']))[3:]
+    assert stream.data_ptr() % 4 == 2
+    xs = torch.zeros((3, 333), dtype=torch.bfloat16, device='cuda')
+    xs[1] = c['x_d']
+    ys = torch.zeros((3, 130), dtype=torch.bfloat16, device='cuda')
+    op.sub1matvec(sub1.DEC[0], stream, c['row_off_d'], c['mm_d'], xs[1], ys[1])
+    check_product(oracle, c, bits_host(ys[1]))
+    assert not ys[0].any() and not ys[2].any()
+
+
+def test_matvec_rejects_bad_tensors(gpu, oracle):
+    sub1, op = gpu
+    c = dev_case(oracle, 16, 64, 0.9, seed=2)
+    y = torch.zeros(16, dtype=torch.bfloat16, device='cuda')
+    with pytest.raises(TypeError):
+        op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], c['x_d'].float(), y)
+    with pytest.raises(ValueError):
+        op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], c['x_d'].cpu(), y)
+    with pytest.raises(ValueError):
+        op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'][:-1], c['mm_d'], c['x_d'], y)
+    from qmoe_amd._lib import Sub1Error
+    big = torch.zeros(12289, dtype=torch.bfloat16, device='cuda')
+    with pytest.raises(Sub1Error):
+        op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], big, y)
+
+
+def test_matvec_tokens(gpu, oracle):
+    sub1, op = gpu
+    c = dev_case(oracle, 300, 768, 0.9, seed=21)
+    xs = np.stack([so.synthetic_activation(768, 50 + i) for i in range(5)])
+    y = torch.zeros((5, 300), dtype=torch.bfloat16, device='cuda')
+    op.sub1matvec_tokens(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], bf16_dev(xs), y)
+    for i in range(5):
+        want = oracle.matvec_seq(c['codes'], c['row_off'], c['mm'], xs[i])
+        assert np.array_equal(bits_host(y[i]), want)
+
+
+@pytest.mark.parametrize('height,width,p0', [(3072, 768, 0.9), (768, 3072, 0.9), (96, 130, 0.4)])
+def test_sub1linear_make_and_forward(gpu, oracle, height, width, p0):
+    """The reference's own smoke check (test.py:180-189): dense product, kernel
+    product and make(w) round trip must agree."""
+    sub1, op = gpu
+    t, mm = so.synthetic_ternary(height, width, p0, seed=31)
+    assert (t == 1).any(1).all() and (t == 2).any(1).all()   # make() needs both signs per row
+    w_bits = oracle.dequant(t.astype(np.uint8), mm)
+    w = bf16_dev(w_bits)
+    lin = sub1.Sub1Linear.make(w)
+    codes, row_off = oracle.encode(t)
+    assert np.array_equal(lin.row_off.cpu().numpy(), row_off)
+    assert np.array_equal(lin.w_comp.cpu().numpy().view(np.uint16), codes)
+    assert np.array_equal(bits_host(lin.ter_minmax), mm)
+    x = torch.randn((3, width), generator=torch.Generator().manual_seed(1)).bfloat16().cuda()
+    y = lin(x)
+    assert y.shape == (3, height) and y.dtype == torch.bfloat16
+    ref = x.float() @ w.float().t()                       # plain fp32 torch reference
+    err = (y.float() - ref).norm() / ref.norm()
+    assert err <= REL_TOL
+    assert lin(x[:0]).shape == (0, height)
+
+
+def small_stack(oracle, experts, d_model, d_ff, p0, seed):
+    from qmoe_amd import sub1, sub1_hip
+    wi, wo = [], []
+    for e in range(experts):
+        ti, mi = so.synthetic_ternary(d_ff, d_model, p0, seed + 2 * e)
+        to, mo = so.synthetic_ternary(d_model, d_ff, p0, seed + 2 * e + 1)
+        wi.append(oracle.encode(ti) + (mi,))
+        wo.append(oracle.encode(to) + (mo,))
+    dev = lambda l: (torch.from_numpy(l[0].view(np.int16)).cuda(),
+                     torch.from_numpy(l[1]).cuda(), bf16_dev(l[2]))
+    stack = sub1_hip.ExpertStack.from_layers(sub1.DEC[0], [dev(l) for l in wi],
+                                             [dev(l) for l in wo])
+    return stack, wi, wo
+
+
+@pytest.mark.parametrize('experts,d_model,d_ff,p0', [(6, 96, 200, 0.8), (4, 768, 3072, 0.9),
+                                                     (3, 333, 77, 0.7)])
+def test_grouped_launch_against_oracle(gpu, oracle, experts, d_model, d_ff, p0):
+    stack, wi, wo = small_stack(oracle, experts, d_model, d_ff, p0, seed=100)
+    # skewed routing: expert 0 gets several tokens, the last expert none, one
+    # token is dropped (-1) and one names an expert that does not exist
+    route = [0, 1, 0, -1, 2 % experts, 0, experts + 5, 1, 0]
+    xs = np.stack([so.synthetic_activation(d_model, 200 + i) for i in range(len(route))])
+    x = bf16_dev(xs)
+    y = stack.forward(x, torch.tensor(route, dtype=torch.int32, device='cuda'))
+    got = bits_host(y)
+    assert stack.launch_faults(len(route)) == (0, 1)
+    for i, e in enumerate(route):
+        if e < 0 or e >= experts:
+            assert np.array_equal(got[i], xs[i])
+        else:
+            want, _ = oracle.expert_ffn(wi[e], wo[e], xs[i], order=1)
+            assert np.array_equal(got[i], want), (i, e)
+            lanes, _ = oracle.expert_ffn(wi[e], wo[e], xs[i], order=0)
+            a, b = so.bf16_bits_to_f32(got[i]), so.bf16_bits_to_f32(lanes)
+            assert np.linalg.norm(a - b) <= REL_TOL * np.linalg.norm(b)
+    # a second launch reuses the workspace
+    y2 = stack.forward(x, torch.tensor(route, dtype=torch.int32, device='cuda'))
+    assert torch.equal(y, y2)
+
+
+def test_grouped_launch_no_tokens_and_all_dropped(gpu, oracle):
+    stack, _, _ = small_stack(oracle, 2, 64, 128, 0.8, seed=300)
+    x = torch.zeros((0, 64), dtype=torch.bfloat16, device='cuda')
+    assert stack.forward(x, torch.zeros(0, dtype=torch.int32, device='cuda')).shape == (0, 64)
+    x = torch.randn((4, 64), device='cuda').bfloat16()
+    y = stack.forward(x, torch.full((4,), -1, dtype=torch.int32, device='cuda'))
+    assert torch.equal(x, y)
