@@ -518,6 +518,7 @@ extern "C" int sub1_matvec_tokens(const int32_t *dec, const int16_t *w_comp,
                                   const int32_t *row_off, const void *ter_minmax,
                                   const void *x, void *y, int height, int width,
                                   int tokens, int64_t ldx, int64_t ldy, void *stream) {
+  if (tokens == 0) return SUB1_OK;
   if (!dec || !row_off || !ter_minmax || !x || !y)
     return fail(SUB1_ERR_NULL, "sub1_matvec: NULL argument");
   if (height < 1 || width < 1 || width > SUB1_MAX_WIDTH)
@@ -531,7 +532,6 @@ extern "C" int sub1_matvec_tokens(const int32_t *dec, const int16_t *w_comp,
   if (misaligned(dec, 4) || misaligned(row_off, 4) || misaligned(ter_minmax, 4) ||
       misaligned(w_comp, 2) || misaligned(x, 2) || misaligned(y, 2))
     return fail(SUB1_ERR_ALIGN, "sub1_matvec: misaligned pointer");
-  if (tokens == 0) return SUB1_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const uint32_t *tab = nullptr;
   int rc = slot_table_for(dec, s, &tab);
@@ -616,7 +616,9 @@ extern "C" int64_t sub1_moe_workspace_bytes(int tokens, int d_ff) {
 extern "C" int sub1_moe_grouped(const sub1_moe_stack *st, const int32_t *token_expert,
                                 const void *x, void *y, int tokens, void *workspace,
                                 int64_t workspace_bytes, void *stream) {
-  if (!st || !token_expert || !x || !y)
+  if (!st) return fail(SUB1_ERR_NULL, "sub1_moe_grouped: NULL stack");
+  if (tokens == 0) return SUB1_OK;
+  if (!token_expert || !x || !y)
     return fail(SUB1_ERR_NULL, "sub1_moe_grouped: NULL argument");
   if (!st->dec || !st->w_comp || !st->wi_code_base || !st->wo_code_base ||
       !st->wi_row_off || !st->wo_row_off || !st->wi_minmax || !st->wo_minmax)
@@ -627,7 +629,6 @@ extern "C" int sub1_moe_grouped(const sub1_moe_stack *st, const int32_t *token_e
                 st->experts, st->d_model, st->d_ff, SUB1_MAX_WIDTH);
   if (tokens < 0 || tokens > (1 << 20))
     return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped: tokens %d outside 0..2^20", tokens);
-  if (tokens == 0) return SUB1_OK;
   if (!workspace || workspace_bytes < sub1_moe_workspace_bytes(tokens, st->d_ff))
     return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped: workspace of %lld bytes needed",
                 static_cast<long long>(sub1_moe_workspace_bytes(tokens, st->d_ff)));

@@ -195,6 +195,8 @@ class ExpertStack:
         p_te = _need(token_expert, torch.int32, 'token_expert', dev, numel=tokens)
         if y is None:
             y = torch.empty_like(x)
+        if tokens == 0:
+            return y
         p_y = _need(y, torch.bfloat16, 'y', dev, numel=x.numel())
         ws = self.workspace(tokens)
         with torch.cuda.device(dev):
