@@ -34,8 +34,8 @@ WORKLOADS = {
 def algorithmic_bytes(stack, experts_used):
     """Bytes the products of one launch have to read and write (per product:
     2*codes + 4*(H+1) row offsets + 4*H min/max + 2*W input + 2*H output), plus
-    the 256 KiB slot table once per launch."""
-    total = 256 * 1024
+    the 61.5 KB decode table once per launch."""
+    total = 15388 * 4
     for e in experts_used:
         total += 2 * int(stack.wi_codes[e]) + 2 * int(stack.wo_codes[e])
         for h, w in ((stack.d_ff, stack.d_model), (stack.d_model, stack.d_ff)):
@@ -151,14 +151,21 @@ def main():
     print('built %d experts in %.1f s, %.3f GB compressed' %
           (experts, time.perf_counter() - tick, stack.compressed_bytes() / 1e9), file=sys.stderr)
 
+    tick = time.perf_counter()
+    prep = stack.prepare()
+    torch.cuda.synchronize()
+    print('prepared in %.2f s: %.3f GB of interleaved codes (%.3f x the packed stream)' %
+          (time.perf_counter() - tick, prep.code_bytes / 1e9,
+           prep.code_bytes / (2.0 * stack.w_comp.numel())), file=sys.stderr)
+
     x = synthetic.activations(experts, d_model, args.seed + 1)
     route = torch.arange(experts, dtype=torch.int32, device='cuda')
     y = torch.empty_like(x)
     stream_ptr = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
-    wall, us_launch = time_launches(lambda: stack.forward(x, route, y), args.steps,
+    wall, us_launch = time_launches(lambda: prep.forward(x, route, y), args.steps,
                                     args.warmup, stream_ptr)
-    assert stack.launch_faults(experts) == (0, 0)
+    assert prep.launch_faults(experts) == (0, 0)
     ms_per_step = wall / args.steps * 1e3
     abytes = algorithmic_bytes(stack, range(experts))
     achieved = abytes / (us_launch * 1e-6) / 1e9
@@ -179,7 +186,7 @@ def main():
                                             / (2.0 * experts * d_model * d_ff), 4)},
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS,
                      'unit': 'GB/s', 'frac': round(achieved / HBM_PEAK_GBS, 4),
-                     'traffic': None, 'kernel': 'moe_kernel',
+                     'traffic': None, 'kernel': 'moe_prepared_kernel',
                      'algorithmic_bytes': abytes, 'us_per_launch': round(us_launch, 2)},
     }
 
@@ -187,8 +194,14 @@ def main():
     # batch-1: one token routed to one seeded uniform expert (launch-latency bound)
     g = torch.Generator().manual_seed(args.seed + 2)
     one = torch.randint(0, experts, (1,), generator=g).to(torch.int32).cuda()
-    _, us1 = time_launches(lambda: stack.forward(x[:1], one, y[:1]), 200, 20, stream_ptr)
+    y1 = torch.empty_like(x[:1])
+    _, us1 = time_launches(lambda: prep.forward(x[:1], one, y1), 200, 20, stream_ptr)
     also['single_token_us'] = round(us1, 2)
+    # the same sweep through the kernel that reads the reference's packed layout directly
+    y2 = torch.empty_like(x)
+    _, us_ref = time_launches(lambda: stack.forward(x, route, y2), 3, 1, stream_ptr)
+    also['reference_layout_kernel_us'] = round(us_ref, 1)
+    also['prepared_equals_reference_layout'] = bool(torch.equal(y, y2))
     if not args.no_dense:
         n = min(experts, 128)
         d_us = dense_gemv_us(stack, x, n)

@@ -56,6 +56,21 @@ int sub1_abi_version(void);
 int sub1_build_tables(int32_t *dec_host, int32_t *trie_host);
 
 /*
+ * The tables the prepared-stack kernels decode with, built on the HOST (no
+ * counterpart in the reference, which decodes from `dec` in global memory,
+ * sub1_cuda_kernel.cu:188).  Codes are renumbered so that the decode table
+ * fits LDS: recode_host[65536] maps a dictionary index to its kernel code;
+ * codes below *single_codes index table_host directly, a code c at or above it
+ * uses word *single_codes + ((c - *single_codes) >> 3) and its low three bits
+ * are the symbol bits of the three slots.  table_host must hold
+ * SUB1_KERNEL_TABLE_MAX words; *table_words receives the number used.  Any
+ * pointer may be NULL.
+ */
+#define SUB1_KERNEL_TABLE_MAX 16384
+int sub1_build_kernel_tables(uint16_t *recode_host, uint32_t *table_host,
+                             int32_t *single_codes, int32_t *table_words);
+
+/*
  * y[r] += bf16( sum_k deq(w[r,k]) * x[k] ),  fp32 accumulation, for any
  * height >= 1 and 1 <= width <= SUB1_MAX_WIDTH.  Replaces `sub1matvec`
  * (reference sub1_cuda.cpp:35-45, sub1_cuda_kernel.cu:70-88,129-202), which
@@ -148,6 +163,51 @@ int64_t sub1_moe_workspace_bytes(int tokens, int d_ff);
 int sub1_moe_grouped(const sub1_moe_stack *stack, const int32_t *token_expert,
                      const void *x, void *y, int tokens, void *workspace,
                      int64_t workspace_bytes, void *stream);
+
+/*
+ * Prepared stack: the fast form of sub1_moe_grouped (no counterpart in the
+ * reference).  Preparing copies the stack once into a layout the GPU streams
+ * at full width - rows ordered by code count and cut into 64-row slices, each
+ * slice's codes interleaved 8 bytes per lane, codes renumbered as
+ * sub1_build_kernel_tables describes - after which the decode table (61.5 KB)
+ * and the activations both live in LDS.  Only for the fixed dictionary (dec is
+ * compared with it, once) and 1 <= d_model, d_ff <= SUB1_PREPARED_MAX_WIDTH.
+ *
+ *   meta_bytes = sub1_moe_prepared_meta_bytes(experts, d_model, d_ff);
+ *   sub1_moe_prepare_layout(stack, meta, meta_bytes, &code_bytes, stream);   // synchronises
+ *   sub1_moe_prepare_codes(stack, meta, codes, code_bytes, stream);
+ *   sub1_moe_prepared p = {meta, codes, meta_bytes, code_bytes, experts, d_model, d_ff};
+ *   sub1_moe_grouped_prepared(&p, token_expert, x, y, tokens, workspace, bytes, stream);
+ *
+ * meta and codes are device buffers the caller owns, 256-byte aligned; the
+ * original stack is not referenced after sub1_moe_prepare_codes has run.
+ * sub1_moe_grouped_prepared has the semantics of sub1_moe_grouped and the same
+ * workspace; every row's sums are taken in the same order, so outputs are
+ * identical.
+ */
+#define SUB1_PREPARED_MAX_WIDTH 8192
+
+typedef struct sub1_moe_prepared {
+  const void *meta;
+  const void *codes;
+  int64_t meta_bytes;
+  int64_t code_bytes;
+  int32_t experts;
+  int32_t d_model;
+  int32_t d_ff;
+} sub1_moe_prepared;
+
+int64_t sub1_moe_prepared_meta_bytes(int experts, int d_model, int d_ff);
+
+int sub1_moe_prepare_layout(const sub1_moe_stack *stack, void *meta, int64_t meta_bytes,
+                            int64_t *code_bytes, void *stream);
+
+int sub1_moe_prepare_codes(const sub1_moe_stack *stack, const void *meta, void *codes,
+                           int64_t code_bytes, void *stream);
+
+int sub1_moe_grouped_prepared(const sub1_moe_prepared *prepared, const int32_t *token_expert,
+                              const void *x, void *y, int tokens, void *workspace,
+                              int64_t workspace_bytes, void *stream);
 
 /*
  * Average duration in microseconds of the most recent launches, measured with

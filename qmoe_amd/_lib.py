@@ -10,6 +10,7 @@ DICT_ENTRIES = 65536
 DEC_WORDS = 2 * DICT_ENTRIES
 TRIE_ROWS = DICT_ENTRIES + 1
 MAX_WIDTH = 12288
+PREPARED_MAX_WIDTH = 8192
 
 _vp = ctypes.c_void_p
 _int = ctypes.c_int
@@ -24,11 +25,19 @@ class MoeStack(ctypes.Structure):
                 ('d_model', ctypes.c_int32), ('d_ff', ctypes.c_int32)]
 
 
+class MoePrepared(ctypes.Structure):
+    """struct sub1_moe_prepared"""
+    _fields_ = [('meta', _vp), ('codes', _vp), ('meta_bytes', _i64), ('code_bytes', _i64),
+                ('experts', ctypes.c_int32), ('d_model', ctypes.c_int32),
+                ('d_ff', ctypes.c_int32)]
+
+
 # every symbol include/sub1_hip.h declares, with its prototype
 PROTOTYPES = {
     'sub1_last_error': (ctypes.c_char_p, []),
     'sub1_abi_version': (_int, []),
     'sub1_build_tables': (_int, [_vp, _vp]),
+    'sub1_build_kernel_tables': (_int, [_vp, _vp, _vp, _vp]),
     'sub1_matvec': (_int, [_vp] * 6 + [_int, _int, _vp]),
     'sub1_matvec_tokens': (_int, [_vp] * 6 + [_int, _int, _int, _i64, _i64, _vp]),
     'sub1_pack_count': (_int, [_vp, _vp, _vp, _int, _int, _vp]),
@@ -37,6 +46,12 @@ PROTOTYPES = {
     'sub1_moe_workspace_bytes': (_i64, [_int, _int]),
     'sub1_moe_grouped': (_int, [ctypes.POINTER(MoeStack), _vp, _vp, _vp, _int, _vp,
                                 _i64, _vp]),
+    'sub1_moe_prepared_meta_bytes': (_i64, [_int, _int, _int]),
+    'sub1_moe_prepare_layout': (_int, [ctypes.POINTER(MoeStack), _vp, _i64,
+                                       ctypes.POINTER(_i64), _vp]),
+    'sub1_moe_prepare_codes': (_int, [ctypes.POINTER(MoeStack), _vp, _vp, _i64, _vp]),
+    'sub1_moe_grouped_prepared': (_int, [ctypes.POINTER(MoePrepared), _vp, _vp, _vp, _int,
+                                         _vp, _i64, _vp]),
     'sub1_timing_begin': (_int, [_vp]),
     'sub1_timing_end': (_int, [_vp, ctypes.POINTER(ctypes.c_double)]),
 }

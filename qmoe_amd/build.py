@@ -6,13 +6,14 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 LIB_PATH = os.path.join(HERE, 'libsub1_hip.so')
 SOURCES = [os.path.join(HERE, 'csrc', 'sub1_kernels.hip'),
+           os.path.join(HERE, 'csrc', 'sub1_prepared.hip'),
            os.path.join(HERE, 'csrc', 'sub1_tables.cpp')]
 
 HIPCC_FLAGS = [
     '-O3', '--offload-arch=gfx950', '-fPIC', '-shared', '-std=c++17',
     # keep the compiler from forming packed fp32 instructions
     '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
-    '-I' + os.path.join(ROOT, 'include'),
+    '-I' + os.path.join(ROOT, 'include'), '-I' + os.path.join(HERE, 'csrc'),
 ]
 
 

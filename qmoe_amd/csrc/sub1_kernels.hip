@@ -19,11 +19,9 @@
 #include <string>
 #include <vector>
 
-#include "sub1_hip.h"
+#include "sub1_common.h"
 
-namespace {
-
-// ------------------------------------------------------------ host errors --
+namespace sub1 {
 
 thread_local std::string g_err;
 
@@ -37,26 +35,15 @@ int fail(int code, const char *fmt, ...) {
   return code;
 }
 
-#define HIP_TRY(expr)                                                          \
-  do {                                                                         \
-    hipError_t e_ = (expr);                                                    \
-    if (e_ != hipSuccess)                                                      \
-      return fail(SUB1_ERR_HIP, "%s: %s", #expr, hipGetErrorString(e_));       \
-  } while (0)
+}  // namespace sub1
 
-// ---------------------------------------------------------- device helpers --
+namespace {
 
-__device__ __forceinline__ float bf16_to_f32(uint16_t h) {
-  return __uint_as_float(static_cast<uint32_t>(h) << 16);
-}
-
-// round-to-nearest-even (what __float2bfloat16 in the reference kernel does)
-__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<uint16_t>(u >> 16);
-}
+using sub1::bf16_to_f32;
+using sub1::f32_to_bf16;
+using sub1::fail;
+using sub1::misaligned;
+using sub1::row_result;
 
 // ------------------------------------------------------------ slot table ---
 //
@@ -180,12 +167,6 @@ __device__ __forceinline__ void row_sums(const uint32_t *__restrict__ tab,
       for (int j = 0; j < rem; j++) add_codeword(tab[codes[j]], M, colw, s1, s2);
     }
   }
-}
-
-__device__ __forceinline__ float row_result(uint32_t minmax, float s1, float s2) {
-  float mn = __uint_as_float(minmax << 16);
-  float mx = __uint_as_float(minmax & 0xffff0000u);
-  return __fmaf_rn(mn, s1, __fmul_rn(mx, s2));
 }
 
 // ------------------------------------------------------------- matvec ------
@@ -389,8 +370,10 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
           if (hb & 0x8000u) hb = 0;  // relu
           a.h[static_cast<int64_t>(t) * a.d_ff + row] = hb;
         }
-        __threadfence();
       }
+      // every wavefront's h stores reach L2, then the barrier, then thread 0's
+      // release writes L2 back for the other dies to see
+      sub1::drain_stores();
       __syncthreads();
       if (threadIdx.x == 0)
         __hip_atomic_fetch_add(&a.ctrl[kCtrlHeader + t], 1, __ATOMIC_RELEASE,
@@ -425,8 +408,7 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
           __builtin_amdgcn_s_sleep(8);
         }
       }
-      __syncthreads();
-      __threadfence();
+      __syncthreads();  // thread 0's acquire now covers the whole workgroup
       stage_activations<kThreads>(lds, a.h + static_cast<int64_t>(t) * a.d_ff, a.d_ff);
       __syncthreads();
       if (row < a.d_model) {
@@ -488,10 +470,6 @@ int slot_table_for(const int32_t *dec, hipStream_t stream, const uint32_t **out)
   return SUB1_OK;
 }
 
-bool misaligned(const void *p, size_t a) {
-  return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0;
-}
-
 constexpr int kMatvecThreads = 256;
 constexpr int kMoeThreads = 256;
 
@@ -510,7 +488,7 @@ hipEvent_t g_ev_begin = nullptr, g_ev_end = nullptr;
 
 // ================================================================ C ABI =====
 
-extern "C" const char *sub1_last_error(void) { return g_err.c_str(); }
+extern "C" const char *sub1_last_error(void) { return sub1::g_err.c_str(); }
 
 extern "C" int sub1_abi_version(void) { return 1; }
 

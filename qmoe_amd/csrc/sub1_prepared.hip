@@ -1,0 +1,726 @@
+// Prepared expert stack: the fast form of the grouped expert launch.
+//
+// sub1_moe_prepare_* turn an expert stack in the reference's packed layout
+// (reference sub1.py:114-130: one row-major code stream per matrix plus
+// row_off) into a form the GPU can stream at full width:
+//
+//   * rows of every matrix are ordered by code count and cut into slices of
+//     64 rows (one wavefront lane each);
+//   * a slice's codes are interleaved in chunks of 4 codes (8 bytes) per lane:
+//     chunk c of lane l sits at slice_base*512 + (c*64 + l)*8 bytes, so one
+//     wavefront load fetches 512 contiguous bytes and every byte of a cache
+//     line is used; lanes are padded to the slice's longest row (about 2%);
+//   * codes are renumbered (sub1_build_kernel_tables) so that the decode table
+//     is 61.5 KB and lives in LDS next to the activations.
+//
+// moe_prepared_kernel then walks 64 rows per wavefront: per codeword one LDS
+// table read and three LDS activation reads, each folded into two running
+// sums (activations under row-min weights, under row-max weights) with
+// v_dot2c_f32_bf16 on (x,0)/(0,x) bf16 pairs; no cross-lane traffic at all.
+// It computes what reference sub1_cuda_kernel.cu:163-201 computes per row.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+#include "sub1_common.h"
+
+namespace {
+
+using sub1::bf16_to_f32;
+using sub1::f32_to_bf16;
+using sub1::fail;
+using sub1::misaligned;
+using sub1::row_result;
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 1024;
+constexpr int kWaves = kThreads / 64;
+constexpr int kChunk = 4;            // codes per lane per chunk
+constexpr int kRing = 4;             // chunks in flight per lane
+constexpr int kMaxLen = 4096;        // codes per row: one per column pair at most
+constexpr int kCtrlHeader = 4;       // ctrl[0] ticket, [1] wait-limit hits, [2] bad expert ids
+constexpr uint32_t kIdleWord = 0x00040404u;  // three empty slots, no advance
+
+// ------------------------------------------------------------- meta layout --
+//
+// One block of device memory, arrays back to back, each 256-byte aligned.
+// Kind 0 = wi (rows d_ff, width d_model), kind 1 = wo.
+struct KindMeta {
+  int64_t slice_base;   // u32 [E*S + 1]   (only kind 0 holds the shared array)
+  int64_t slice_nch;    // u16 [E*S]
+  int64_t slice_nfull;  // u16 [E*S]
+  int64_t row_len;      // u16 [E*S*64]
+  int64_t row_idx;      // u16 [E*S*64]
+  int64_t minmax;       // u32 [E*S*64]
+  int slices;           // S
+  int height, width;
+};
+
+struct MetaLayout {
+  KindMeta k[2];
+  int64_t counts;       // i32 [E*S0 + E*S1 + 1] chunk counts, scanned in place
+  int64_t status;       // i32 [4]: [0] rows with a bad code count
+  int64_t bytes;
+};
+
+int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
+
+MetaLayout meta_layout(int experts, int d_model, int d_ff) {
+  MetaLayout m;
+  int64_t off = 0;
+  auto take = [&](int64_t bytes) {
+    int64_t o = off;
+    off += align256(bytes);
+    return o;
+  };
+  const int h[2] = {d_ff, d_model}, w[2] = {d_model, d_ff};
+  int64_t nslices = 0;
+  for (int i = 0; i < 2; i++) {
+    KindMeta &k = m.k[i];
+    k.height = h[i];
+    k.width = w[i];
+    k.slices = (h[i] + 63) / 64;
+    int64_t es = static_cast<int64_t>(experts) * k.slices;
+    nslices += es;
+    k.slice_base = 0;  // set below
+    k.slice_nch = take(es * 2);
+    k.slice_nfull = take(es * 2);
+    k.row_len = take(es * 64 * 2);
+    k.row_idx = take(es * 64 * 2);
+    k.minmax = take(es * 64 * 4);
+  }
+  m.counts = take((nslices + 1) * 4);
+  m.k[0].slice_base = m.counts;
+  m.k[1].slice_base = m.counts + static_cast<int64_t>(experts) * m.k[0].slices * 4;
+  m.status = take(16);
+  m.bytes = off;
+  return m;
+}
+
+// ---------------------------------------------------------- prepare kernels --
+
+// One workgroup per matrix: order the rows by code count, longest first, and
+// describe the 64-row slices.  The order is a counting sort carried out by one
+// thread, so it is the same on every run.
+__global__ __launch_bounds__(256) void order_rows_kernel(
+    const int32_t *__restrict__ row_off_all, const uint32_t *__restrict__ minmax_all,
+    uint16_t *__restrict__ row_len, uint16_t *__restrict__ row_idx,
+    uint32_t *__restrict__ minmax_sorted, uint16_t *__restrict__ slice_nch,
+    uint16_t *__restrict__ slice_nfull, int32_t *__restrict__ counts,
+    int32_t *__restrict__ status, int height, int width, int slices) {
+  __shared__ int hist[kMaxLen + 2];
+  const int e = blockIdx.x;
+  const int32_t *ro = row_off_all + static_cast<int64_t>(e) * (height + 1);
+  const uint32_t *mm = minmax_all + static_cast<int64_t>(e) * height;
+  const int64_t lane0 = static_cast<int64_t>(e) * slices * 64;
+  const int max_len = (width + 1) / 2;
+  for (int i = threadIdx.x; i < kMaxLen + 2; i += blockDim.x) hist[i] = 0;
+  __syncthreads();
+  for (int r = threadIdx.x; r < height; r += blockDim.x) {
+    int len = ro[r + 1] - ro[r];
+    if (len < 1 || len > max_len) {
+      atomicAdd(&status[0], 1);
+      len = len < 1 ? 0 : max_len;
+    }
+    atomicAdd(&hist[len], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;  // rows with a larger count come first
+    for (int len = max_len; len >= 0; len--) {
+      int n = hist[len];
+      hist[len] = run;
+      run += n;
+    }
+    for (int r = 0; r < height; r++) {
+      int len = ro[r + 1] - ro[r];
+      len = len < 1 ? 0 : (len > max_len ? max_len : len);
+      int p = hist[len]++;
+      row_len[lane0 + p] = static_cast<uint16_t>(len);
+      row_idx[lane0 + p] = static_cast<uint16_t>(r);
+      minmax_sorted[lane0 + p] = mm[r];
+    }
+  }
+  for (int p = height + threadIdx.x; p < slices * 64; p += blockDim.x) {
+    row_len[lane0 + p] = 0;
+    row_idx[lane0 + p] = 0xffffu;
+    minmax_sorted[lane0 + p] = 0u;
+  }
+  __syncthreads();
+  for (int s = threadIdx.x; s < slices; s += blockDim.x) {
+    int first = 64 * s;
+    int last = min(64 * s + 63, height - 1);
+    int nch = (row_len[lane0 + first] + kChunk - 1) / kChunk;
+    int nfull = row_len[lane0 + last] / kChunk;
+    int64_t g = static_cast<int64_t>(e) * slices + s;
+    slice_nch[g] = static_cast<uint16_t>(nch);
+    slice_nfull[g] = static_cast<uint16_t>(nfull);
+    counts[g + 1] = nch;
+  }
+}
+
+// In-place inclusive prefix sum over v[1..n], v[0] = 0; one workgroup.
+__global__ __launch_bounds__(1024) void scan_counts_kernel(int32_t *__restrict__ v, int n) {
+  __shared__ int32_t part[1024];
+  const int tid = threadIdx.x;
+  const int seg = (n + 1023) / 1024;
+  const int lo = 1 + tid * seg;
+  const int hi = min(n + 1, lo + seg);
+  int32_t s = 0;
+  for (int i = lo; i < hi; i++) s += v[i];
+  part[tid] = s;
+  __syncthreads();
+  for (int d = 1; d < 1024; d *= 2) {
+    int32_t t = tid >= d ? part[tid - d] : 0;
+    __syncthreads();
+    part[tid] += t;
+    __syncthreads();
+  }
+  int32_t run = tid ? part[tid - 1] : 0;
+  if (tid == 0) v[0] = 0;
+  for (int i = lo; i < hi; i++) {
+    run += v[i];
+    v[i] = run;
+  }
+}
+
+// One wavefront per ordered row: renumber its codes and write them, and the
+// zero padding up to the slice's chunk count, into the interleaved stream.
+__global__ __launch_bounds__(256) void interleave_codes_kernel(
+    const uint16_t *__restrict__ src, const int64_t *__restrict__ code_base,
+    const int32_t *__restrict__ row_off_all, const uint16_t *__restrict__ recode,
+    const uint32_t *__restrict__ slice_base, const uint16_t *__restrict__ slice_nch,
+    const uint16_t *__restrict__ row_idx, uint16_t *__restrict__ dst, int height,
+    int slices, int64_t lanes_total) {
+  const int64_t gl = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / 64;
+  if (gl >= lanes_total) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t slice = gl / 64;
+  const int ln = static_cast<int>(gl % 64);
+  const int e = static_cast<int>(slice / slices);
+  const int ridx = row_idx[gl];
+  uint16_t *d = dst + static_cast<int64_t>(slice_base[slice]) * 256;
+  const int padded = slice_nch[slice] * kChunk;
+  int len = 0;
+  const uint16_t *s = src;
+  if (ridx != 0xffff) {
+    const int32_t *ro = row_off_all + static_cast<int64_t>(e) * (height + 1);
+    s = src + code_base[e] + ro[ridx];
+    len = min(max(ro[ridx + 1] - ro[ridx], 0), padded);
+  }
+  for (int j = lane; j < padded; j += 64) {
+    // padding decodes as one zero pair, the shortest entry (dictionary index 0)
+    uint16_t c = recode[j < len ? s[j] : 0];
+    d[(j / kChunk) * 256 + ln * kChunk + (j % kChunk)] = c;
+  }
+}
+
+__global__ void zero_words_kernel(int32_t *p, int n) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// ------------------------------------------------------------- main kernel --
+
+struct KindArgs {
+  const uint32_t *slice_base;
+  const uint16_t *slice_nch;
+  const uint16_t *slice_nfull;
+  const uint16_t *row_len;
+  const uint16_t *row_idx;
+  const uint32_t *minmax;
+  int slices, height, width, tiles;
+};
+
+struct PreparedArgs {
+  const uint32_t *table;      // kernel decode table (global copy, staged into LDS)
+  const uint16_t *codes;
+  KindArgs k[2];
+  const int32_t *token_expert;
+  const uint16_t *x;
+  uint16_t *y;
+  uint16_t *h;
+  int32_t *ctrl;
+  int tokens, experts;
+  int table_words, single_codes, group_shift;  // group_shift = single_codes - single_codes/8
+  int xdwords;                                 // LDS dwords reserved for the activations
+  int spin_limit;
+};
+
+// Activations in LDS, 6 dwords per column pair:
+//   [A_even, B_even, A_odd, B_odd, 0, 0],  A = (x, 0), B = (0, x) as bf16 pairs.
+// Slot offset 6m + 2q + sym-1 selects the value for the row-min sum (A) or the
+// row-max sum (B); offsets 4 and 5 read zeros.  28 zero columns follow the row
+// (digits of a last codeword that overhang the width, as the reference pads).
+__host__ __device__ constexpr int activation_dwords(int width) {
+  return 6 * ((width + 28 + 1) / 2 + 1);
+}
+
+__device__ __forceinline__ void stage_activations(uint32_t *xa, const uint16_t *x, int width) {
+  const int npairs = (width + 28 + 1) / 2 + 1;
+  for (int m = threadIdx.x; m < npairs; m += kThreads) {
+    uint32_t xe = 2 * m < width ? x[2 * m] : 0u;
+    uint32_t xo = 2 * m + 1 < width ? x[2 * m + 1] : 0u;
+    uint32_t *p = xa + 6 * m;
+    p[0] = xe;
+    p[1] = xe << 16;
+    p[2] = xo;
+    p[3] = xo << 16;
+    p[4] = 0u;
+    p[5] = 0u;
+  }
+}
+
+struct DotConsts {
+  bf16x2 lo, hi;   // (1, 0) and (0, 1)
+};
+
+__device__ __forceinline__ DotConsts dot_consts() {
+  // Kept in scalar registers through asm so that the compiler cannot turn
+  // (1.0, 0) into an inline constant of the packed-bf16 operand.
+  uint32_t k1, k2;
+  asm volatile("s_mov_b32 %0, 0x3f80" : "=s"(k1));
+  asm volatile("s_mov_b32 %0, 0x3f800000" : "=s"(k2));
+  DotConsts c;
+  c.lo = __builtin_bit_cast(bf16x2, k1);
+  c.hi = __builtin_bit_cast(bf16x2, k2);
+  return c;
+}
+
+// Table word of kernel code c with the code's symbol bits put in place.
+__device__ __forceinline__ uint32_t lookup(const uint32_t *tab, uint32_t c, int group_shift) {
+  uint32_t idx = min(c, (c >> 3) + static_cast<uint32_t>(group_shift));
+  uint32_t word = tab[idx];
+  uint32_t bits = (c & 7u) * 0x4081u;      // bit j of c -> bit 8j
+  return (word & ~0x00010101u) | (bits & 0x00010101u);
+}
+
+__device__ __forceinline__ void add_codeword(uint32_t e, const uint32_t *xa, int &colw,
+                                             float &s1, float &s2, const DotConsts &k) {
+#pragma unroll
+  for (int j = 0; j < 3; j++) {
+    int idx = colw + static_cast<int>((e >> (8 * j)) & 0xffu);
+    bf16x2 v = __builtin_bit_cast(bf16x2, xa[idx]);
+    s1 = __builtin_amdgcn_fdot2_f32_bf16(v, k.lo, s1, false);
+    s2 = __builtin_amdgcn_fdot2_f32_bf16(v, k.hi, s2, false);
+  }
+  colw += static_cast<int>(e >> 24);
+}
+
+// The two sums of this lane's row of slice `sl`.
+__device__ __forceinline__ void slice_sums(const PreparedArgs &a, const KindArgs &k,
+                                           int64_t sl, const uint32_t *tab,
+                                           const uint32_t *xa, float &s1, float &s2) {
+  const int lane = threadIdx.x & 63;
+  const DotConsts dk = dot_consts();
+  const int nch = __builtin_amdgcn_readfirstlane(k.slice_nch[sl]);
+  const int nfull = __builtin_amdgcn_readfirstlane(k.slice_nfull[sl]);
+  const int len = k.row_len[sl * 64 + lane];
+  const uint2 *p =
+      reinterpret_cast<const uint2 *>(a.codes + static_cast<int64_t>(k.slice_base[sl]) * 256) +
+      lane;
+  s1 = 0.f;
+  s2 = 0.f;
+  int colw = 0;
+  uint2 ring[kRing];
+#pragma unroll
+  for (int i = 0; i < kRing; i++)
+    if (i < nch) ring[i] = p[i * 64];
+  int c = 0;
+  // chunks every lane of the slice has in full: no per-code checks
+  for (; c + kRing <= nfull; c += kRing) {
+#pragma unroll
+    for (int i = 0; i < kRing; i++) {
+      uint2 w = ring[i];
+      if (c + kRing + i < nch) ring[i] = p[(c + kRing + i) * 64];
+      uint32_t e0 = lookup(tab, w.x & 0xffffu, a.group_shift);
+      uint32_t e1 = lookup(tab, w.x >> 16, a.group_shift);
+      uint32_t e2 = lookup(tab, w.y & 0xffffu, a.group_shift);
+      uint32_t e3 = lookup(tab, w.y >> 16, a.group_shift);
+      add_codeword(e0, xa, colw, s1, s2, dk);
+      add_codeword(e1, xa, colw, s1, s2, dk);
+      add_codeword(e2, xa, colw, s1, s2, dk);
+      add_codeword(e3, xa, colw, s1, s2, dk);
+    }
+  }
+  // the rest, each code checked against the lane's own count
+  for (; c < nch; c += kRing) {
+#pragma unroll
+    for (int i = 0; i < kRing; i++) {
+      if (c + i < nch) {
+        uint2 w = ring[i];
+        if (c + kRing + i < nch) ring[i] = p[(c + kRing + i) * 64];
+        const int j = kChunk * (c + i);
+        uint32_t e0 = lookup(tab, w.x & 0xffffu, a.group_shift);
+        uint32_t e1 = lookup(tab, w.x >> 16, a.group_shift);
+        uint32_t e2 = lookup(tab, w.y & 0xffffu, a.group_shift);
+        uint32_t e3 = lookup(tab, w.y >> 16, a.group_shift);
+        if (j + 0 >= len) e0 = kIdleWord;
+        if (j + 1 >= len) e1 = kIdleWord;
+        if (j + 2 >= len) e2 = kIdleWord;
+        if (j + 3 >= len) e3 = kIdleWord;
+        add_codeword(e0, xa, colw, s1, s2, dk);
+        add_codeword(e1, xa, colw, s1, s2, dk);
+        add_codeword(e2, xa, colw, s1, s2, dk);
+        add_codeword(e3, xa, colw, s1, s2, dk);
+      }
+    }
+  }
+}
+
+// Persistent grid; tiles = (token, projection, 16 slices), all wi tiles
+// numbered before all wo tiles and handed out by an atomic ticket.  A wo tile
+// waits for the wi tiles of its token, which hold smaller tickets and so are
+// running or done: the wait always ends.  h is published by ONE agent-scope
+// release per tile (thread 0, after the workgroup barrier) and picked up by one
+// acquire; an agent-scope fence costs an L2 write-back on this part, which is
+// why the lanes do not fence individually.
+__global__ __launch_bounds__(kThreads) void moe_prepared_kernel(PreparedArgs a) {
+  extern __shared__ uint32_t lds[];
+  __shared__ int s_ticket;
+  uint32_t *tab = lds;
+  uint32_t *xa = lds + a.table_words;
+  for (int i = threadIdx.x; i < a.table_words; i += kThreads) tab[i] = a.table[i];
+  const int n_wi = a.tokens * a.k[0].tiles;
+  const int n_all = n_wi + a.tokens * a.k[1].tiles;
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  for (;;) {
+    __syncthreads();
+    if (threadIdx.x == 0)
+      s_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const int ticket = s_ticket;
+    if (ticket >= n_all) break;
+    const int kind = ticket < n_wi ? 0 : 1;
+    const KindArgs &k = a.k[kind];
+    const int rel = kind ? ticket - n_wi : ticket;
+    const int t = rel / k.tiles;
+    const int tile = rel - t * k.tiles;
+    int e = a.token_expert[t];
+    if (e >= a.experts) {
+      if (kind == 1 && tile == 0 && threadIdx.x == 0)
+        __hip_atomic_fetch_add(&a.ctrl[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      e = -1;
+    }
+    if (kind == 0) {
+      if (e >= 0) {
+        stage_activations(xa, a.x + static_cast<int64_t>(t) * k.width, k.width);
+        __syncthreads();
+        const int s = tile * kWaves + wave;
+        if (s < k.slices) {
+          const int64_t sl = static_cast<int64_t>(e) * k.slices + s;
+          float s1, s2;
+          slice_sums(a, k, sl, tab, xa, s1, s2);
+          const int ridx = k.row_idx[sl * 64 + lane];
+          if (ridx != 0xffff) {
+            uint16_t hb = f32_to_bf16(row_result(k.minmax[sl * 64 + lane], s1, s2));
+            if (hb & 0x8000u) hb = 0;  // relu
+            a.h[static_cast<int64_t>(t) * k.height + ridx] = hb;
+          }
+        }
+      }
+      sub1::drain_stores();   // this wavefront's h stores are in L2 ...
+      __syncthreads();        // ... so are everyone's, and thread 0's release publishes them
+      if (threadIdx.x == 0)
+        __hip_atomic_fetch_add(&a.ctrl[kCtrlHeader + t], 1, __ATOMIC_RELEASE,
+                               __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+      if (e < 0) {
+        // a dropped token keeps its input (reference sub1.py:312)
+        for (int i = tile * kThreads + threadIdx.x; i < min(k.height, (tile + 1) * kThreads);
+             i += kThreads) {
+          int64_t g = static_cast<int64_t>(t) * k.height + i;
+          a.y[g] = a.x[g];
+        }
+        // rows of a dropped token beyond the tiles' reach (height > tiles*1024 cannot
+        // happen: tiles covers every slice)
+        continue;
+      }
+      if (threadIdx.x == 0) {
+        int spins = 0;
+        while (__hip_atomic_load(&a.ctrl[kCtrlHeader + t], __ATOMIC_ACQUIRE,
+                                 __HIP_MEMORY_SCOPE_AGENT) < a.k[0].tiles) {
+          if (++spins > a.spin_limit) {
+            __hip_atomic_fetch_add(&a.ctrl[1], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+          }
+          __builtin_amdgcn_s_sleep(8);
+        }
+      }
+      __syncthreads();
+      stage_activations(xa, a.h + static_cast<int64_t>(t) * k.width, k.width);
+      __syncthreads();
+      const int s = tile * kWaves + wave;
+      if (s < k.slices) {
+        const int64_t sl = static_cast<int64_t>(e) * k.slices + s;
+        float s1, s2;
+        slice_sums(a, k, sl, tab, xa, s1, s2);
+        const int ridx = k.row_idx[sl * 64 + lane];
+        if (ridx != 0xffff)
+          a.y[static_cast<int64_t>(t) * k.height + ridx] =
+              f32_to_bf16(row_result(k.minmax[sl * 64 + lane], s1, s2));
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------ per-device tables --
+
+struct DeviceTables {
+  int device;
+  uint16_t *recode;
+  uint32_t *table;
+  int single_codes, words;
+};
+
+std::mutex g_mutex;
+std::vector<DeviceTables> g_tables;
+std::vector<std::pair<int, const int32_t *>> g_checked_dec;   // (device, dec) known to be the fixed table
+
+int device_tables(hipStream_t stream, const DeviceTables **out) {
+  int device = 0;
+  HIP_TRY(hipGetDevice(&device));
+  std::lock_guard<std::mutex> lock(g_mutex);
+  for (const DeviceTables &t : g_tables)
+    if (t.device == device) {
+      *out = &t;
+      return SUB1_OK;
+    }
+  std::vector<uint16_t> recode(SUB1_DICT_ENTRIES);
+  std::vector<uint32_t> table(SUB1_KERNEL_TABLE_MAX, 0u);
+  DeviceTables t;
+  t.device = device;
+  int rc = sub1_build_kernel_tables(recode.data(), table.data(), &t.single_codes, &t.words);
+  if (rc) return fail(rc, "sub1_build_kernel_tables failed");
+  HIP_TRY(hipMalloc(&t.recode, recode.size() * sizeof(uint16_t)));
+  HIP_TRY(hipMalloc(&t.table, table.size() * sizeof(uint32_t)));
+  HIP_TRY(hipMemcpyAsync(t.recode, recode.data(), recode.size() * sizeof(uint16_t),
+                         hipMemcpyHostToDevice, stream));
+  HIP_TRY(hipMemcpyAsync(t.table, table.data(), table.size() * sizeof(uint32_t),
+                         hipMemcpyHostToDevice, stream));
+  HIP_TRY(hipStreamSynchronize(stream));  // the host vectors go away
+  g_tables.push_back(t);
+  *out = &g_tables.back();
+  return SUB1_OK;
+}
+
+// The renumbering belongs to the fixed dictionary: refuse any other dec.
+int check_dec(const int32_t *dec, hipStream_t stream) {
+  int device = 0;
+  HIP_TRY(hipGetDevice(&device));
+  {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    for (const auto &p : g_checked_dec)
+      if (p.first == device && p.second == dec) return SUB1_OK;
+  }
+  std::vector<int32_t> want(SUB1_DEC_WORDS), got(SUB1_DEC_WORDS);
+  int rc = sub1_build_tables(want.data(), nullptr);
+  if (rc) return fail(rc, "sub1_build_tables failed");
+  HIP_TRY(hipMemcpyAsync(got.data(), dec, got.size() * sizeof(int32_t), hipMemcpyDeviceToHost,
+                         stream));
+  HIP_TRY(hipStreamSynchronize(stream));
+  if (std::memcmp(want.data(), got.data(), want.size() * sizeof(int32_t)) != 0)
+    return fail(SUB1_ERR_SHAPE,
+                "sub1_moe_prepare: dec is not the fixed dictionary; use sub1_moe_grouped");
+  std::lock_guard<std::mutex> lock(g_mutex);
+  g_checked_dec.push_back({device, dec});
+  return SUB1_OK;
+}
+
+int check_stack(const sub1_moe_stack *st, const char *who) {
+  if (!st) return fail(SUB1_ERR_NULL, "%s: NULL stack", who);
+  if (!st->dec || !st->w_comp || !st->wi_code_base || !st->wo_code_base || !st->wi_row_off ||
+      !st->wo_row_off || !st->wi_minmax || !st->wo_minmax)
+    return fail(SUB1_ERR_NULL, "%s: NULL pointer in the stack", who);
+  if (st->experts < 1 || st->d_model < 1 || st->d_ff < 1 ||
+      st->d_model > SUB1_PREPARED_MAX_WIDTH || st->d_ff > SUB1_PREPARED_MAX_WIDTH)
+    return fail(SUB1_ERR_SHAPE, "%s: experts %d d_model %d d_ff %d (sizes 1..%d)", who,
+                st->experts, st->d_model, st->d_ff, SUB1_PREPARED_MAX_WIDTH);
+  if (static_cast<int64_t>(st->experts) * ((st->d_ff + 63) / 64 + (st->d_model + 63) / 64) >
+      (1 << 24))
+    return fail(SUB1_ERR_SHAPE, "%s: too many 64-row slices", who);
+  if (misaligned(st->dec, 4) || misaligned(st->w_comp, 2) || misaligned(st->wi_code_base, 8) ||
+      misaligned(st->wo_code_base, 8) || misaligned(st->wi_row_off, 4) ||
+      misaligned(st->wo_row_off, 4) || misaligned(st->wi_minmax, 4) ||
+      misaligned(st->wo_minmax, 4))
+    return fail(SUB1_ERR_ALIGN, "%s: misaligned pointer in the stack", who);
+  return SUB1_OK;
+}
+
+}  // namespace
+
+// ================================================================ C ABI =====
+
+extern "C" int64_t sub1_moe_prepared_meta_bytes(int experts, int d_model, int d_ff) {
+  if (experts < 1 || d_model < 1 || d_ff < 1) return 0;
+  return meta_layout(experts, d_model, d_ff).bytes;
+}
+
+extern "C" int sub1_moe_prepare_layout(const sub1_moe_stack *st, void *meta, int64_t meta_bytes,
+                                       int64_t *code_bytes, void *stream) {
+  int rc = check_stack(st, "sub1_moe_prepare_layout");
+  if (rc) return rc;
+  if (!meta || !code_bytes) return fail(SUB1_ERR_NULL, "sub1_moe_prepare_layout: NULL argument");
+  if (misaligned(meta, 256)) return fail(SUB1_ERR_ALIGN, "sub1_moe_prepare_layout: meta must be 256-byte aligned");
+  const MetaLayout m = meta_layout(st->experts, st->d_model, st->d_ff);
+  if (meta_bytes < m.bytes)
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_prepare_layout: meta needs %lld bytes",
+                static_cast<long long>(m.bytes));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  rc = check_dec(st->dec, s);
+  if (rc) return rc;
+  char *base = static_cast<char *>(meta);
+  int32_t *status = reinterpret_cast<int32_t *>(base + m.status);
+  int32_t *counts = reinterpret_cast<int32_t *>(base + m.counts);
+  zero_words_kernel<<<1, 64, 0, s>>>(status, 4);
+  const int32_t *row_off[2] = {st->wi_row_off, st->wo_row_off};
+  const void *minmax[2] = {st->wi_minmax, st->wo_minmax};
+  int64_t slice0 = 0;
+  for (int i = 0; i < 2; i++) {
+    const KindMeta &k = m.k[i];
+    order_rows_kernel<<<st->experts, 256, 0, s>>>(
+        row_off[i], static_cast<const uint32_t *>(minmax[i]),
+        reinterpret_cast<uint16_t *>(base + k.row_len),
+        reinterpret_cast<uint16_t *>(base + k.row_idx),
+        reinterpret_cast<uint32_t *>(base + k.minmax),
+        reinterpret_cast<uint16_t *>(base + k.slice_nch),
+        reinterpret_cast<uint16_t *>(base + k.slice_nfull), counts + slice0, status, k.height,
+        k.width, k.slices);
+    slice0 += static_cast<int64_t>(st->experts) * k.slices;
+  }
+  scan_counts_kernel<<<1, 1024, 0, s>>>(counts, static_cast<int>(slice0));
+  HIP_TRY(hipGetLastError());
+  int32_t host[2] = {0, 0};
+  HIP_TRY(hipMemcpyAsync(&host[0], status, 4, hipMemcpyDeviceToHost, s));
+  HIP_TRY(hipMemcpyAsync(&host[1], counts + slice0, 4, hipMemcpyDeviceToHost, s));
+  HIP_TRY(hipStreamSynchronize(s));
+  if (host[0])
+    return fail(SUB1_ERR_SHAPE,
+                "sub1_moe_prepare_layout: %d rows have a code count outside 1..width/2", host[0]);
+  if (host[1] < 0) return fail(SUB1_ERR_SHAPE, "sub1_moe_prepare_layout: stream too large");
+  *code_bytes = static_cast<int64_t>(host[1]) * 512;
+  return SUB1_OK;
+}
+
+extern "C" int sub1_moe_prepare_codes(const sub1_moe_stack *st, const void *meta, void *codes,
+                                      int64_t code_bytes, void *stream) {
+  int rc = check_stack(st, "sub1_moe_prepare_codes");
+  if (rc) return rc;
+  if (!meta || !codes) return fail(SUB1_ERR_NULL, "sub1_moe_prepare_codes: NULL argument");
+  if (misaligned(meta, 256) || misaligned(codes, 256))
+    return fail(SUB1_ERR_ALIGN, "sub1_moe_prepare_codes: buffers must be 256-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const DeviceTables *t = nullptr;
+  rc = device_tables(s, &t);
+  if (rc) return rc;
+  const MetaLayout m = meta_layout(st->experts, st->d_model, st->d_ff);
+  const char *base = static_cast<const char *>(meta);
+  // the layout pass left the total in the last count; make sure the buffer holds it
+  int64_t nslices = static_cast<int64_t>(st->experts) * (m.k[0].slices + m.k[1].slices);
+  int32_t total = 0;
+  HIP_TRY(hipMemcpyAsync(&total, reinterpret_cast<const int32_t *>(base + m.counts) + nslices, 4,
+                         hipMemcpyDeviceToHost, s));
+  HIP_TRY(hipStreamSynchronize(s));
+  if (code_bytes < static_cast<int64_t>(total) * 512)
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_prepare_codes: code buffer needs %lld bytes",
+                static_cast<long long>(total) * 512);
+  const int64_t *code_base[2] = {st->wi_code_base, st->wo_code_base};
+  const int32_t *row_off[2] = {st->wi_row_off, st->wo_row_off};
+  for (int i = 0; i < 2; i++) {
+    const KindMeta &k = m.k[i];
+    int64_t lanes = static_cast<int64_t>(st->experts) * k.slices * 64;
+    interleave_codes_kernel<<<static_cast<unsigned>((lanes + 3) / 4), 256, 0, s>>>(
+        reinterpret_cast<const uint16_t *>(st->w_comp), code_base[i], row_off[i], t->recode,
+        reinterpret_cast<const uint32_t *>(base + k.slice_base),
+        reinterpret_cast<const uint16_t *>(base + k.slice_nch),
+        reinterpret_cast<const uint16_t *>(base + k.row_idx), static_cast<uint16_t *>(codes),
+        k.height, k.slices, lanes);
+  }
+  HIP_TRY(hipGetLastError());
+  return SUB1_OK;
+}
+
+extern "C" int sub1_moe_grouped_prepared(const sub1_moe_prepared *p, const int32_t *token_expert,
+                                         const void *x, void *y, int tokens, void *workspace,
+                                         int64_t workspace_bytes, void *stream) {
+  if (!p) return fail(SUB1_ERR_NULL, "sub1_moe_grouped_prepared: NULL argument");
+  if (tokens == 0) return SUB1_OK;
+  if (!p->meta || !p->codes || !token_expert || !x || !y)
+    return fail(SUB1_ERR_NULL, "sub1_moe_grouped_prepared: NULL argument");
+  if (p->experts < 1 || p->d_model < 1 || p->d_ff < 1 ||
+      p->d_model > SUB1_PREPARED_MAX_WIDTH || p->d_ff > SUB1_PREPARED_MAX_WIDTH)
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: experts %d d_model %d d_ff %d",
+                p->experts, p->d_model, p->d_ff);
+  if (tokens < 0 || tokens > (1 << 20))
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: tokens %d outside 0..2^20", tokens);
+  if (!workspace || workspace_bytes < sub1_moe_workspace_bytes(tokens, p->d_ff))
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: workspace of %lld bytes needed",
+                static_cast<long long>(sub1_moe_workspace_bytes(tokens, p->d_ff)));
+  if (misaligned(workspace, 256) || misaligned(p->meta, 256) || misaligned(p->codes, 256) ||
+      misaligned(token_expert, 4) || misaligned(x, 2) || misaligned(y, 2))
+    return fail(SUB1_ERR_ALIGN, "sub1_moe_grouped_prepared: misaligned pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const DeviceTables *t = nullptr;
+  int rc = device_tables(s, &t);
+  if (rc) return rc;
+  const MetaLayout m = meta_layout(p->experts, p->d_model, p->d_ff);
+  if (p->meta_bytes < m.bytes)
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: meta smaller than its layout");
+  const char *base = static_cast<const char *>(p->meta);
+
+  PreparedArgs a;
+  a.table = t->table;
+  a.codes = static_cast<const uint16_t *>(p->codes);
+  for (int i = 0; i < 2; i++) {
+    const KindMeta &k = m.k[i];
+    a.k[i].slice_base = reinterpret_cast<const uint32_t *>(base + k.slice_base);
+    a.k[i].slice_nch = reinterpret_cast<const uint16_t *>(base + k.slice_nch);
+    a.k[i].slice_nfull = reinterpret_cast<const uint16_t *>(base + k.slice_nfull);
+    a.k[i].row_len = reinterpret_cast<const uint16_t *>(base + k.row_len);
+    a.k[i].row_idx = reinterpret_cast<const uint16_t *>(base + k.row_idx);
+    a.k[i].minmax = reinterpret_cast<const uint32_t *>(base + k.minmax);
+    a.k[i].slices = k.slices;
+    a.k[i].height = k.height;
+    a.k[i].width = k.width;
+    a.k[i].tiles = (k.slices + kWaves - 1) / kWaves;
+  }
+  a.token_expert = token_expert;
+  a.x = static_cast<const uint16_t *>(x);
+  a.y = static_cast<uint16_t *>(y);
+  a.ctrl = static_cast<int32_t *>(workspace);
+  int64_t ctrl_bytes = (static_cast<int64_t>(kCtrlHeader + tokens) * 4 + 255) / 256 * 256;
+  a.h = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + ctrl_bytes);
+  a.tokens = tokens;
+  a.experts = p->experts;
+  a.table_words = t->words;
+  a.single_codes = t->single_codes;
+  a.group_shift = t->single_codes - t->single_codes / 8;
+  int wmax = p->d_model > p->d_ff ? p->d_model : p->d_ff;
+  a.xdwords = activation_dwords(wmax);
+  a.spin_limit = 1 << 24;
+  int64_t tiles = static_cast<int64_t>(tokens) * (a.k[0].tiles + a.k[1].tiles);
+  if (tiles > INT32_MAX - (1 << 20))
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: too many tiles");
+
+  size_t lds = (static_cast<size_t>(a.table_words) + a.xdwords) * 4;
+  if (lds > 160 * 1024 - 64)
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: width %d does not fit LDS", wmax);
+  HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(moe_prepared_kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+  int device = 0, cus = 0;
+  HIP_TRY(hipGetDevice(&device));
+  HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+  int64_t grid = cus;  // one 1024-lane workgroup per compute unit
+  if (grid > tiles) grid = tiles;
+  int nctrl = kCtrlHeader + tokens;
+  zero_words_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl);
+  moe_prepared_kernel<<<static_cast<unsigned>(grid), kThreads, lds, s>>>(a);
+  HIP_TRY(hipGetLastError());
+  return SUB1_OK;
+}

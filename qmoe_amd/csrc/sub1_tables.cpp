@@ -114,3 +114,217 @@ extern "C" int sub1_build_tables(int32_t *dec_host, int32_t *trie_host) {
   }
   return SUB1_OK;
 }
+
+// ---------------------------------------------------------------------------
+// Kernel tables: a renumbering of the dictionary under which the decode table
+// fits LDS.
+//
+// An entry has at most three non-zero weights.  Entries that differ only in
+// the symbols (row min / row max) of their non-zeros form a group; 7164 groups
+// of three non-zeros are complete (all 8 symbol patterns are entries).  The
+// kernels work on streams whose codes were renumbered so that
+//   * a complete group g owns the 8 consecutive codes B + 8g .. B + 8g + 7 and
+//     the code's low three bits ARE the symbol pattern (bit j set = non-zero j
+//     is the row max): the group needs ONE table word;
+//   * every other entry (B of them) owns one code below B and one table word
+//     of its own, and its code is chosen so that its low three bits agree
+//     with its symbols too (bits of empty slots are free).  This is what lets
+//     the kernel insert the code's low bits into the table word unconditionally.
+// Table word: byte j (j = 0..2) = slot j, the dword offset of that non-zero in
+// the activation array relative to the codeword's first column, with the
+// symbol bit cleared; byte 3 = 6 * pair count.  The activation array spends 6
+// dwords per column pair: [A_even, B_even, A_odd, B_odd, 0, 0], A = value
+// routed to the row-min sum, B = to the row-max sum, so a non-zero at in-code
+// position p = 2m + q with symbol s sits at 6m + 2q + (s - 1) and an empty slot
+// points at the zero pair, offset 4.
+//
+// Slots are in column order, except that slots feeding different sums may be
+// swapped (that changes no sum's order of additions): the freedom is needed to
+// balance the code classes.
+namespace {
+
+struct Parsed {
+  int len;        // pairs
+  int n;          // non-zeros
+  int pos[3];
+  int sym[3];     // 1 or 2
+};
+
+bool parse_entry(const Str &s, Parsed &p) {
+  p.len = s.len;
+  p.n = 0;
+  for (int j = 0; j < s.len; j++) {
+    int r = s.s[j];
+    int d[2] = {r % 3, r / 3};
+    for (int q = 0; q < 2; q++) {
+      if (!d[q]) continue;
+      if (p.n == 3) return false;
+      p.pos[p.n] = 2 * j + q;
+      p.sym[p.n] = d[q];
+      p.n++;
+    }
+  }
+  return true;
+}
+
+inline uint32_t slot_offset(int pos) { return 6u * (pos / 2) + 2u * (pos & 1); }
+constexpr uint32_t kEmptySlot = 4;
+
+struct Arrangement {
+  int cls_mask;   // bits of the code class that are fixed
+  int cls_val;    // their values
+  int slot_of[3]; // slot index of non-zero i
+};
+
+// All ways to put the non-zeros of an entry into the three slots such that
+// non-zeros with the same symbol stay in column order.
+void arrangements(const Parsed &p, std::vector<Arrangement> &out) {
+  out.clear();
+  int perm[3] = {0, 1, 2};
+  do {
+    // perm[i] = slot of non-zero i (only the first p.n matter)
+    bool ok = true;
+    for (int a = 0; a < p.n && ok; a++)
+      for (int b = a + 1; b < p.n && ok; b++)
+        if (p.sym[a] == p.sym[b] && perm[a] > perm[b]) ok = false;
+    if (!ok) continue;
+    Arrangement ar;
+    ar.cls_mask = 0;
+    ar.cls_val = 0;
+    for (int i = 0; i < 3; i++) ar.slot_of[i] = perm[i];
+    for (int i = 0; i < p.n; i++) {
+      ar.cls_mask |= 1 << perm[i];
+      if (p.sym[i] == 2) ar.cls_val |= 1 << perm[i];
+    }
+    bool dup = false;
+    for (const Arrangement &o : out)
+      if (o.cls_mask == ar.cls_mask && o.cls_val == ar.cls_val) {
+        bool same = true;
+        for (int i = 0; i < p.n; i++) same = same && o.slot_of[i] == ar.slot_of[i];
+        if (same) dup = true;
+      }
+    if (!dup) out.push_back(ar);
+  } while (std::next_permutation(perm, perm + 3));
+}
+
+uint32_t table_word(const Parsed &p, const int slot_of[3]) {
+  uint32_t f[3] = {kEmptySlot, kEmptySlot, kEmptySlot};
+  for (int i = 0; i < p.n; i++) f[slot_of[i]] = slot_offset(p.pos[i]);
+  return f[0] | (f[1] << 8) | (f[2] << 16) | (static_cast<uint32_t>(6 * p.len) << 24);
+}
+
+}  // namespace
+
+extern "C" int sub1_build_kernel_tables(uint16_t *recode_host, uint32_t *table_host,
+                                        int32_t *single_codes, int32_t *table_words) {
+  std::vector<Str> res;
+  if (!sub1::dictionary_strings(res)) return SUB1_ERR_INTERNAL;
+  std::vector<Parsed> ps(kCount);
+  for (int i = 0; i < kCount; i++)
+    if (!parse_entry(res[i], ps[i])) return SUB1_ERR_INTERNAL;
+
+  // groups of three non-zeros keyed by (length, positions)
+  struct Group {
+    int member[8];
+    int count;
+  };
+  std::vector<Group> groups;
+  std::vector<int> group_of(kCount, -1);
+  {
+    std::vector<std::pair<uint32_t, int>> keyed;
+    for (int i = 0; i < kCount; i++)
+      if (ps[i].n == 3) {
+        uint32_t key = (ps[i].len << 15) | (ps[i].pos[0] << 10) | (ps[i].pos[1] << 5) | ps[i].pos[2];
+        keyed.push_back({key, i});
+      }
+    std::sort(keyed.begin(), keyed.end());
+    for (size_t a = 0; a < keyed.size();) {
+      size_t b = a;
+      Group g;
+      g.count = 0;
+      for (int k = 0; k < 8; k++) g.member[k] = -1;
+      while (b < keyed.size() && keyed[b].first == keyed[a].first) {
+        const Parsed &p = ps[keyed[b].second];
+        int pat = (p.sym[0] == 2) | ((p.sym[1] == 2) << 1) | ((p.sym[2] == 2) << 2);
+        g.member[pat] = keyed[b].second;
+        g.count++;
+        b++;
+      }
+      if (g.count == 8) {
+        for (int k = 0; k < 8; k++) group_of[g.member[k]] = static_cast<int>(groups.size());
+        groups.push_back(g);
+      }
+      a = b;
+    }
+  }
+  // complete groups in order of their first entry, so the numbering is canonical
+  std::sort(groups.begin(), groups.end(), [](const Group &a, const Group &b) {
+    return *std::min_element(a.member, a.member + 8) < *std::min_element(b.member, b.member + 8);
+  });
+
+  std::vector<int> singles;
+  for (int i = 0; i < kCount; i++)
+    if (group_of[i] < 0) singles.push_back(i);
+  const int nb = static_cast<int>(singles.size());
+  if (nb % 8 != 0 || nb + 8 * static_cast<int>(groups.size()) != kCount) return SUB1_ERR_INTERNAL;
+  const int words = nb + static_cast<int>(groups.size());
+  if (single_codes) *single_codes = nb;
+  if (table_words) *table_words = words;
+  if (!recode_host && !table_host) return SUB1_OK;
+
+  std::vector<uint16_t> recode(kCount);
+  std::vector<uint32_t> table(words);
+
+  // singles: most constrained first, each to the admissible class with most room
+  std::vector<std::vector<Arrangement>> opts(nb);
+  std::vector<int> order(nb);
+  for (int k = 0; k < nb; k++) {
+    arrangements(ps[singles[k]], opts[k]);
+    order[k] = k;
+  }
+  auto classes_of = [&](int k) {
+    int m = 0;
+    for (const Arrangement &a : opts[k])
+      for (int c = 0; c < 8; c++)
+        if ((c & a.cls_mask) == a.cls_val) m |= 1 << c;
+    return __builtin_popcount(m);
+  };
+  std::vector<int> nclasses(nb);
+  for (int k = 0; k < nb; k++) nclasses[k] = classes_of(k);
+  std::stable_sort(order.begin(), order.end(),
+                   [&](int a, int b) { return nclasses[a] < nclasses[b]; });
+  // Classes 000 and 111 admit only entries whose non-zeros all feed one sum, so
+  // they are filled first; the one-bit and two-bit classes come after.
+  const int rank_of[8] = {0, 1, 1, 2, 1, 2, 2, 0};
+  int used[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int cap = nb / 8;
+  for (int k : order) {
+    int best_c = -1;
+    const Arrangement *best_a = nullptr;
+    for (const Arrangement &a : opts[k])
+      for (int c = 0; c < 8; c++) {
+        if ((c & a.cls_mask) != a.cls_val || used[c] >= cap) continue;
+        bool better = best_c < 0 || rank_of[c] < rank_of[best_c] ||
+                      (rank_of[c] == rank_of[best_c] && used[c] < used[best_c]);
+        if (better) {
+          best_c = c;
+          best_a = &a;
+        }
+      }
+    if (best_c < 0) return SUB1_ERR_INTERNAL;  // classes cannot be balanced
+    int code = best_c + 8 * used[best_c]++;
+    recode[singles[k]] = static_cast<uint16_t>(code);
+    table[code] = table_word(ps[singles[k]], best_a->slot_of);
+  }
+
+  const int identity[3] = {0, 1, 2};
+  for (size_t g = 0; g < groups.size(); g++) {
+    for (int pat = 0; pat < 8; pat++)
+      recode[groups[g].member[pat]] = static_cast<uint16_t>(nb + 8 * g + pat);
+    table[nb + g] = table_word(ps[groups[g].member[0]], identity);
+  }
+
+  if (recode_host) std::copy(recode.begin(), recode.end(), recode_host);
+  if (table_host) std::copy(table.begin(), table.end(), table_host);
+  return SUB1_OK;
+}

@@ -205,9 +205,72 @@ class ExpertStack:
                 ws.numel(), _stream()))
         return y
 
+    def prepare(self):
+        """The fast form of this stack (see PreparedStack); the stack itself
+        is left as it is and is not referenced by the result."""
+        return PreparedStack(self)
+
     def launch_faults(self, tokens):
         """(waits inside the last forward that gave up, tokens whose expert id
         was >= experts and were passed through); both 0 when all is well.
         Reads the control words of the workspace, synchronising."""
+        ctrl = self.workspace(tokens)[:16].view(torch.int32).tolist()
+        return ctrl[1], ctrl[2]
+
+
+class PreparedStack:
+    """An ExpertStack copied into the layout the GPU streams at full width
+    (rows ordered by code count, 64-row slices, interleaved and renumbered
+    codes; decode table and activations in LDS).  `forward` has the semantics
+    of ExpertStack.forward and gives identical outputs."""
+
+    def __init__(self, stack):
+        lib = _lib.load()
+        dev = stack.device
+        self.device = dev
+        self.experts, self.d_model, self.d_ff = stack.experts, stack.d_model, stack.d_ff
+        meta_bytes = lib.sub1_moe_prepared_meta_bytes(stack.experts, stack.d_model, stack.d_ff)
+        if meta_bytes <= 0:
+            raise ValueError('bad stack dimensions')
+        self.meta = torch.empty(meta_bytes, dtype=torch.uint8, device=dev)
+        code_bytes = ctypes.c_int64()
+        with torch.cuda.device(dev):
+            _lib.check(lib.sub1_moe_prepare_layout(ctypes.byref(stack._c), self.meta.data_ptr(),
+                                                   meta_bytes, ctypes.byref(code_bytes), _stream()))
+            self.codes = torch.empty(max(code_bytes.value, 256), dtype=torch.uint8, device=dev)
+            _lib.check(lib.sub1_moe_prepare_codes(ctypes.byref(stack._c), self.meta.data_ptr(),
+                                                  self.codes.data_ptr(), code_bytes.value,
+                                                  _stream()))
+        self.code_bytes = code_bytes.value
+        self._c = _lib.MoePrepared(self.meta.data_ptr(), self.codes.data_ptr(), meta_bytes,
+                                   code_bytes.value, stack.experts, stack.d_model, stack.d_ff)
+        self._ws = None
+
+    def workspace(self, tokens):
+        need = _lib.load().sub1_moe_workspace_bytes(tokens, self.d_ff)
+        if self._ws is None or self._ws.numel() < need:
+            self._ws = torch.empty(need, dtype=torch.uint8, device=self.device)
+        return self._ws
+
+    def forward(self, x, token_expert, y=None):
+        dev = self.device
+        p_x = _need(x, torch.bfloat16, 'x', dev, dim=2)
+        tokens = x.shape[0]
+        if x.shape[1] != self.d_model:
+            raise ValueError('x must be [T, %d]' % self.d_model)
+        p_te = _need(token_expert, torch.int32, 'token_expert', dev, numel=tokens)
+        if y is None:
+            y = torch.empty_like(x)
+        if tokens == 0:
+            return y
+        p_y = _need(y, torch.bfloat16, 'y', dev, numel=x.numel())
+        ws = self.workspace(tokens)
+        with torch.cuda.device(dev):
+            _lib.check(_lib.load().sub1_moe_grouped_prepared(
+                ctypes.byref(self._c), p_te, p_x, p_y, tokens, ws.data_ptr(), ws.numel(),
+                _stream()))
+        return y
+
+    def launch_faults(self, tokens):
         ctrl = self.workspace(tokens)[:16].view(torch.int32).tolist()
         return ctrl[1], ctrl[2]

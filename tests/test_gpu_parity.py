@@ -260,3 +260,87 @@ def test_grouped_launch_no_tokens_and_all_dropped(gpu, oracle):
     x = torch.randn((4, 64), device='cuda').bfloat16()
     y = stack.forward(x, torch.full((4,), -1, dtype=torch.int32, device='cuda'))
     assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize('experts,d_model,d_ff,p0', [(6, 96, 200, 0.8), (4, 768, 3072, 0.9),
+                                                     (3, 333, 77, 0.7), (2, 2080, 6144, 0.9),
+                                                     (2, 1024, 4096, 0.88)])
+def test_prepared_stack_against_oracle(gpu, oracle, experts, d_model, d_ff, p0):
+    """The fast path: same bars as the grouped launch, and identical to it."""
+    stack, wi, wo = small_stack(oracle, experts, d_model, d_ff, p0, seed=400)
+    prep = stack.prepare()
+    route = [0, 1, 0, -1, 2 % experts, 0, experts + 5, 1, 0, experts - 1]
+    xs = np.stack([so.synthetic_activation(d_model, 500 + i) for i in range(len(route))])
+    x = bf16_dev(xs)
+    te = torch.tensor(route, dtype=torch.int32, device='cuda')
+    y = prep.forward(x, te)
+    got = bits_host(y)
+    assert prep.launch_faults(len(route)) == (0, 1)
+    for i, e in enumerate(route):
+        if e < 0 or e >= experts:
+            assert np.array_equal(got[i], xs[i])
+        else:
+            want, _ = oracle.expert_ffn(wi[e], wo[e], xs[i], order=1)
+            assert np.array_equal(got[i], want), (i, e)
+            lanes, _ = oracle.expert_ffn(wi[e], wo[e], xs[i], order=0)
+            a, b = so.bf16_bits_to_f32(got[i]), so.bf16_bits_to_f32(lanes)
+            assert np.linalg.norm(a - b) <= REL_TOL * np.linalg.norm(b)
+    assert torch.equal(y, stack.forward(x, te))
+    assert torch.equal(y, prep.forward(x, te))          # workspace reuse
+
+
+def test_prepared_stack_tiny_and_huge_activations(gpu, oracle):
+    """bf16 subnormals and values near the top of the range through the
+    dot-product instruction the fast path adds with."""
+    stack, wi, wo = small_stack(oracle, 2, 128, 192, 0.6, seed=600)
+    prep = stack.prepare()
+    rng = np.random.default_rng(5)
+    scales = [1e-40, 1e-38, 1e-30, 1.0, 1e30]
+    xs = np.stack([so.f32_to_bf16_bits((rng.standard_normal(128) * sc).astype(np.float32))
+                   for sc in scales])
+    te = torch.tensor([0, 1, 0, 1, 0], dtype=torch.int32, device='cuda')
+    got = bits_host(prep.forward(bf16_dev(xs), te))
+    ref = bits_host(stack.forward(bf16_dev(xs), te))
+    for i in range(len(scales)):
+        a, b = so.bf16_bits_to_f32(got[i]).astype(np.float64), so.bf16_bits_to_f32(ref[i]).astype(np.float64)
+        assert np.all(np.isfinite(a))
+        assert np.linalg.norm(a - b) <= REL_TOL * max(np.linalg.norm(b), 1e-37), scales[i]
+
+
+def test_prepare_rejects_foreign_dictionary(gpu, oracle):
+    from qmoe_amd._lib import Sub1Error
+    from qmoe_amd import sub1, sub1_hip
+    stack, _, _ = small_stack(oracle, 2, 64, 128, 0.8, seed=700)
+    other = sub1.DEC[0].clone()
+    other[5] += 16
+    bad = sub1_hip.ExpertStack(other, stack.w_comp, stack.wi_code_base, stack.wo_code_base,
+                               stack.wi_row_off, stack.wo_row_off, stack.wi_minmax,
+                               stack.wo_minmax, 64, 128)
+    with pytest.raises(Sub1Error):
+        bad.prepare()
+
+
+def test_large_stack_paths_agree_and_match_oracle(gpu, oracle):
+    """128 Switch-base experts, one token each (the Switch-base-128 layer):
+    many tiles on many compute units, so the hand-off of the intermediate
+    activations between workgroups is exercised.  The two kernels must agree
+    everywhere, repeatedly, and sampled tokens must match the oracle."""
+    from qmoe_amd import synthetic
+    experts, d_model, d_ff = 128, 768, 3072
+    stack = synthetic.build_stack(experts, d_model, d_ff, 0.9, seed=99)
+    prep = stack.prepare()
+    x = synthetic.activations(experts, d_model, seed=100)
+    route = torch.arange(experts, dtype=torch.int32, device='cuda')
+    y_ref = stack.forward(x, route).clone()
+    for _ in range(5):
+        assert torch.equal(prep.forward(x, route), y_ref)
+        assert torch.equal(stack.forward(x, route), y_ref)
+    assert prep.launch_faults(experts) == (0, 0)
+    got = bits_host(y_ref)
+    xs = bits_host(x)
+    for e in (0, 17, 63, 127):
+        wi, wo = synthetic.expert_layers(stack, e)
+        host = [tuple(bits_host(t) if t.dtype != torch.int32 else t.cpu().numpy() for t in l)
+                for l in (wi, wo)]
+        want, _ = oracle.expert_ffn(host[0], host[1], xs[e], order=1)
+        assert np.array_equal(got[e], want), e
