@@ -22,6 +22,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 counter runs of this same
+# command (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a 1 GiB device copy reads on
+# those counters); the summaries are under profiles/.  None where no run was made.
+MEASURED_TRAFFIC = {'c2048-sweep': 4.85e9 + 0.234e9}
+
 WORKLOADS = {
     # name: (shape key, experts, p_zero, description)
     'c2048-sweep': ('c2048', 2048, 0.90,
@@ -130,10 +135,25 @@ def main():
     ap.add_argument('--experts', type=int, default=0, help='override the expert count (debugging)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline')
     ap.add_argument('--no-dense', action='store_true', help='skip the dense bf16 comparison')
+    ap.add_argument('--sweep-only', action='store_true',
+                    help='only the headline sweep (what a profiler run should see)')
     ap.add_argument('--seed', type=int, default=20231116)
+    ap.add_argument('--calibrate-copy', type=int, default=0, metavar='MIB',
+                    help='instead of the benchmark, run a plain device copy of this many MiB '
+                         '(to scale the FETCH_SIZE / WRITE_SIZE counters of a profiler run)')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py measures one GPU: this build has no multi-GPU path (--gpus 1 only)')
+    if args.calibrate_copy:
+        import torch
+        n = args.calibrate_copy << 20
+        src = torch.ones(n, dtype=torch.uint8, device='cuda')
+        dst = torch.empty_like(src)
+        for _ in range(args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({'copy_bytes_read': n, 'copy_bytes_written': n, 'copies': args.steps}))
+        return
 
     import ctypes
     import torch
@@ -186,10 +206,14 @@ def main():
                                             / (2.0 * experts * d_model * d_ff), 4)},
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS,
                      'unit': 'GB/s', 'frac': round(achieved / HBM_PEAK_GBS, 4),
-                     'traffic': None, 'kernel': 'moe_prepared_kernel',
+                     'traffic': MEASURED_TRAFFIC.get(args.workload) if not args.experts else None,
+                     'kernel': 'moe_prepared_kernel',
                      'algorithmic_bytes': abytes, 'us_per_launch': round(us_launch, 2)},
     }
 
+    if args.sweep_only:
+        print(json.dumps(out))
+        return
     also = {}
     # batch-1: one token routed to one seeded uniform expert (launch-latency bound)
     g = torch.Generator().manual_seed(args.seed + 2)
