@@ -37,8 +37,7 @@ using sub1::row_result;
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kThreads = 1024;
-constexpr int kWaves = kThreads / 64;
+constexpr int kMaxThreads = 1024;      // the launch picks 8..16 wavefronts per workgroup
 constexpr int kChunk = 4;            // codes per lane per chunk
 constexpr int kRing = 4;             // chunks in flight per lane
 constexpr int kMaxLen = 4096;        // codes per row: one per column pair at most
@@ -233,7 +232,7 @@ struct KindArgs {
   const uint16_t *row_len;
   const uint16_t *row_idx;
   const uint32_t *minmax;
-  int slices, height, width, tiles;
+  int slices, height, width, parts;
 };
 
 struct PreparedArgs {
@@ -262,7 +261,7 @@ __host__ __device__ constexpr int activation_dwords(int width) {
 
 __device__ __forceinline__ void stage_activations(uint32_t *xa, const uint16_t *x, int width) {
   const int npairs = (width + 28 + 1) / 2 + 1;
-  for (int m = threadIdx.x; m < npairs; m += kThreads) {
+  for (int m = threadIdx.x; m < npairs; m += blockDim.x) {
     uint32_t xe = 2 * m < width ? x[2 * m] : 0u;
     uint32_t xo = 2 * m + 1 < width ? x[2 * m + 1] : 0u;
     uint32_t *p = xa + 6 * m;
@@ -291,12 +290,28 @@ __device__ __forceinline__ DotConsts dot_consts() {
   return c;
 }
 
-// Table word of kernel code c with the code's symbol bits put in place.
-__device__ __forceinline__ uint32_t lookup(const uint32_t *tab, uint32_t c, int group_shift) {
-  uint32_t idx = min(c, (c >> 3) + static_cast<uint32_t>(group_shift));
-  uint32_t word = tab[idx];
-  uint32_t bits = (c & 7u) * 0x4081u;      // bit j of c -> bit 8j
-  return (word & ~0x00010101u) | (bits & 0x00010101u);
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+// Table words of the two kernel codes packed in `pair`, with each code's symbol
+// bits put in place.  idx = min(c, (c >> 3) + group_shift) per 16-bit half.
+__device__ __forceinline__ void lookup2(const uint32_t *tab, uint32_t pair, uint32_t shift2,
+                                        uint32_t &e_lo, uint32_t &e_hi) {
+  u16x2 c = __builtin_bit_cast(u16x2, pair);
+  u16x2 g = (c >> static_cast<unsigned short>(3)) + __builtin_bit_cast(u16x2, shift2);
+  u16x2 idx = __builtin_elementwise_min(c, g);
+  uint32_t w_lo = tab[idx.x];
+  uint32_t w_hi = tab[idx.y];
+  uint32_t sym = pair & 0x00070007u;
+  uint32_t b_lo = (sym & 0xffffu) * 0x4081u;   // bit j of the code -> bit 8j
+  uint32_t b_hi = (sym >> 16) * 0x4081u;
+  e_lo = (w_lo & ~0x00010101u) | (b_lo & 0x00010101u);
+  e_hi = (w_hi & ~0x00010101u) | (b_hi & 0x00010101u);
+}
+
+__device__ __forceinline__ void lookup4(const uint32_t *tab, uint2 w, uint32_t shift2,
+                                        uint32_t (&e)[4]) {
+  lookup2(tab, w.x, shift2, e[0], e[1]);
+  lookup2(tab, w.y, shift2, e[2], e[3]);
 }
 
 __device__ __forceinline__ void add_codeword(uint32_t e, const uint32_t *xa, int &colw,
@@ -311,40 +326,54 @@ __device__ __forceinline__ void add_codeword(uint32_t e, const uint32_t *xa, int
   colw += static_cast<int>(e >> 24);
 }
 
-// The two sums of this lane's row of slice `sl`.
-__device__ __forceinline__ void slice_sums(const PreparedArgs &a, const KindArgs &k,
-                                           int64_t sl, const uint32_t *tab,
-                                           const uint32_t *xa, float &s1, float &s2) {
+// What a lane needs to walk its row of one slice; load_slice issues the loads
+// of the first chunks, so calling it for the NEXT slice before walking the
+// current one hides their latency.
+struct SliceWalk {
+  const uint2 *p;
+  int nch, nfull, len, ridx;
+  uint32_t minmax;
+  uint2 ring[kRing];
+};
+
+__device__ __forceinline__ SliceWalk load_slice(const PreparedArgs &a, const KindArgs &k,
+                                                int64_t sl) {
   const int lane = threadIdx.x & 63;
+  SliceWalk w;
+  w.nch = __builtin_amdgcn_readfirstlane(k.slice_nch[sl]);
+  w.nfull = __builtin_amdgcn_readfirstlane(k.slice_nfull[sl]);
+  w.len = k.row_len[sl * 64 + lane];
+  w.ridx = k.row_idx[sl * 64 + lane];
+  w.minmax = k.minmax[sl * 64 + lane];
+  w.p = reinterpret_cast<const uint2 *>(a.codes + static_cast<int64_t>(k.slice_base[sl]) * 256) +
+        lane;
+#pragma unroll
+  for (int i = 0; i < kRing; i++)
+    if (i < w.nch) w.ring[i] = w.p[i * 64];
+  return w;
+}
+
+// The two sums of this lane's row.
+__device__ __forceinline__ void run_slice(SliceWalk &w, int group_shift, const uint32_t *tab,
+                                          const uint32_t *xa, float &s1, float &s2) {
   const DotConsts dk = dot_consts();
-  const int nch = __builtin_amdgcn_readfirstlane(k.slice_nch[sl]);
-  const int nfull = __builtin_amdgcn_readfirstlane(k.slice_nfull[sl]);
-  const int len = k.row_len[sl * 64 + lane];
-  const uint2 *p =
-      reinterpret_cast<const uint2 *>(a.codes + static_cast<int64_t>(k.slice_base[sl]) * 256) +
-      lane;
+  const uint32_t shift2 = static_cast<uint32_t>(group_shift) * 0x00010001u;
+  const int nch = w.nch, nfull = w.nfull, len = w.len;
+  const uint2 *p = w.p;
   s1 = 0.f;
   s2 = 0.f;
   int colw = 0;
-  uint2 ring[kRing];
-#pragma unroll
-  for (int i = 0; i < kRing; i++)
-    if (i < nch) ring[i] = p[i * 64];
   int c = 0;
   // chunks every lane of the slice has in full: no per-code checks
   for (; c + kRing <= nfull; c += kRing) {
 #pragma unroll
     for (int i = 0; i < kRing; i++) {
-      uint2 w = ring[i];
-      if (c + kRing + i < nch) ring[i] = p[(c + kRing + i) * 64];
-      uint32_t e0 = lookup(tab, w.x & 0xffffu, a.group_shift);
-      uint32_t e1 = lookup(tab, w.x >> 16, a.group_shift);
-      uint32_t e2 = lookup(tab, w.y & 0xffffu, a.group_shift);
-      uint32_t e3 = lookup(tab, w.y >> 16, a.group_shift);
-      add_codeword(e0, xa, colw, s1, s2, dk);
-      add_codeword(e1, xa, colw, s1, s2, dk);
-      add_codeword(e2, xa, colw, s1, s2, dk);
-      add_codeword(e3, xa, colw, s1, s2, dk);
+      const uint2 cw = w.ring[i];
+      if (c + kRing + i < nch) w.ring[i] = p[(c + kRing + i) * 64];
+      uint32_t e[4];
+      lookup4(tab, cw, shift2, e);
+#pragma unroll
+      for (int q = 0; q < 4; q++) add_codeword(e[q], xa, colw, s1, s2, dk);
     }
   }
   // the rest, each code checked against the lane's own count
@@ -352,120 +381,124 @@ __device__ __forceinline__ void slice_sums(const PreparedArgs &a, const KindArgs
 #pragma unroll
     for (int i = 0; i < kRing; i++) {
       if (c + i < nch) {
-        uint2 w = ring[i];
-        if (c + kRing + i < nch) ring[i] = p[(c + kRing + i) * 64];
+        const uint2 cw = w.ring[i];
+        if (c + kRing + i < nch) w.ring[i] = p[(c + kRing + i) * 64];
+        uint32_t e[4];
+        lookup4(tab, cw, shift2, e);
         const int j = kChunk * (c + i);
-        uint32_t e0 = lookup(tab, w.x & 0xffffu, a.group_shift);
-        uint32_t e1 = lookup(tab, w.x >> 16, a.group_shift);
-        uint32_t e2 = lookup(tab, w.y & 0xffffu, a.group_shift);
-        uint32_t e3 = lookup(tab, w.y >> 16, a.group_shift);
-        if (j + 0 >= len) e0 = kIdleWord;
-        if (j + 1 >= len) e1 = kIdleWord;
-        if (j + 2 >= len) e2 = kIdleWord;
-        if (j + 3 >= len) e3 = kIdleWord;
-        add_codeword(e0, xa, colw, s1, s2, dk);
-        add_codeword(e1, xa, colw, s1, s2, dk);
-        add_codeword(e2, xa, colw, s1, s2, dk);
-        add_codeword(e3, xa, colw, s1, s2, dk);
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+          add_codeword(j + q < len ? e[q] : kIdleWord, xa, colw, s1, s2, dk);
       }
     }
   }
 }
 
-// Persistent grid; tiles = (token, projection, 16 slices), all wi tiles
-// numbered before all wo tiles and handed out by an atomic ticket.  A wo tile
-// waits for the wi tiles of its token, which hold smaller tickets and so are
-// running or done: the wait always ends.  h is published by ONE agent-scope
-// release per tile (thread 0, after the workgroup barrier) and picked up by one
-// acquire; an agent-scope fence costs an L2 write-back on this part, which is
-// why the lanes do not fence individually.
-__global__ __launch_bounds__(kThreads) void moe_prepared_kernel(PreparedArgs a) {
+// Persistent grid.  A tile is (token, projection, part): the slices of one
+// matrix, or of one of `parts` equal ranges of them when there are too few
+// tokens to occupy the GPU otherwise; a workgroup stages the token's
+// activations once per tile and its wavefronts take the tile's slices in turn.
+// All wi tiles are numbered before all wo tiles and handed out by an atomic
+// ticket.  A wo tile waits for the wi tiles of its token, which hold smaller
+// tickets and so are running or done: the wait always ends.  h is published by
+// ONE agent-scope release per tile (thread 0, after every wavefront drained its
+// stores and the workgroup barrier) and picked up by one acquire; an agent-scope
+// fence costs an L2 write-back on this part, which is why the lanes do not fence
+// individually.
+__global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs a) {
   extern __shared__ uint32_t lds[];
   __shared__ int s_ticket;
   uint32_t *tab = lds;
   uint32_t *xa = lds + a.table_words;
-  for (int i = threadIdx.x; i < a.table_words; i += kThreads) tab[i] = a.table[i];
-  const int n_wi = a.tokens * a.k[0].tiles;
-  const int n_all = n_wi + a.tokens * a.k[1].tiles;
+  const int threads = blockDim.x;
+  const int waves = threads >> 6;
+  for (int i = threadIdx.x; i < a.table_words; i += threads) tab[i] = a.table[i];
+  const int n_wi = a.tokens * a.k[0].parts;
+  const int n_all = n_wi + a.tokens * a.k[1].parts;
   const int wave = threadIdx.x >> 6;
-  const int lane = threadIdx.x & 63;
+  // thread 0 keeps one ticket ahead so that the atomic's round trip overlaps a tile
+  int next_ticket = 0;
+  if (threadIdx.x == 0)
+    next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
   for (;;) {
     __syncthreads();
-    if (threadIdx.x == 0)
-      s_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
-                                        __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) {
+      s_ticket = next_ticket;
+      if (next_ticket < n_all)
+        next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
+    }
     __syncthreads();
     const int ticket = s_ticket;
     if (ticket >= n_all) break;
     const int kind = ticket < n_wi ? 0 : 1;
     const KindArgs &k = a.k[kind];
     const int rel = kind ? ticket - n_wi : ticket;
-    const int t = rel / k.tiles;
-    const int tile = rel - t * k.tiles;
+    const int t = rel / k.parts;
+    const int part = rel - t * k.parts;
+    // slices [s_lo, s_hi) of the matrix
+    const int s_lo = static_cast<int>(static_cast<int64_t>(k.slices) * part / k.parts);
+    const int s_hi = static_cast<int>(static_cast<int64_t>(k.slices) * (part + 1) / k.parts);
     int e = a.token_expert[t];
     if (e >= a.experts) {
-      if (kind == 1 && tile == 0 && threadIdx.x == 0)
+      if (kind == 1 && part == 0 && threadIdx.x == 0)
         __hip_atomic_fetch_add(&a.ctrl[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       e = -1;
     }
-    if (kind == 0) {
-      if (e >= 0) {
-        stage_activations(xa, a.x + static_cast<int64_t>(t) * k.width, k.width);
-        __syncthreads();
-        const int s = tile * kWaves + wave;
-        if (s < k.slices) {
-          const int64_t sl = static_cast<int64_t>(e) * k.slices + s;
-          float s1, s2;
-          slice_sums(a, k, sl, tab, xa, s1, s2);
-          const int ridx = k.row_idx[sl * 64 + lane];
-          if (ridx != 0xffff) {
-            uint16_t hb = f32_to_bf16(row_result(k.minmax[sl * 64 + lane], s1, s2));
-            if (hb & 0x8000u) hb = 0;  // relu
-            a.h[static_cast<int64_t>(t) * k.height + ridx] = hb;
+    if (kind == 1 && e < 0) {
+      // a dropped token keeps its input (reference sub1.py:312)
+      const int r_lo = min(64 * s_lo, k.height), r_hi = min(64 * s_hi, k.height);
+      for (int i = r_lo + threadIdx.x; i < r_hi; i += threads) {
+        int64_t g = static_cast<int64_t>(t) * k.height + i;
+        a.y[g] = a.x[g];
+      }
+      continue;
+    }
+    if (e >= 0) {
+      // the first slice's loads go out before the wait and the staging
+      int s = s_lo + wave;
+      SliceWalk cur;
+      if (s < s_hi) cur = load_slice(a, k, static_cast<int64_t>(e) * k.slices + s);
+      if (kind == 1) {
+        if (threadIdx.x == 0) {
+          int spins = 0;
+          while (__hip_atomic_load(&a.ctrl[kCtrlHeader + t], __ATOMIC_ACQUIRE,
+                                   __HIP_MEMORY_SCOPE_AGENT) < a.k[0].parts) {
+            if (++spins > a.spin_limit) {
+              __hip_atomic_fetch_add(&a.ctrl[1], 1, __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_AGENT);
+              break;
+            }
+            __builtin_amdgcn_s_sleep(8);
           }
         }
+        __syncthreads();  // thread 0's acquire now covers the whole workgroup
       }
+      const uint16_t *src = kind ? a.h : a.x;
+      stage_activations(xa, src + static_cast<int64_t>(t) * k.width, k.width);
+      __syncthreads();
+      uint16_t *dst = (kind ? a.y : a.h) + static_cast<int64_t>(t) * k.height;
+      for (; s < s_hi; s += waves) {
+        const bool more = s + waves < s_hi;
+        SliceWalk nxt;
+        if (more) nxt = load_slice(a, k, static_cast<int64_t>(e) * k.slices + s + waves);
+        float s1, s2;
+        run_slice(cur, a.group_shift, tab, xa, s1, s2);
+        if (cur.ridx != 0xffff) {
+          uint16_t out = f32_to_bf16(row_result(cur.minmax, s1, s2));
+          if (kind == 0 && (out & 0x8000u)) out = 0;  // relu between the projections
+          dst[cur.ridx] = out;
+        }
+        if (more) cur = nxt;
+      }
+    }
+    if (kind == 0) {
       sub1::drain_stores();   // this wavefront's h stores are in L2 ...
       __syncthreads();        // ... so are everyone's, and thread 0's release publishes them
       if (threadIdx.x == 0)
         __hip_atomic_fetch_add(&a.ctrl[kCtrlHeader + t], 1, __ATOMIC_RELEASE,
                                __HIP_MEMORY_SCOPE_AGENT);
-    } else {
-      if (e < 0) {
-        // a dropped token keeps its input (reference sub1.py:312)
-        for (int i = tile * kThreads + threadIdx.x; i < min(k.height, (tile + 1) * kThreads);
-             i += kThreads) {
-          int64_t g = static_cast<int64_t>(t) * k.height + i;
-          a.y[g] = a.x[g];
-        }
-        // rows of a dropped token beyond the tiles' reach (height > tiles*1024 cannot
-        // happen: tiles covers every slice)
-        continue;
-      }
-      if (threadIdx.x == 0) {
-        int spins = 0;
-        while (__hip_atomic_load(&a.ctrl[kCtrlHeader + t], __ATOMIC_ACQUIRE,
-                                 __HIP_MEMORY_SCOPE_AGENT) < a.k[0].tiles) {
-          if (++spins > a.spin_limit) {
-            __hip_atomic_fetch_add(&a.ctrl[1], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            break;
-          }
-          __builtin_amdgcn_s_sleep(8);
-        }
-      }
-      __syncthreads();
-      stage_activations(xa, a.h + static_cast<int64_t>(t) * k.width, k.width);
-      __syncthreads();
-      const int s = tile * kWaves + wave;
-      if (s < k.slices) {
-        const int64_t sl = static_cast<int64_t>(e) * k.slices + s;
-        float s1, s2;
-        slice_sums(a, k, sl, tab, xa, s1, s2);
-        const int ridx = k.row_idx[sl * 64 + lane];
-        if (ridx != 0xffff)
-          a.y[static_cast<int64_t>(t) * k.height + ridx] =
-              f32_to_bf16(row_result(k.minmax[sl * 64 + lane], s1, s2));
-      }
     }
   }
 }
@@ -688,7 +721,21 @@ extern "C" int sub1_moe_grouped_prepared(const sub1_moe_prepared *p, const int32
     a.k[i].slices = k.slices;
     a.k[i].height = k.height;
     a.k[i].width = k.width;
-    a.k[i].tiles = (k.slices + kWaves - 1) / kWaves;
+  }
+  // 16 wavefronts per workgroup.  A count that divides the slice counts better
+  // (11 for the c-2048 shapes) leaves fewer idle wavefront slots but measured
+  // 10% slower: the kernel needs the wavefronts to hide LDS latency.
+  const int waves = 16;
+  int device = 0, cus = 0;
+  HIP_TRY(hipGetDevice(&device));
+  HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+  // Whole matrices per tile when the tokens alone give every compute unit two
+  // tiles; otherwise each matrix is cut into parts, down to one slice per
+  // wavefront.
+  for (int i = 0; i < 2; i++) {
+    int max_parts = (a.k[i].slices + waves - 1) / waves;
+    int want = (2 * cus + 2 * tokens - 1) / (2 * tokens);
+    a.k[i].parts = want < 1 ? 1 : (want > max_parts ? max_parts : want);
   }
   a.token_expert = token_expert;
   a.x = static_cast<const uint16_t *>(x);
@@ -704,7 +751,7 @@ extern "C" int sub1_moe_grouped_prepared(const sub1_moe_prepared *p, const int32
   int wmax = p->d_model > p->d_ff ? p->d_model : p->d_ff;
   a.xdwords = activation_dwords(wmax);
   a.spin_limit = 1 << 24;
-  int64_t tiles = static_cast<int64_t>(tokens) * (a.k[0].tiles + a.k[1].tiles);
+  int64_t tiles = static_cast<int64_t>(tokens) * (a.k[0].parts + a.k[1].parts);
   if (tiles > INT32_MAX - (1 << 20))
     return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: too many tiles");
 
@@ -713,14 +760,11 @@ extern "C" int sub1_moe_grouped_prepared(const sub1_moe_prepared *p, const int32
     return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: width %d does not fit LDS", wmax);
   HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(moe_prepared_kernel),
                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-  int device = 0, cus = 0;
-  HIP_TRY(hipGetDevice(&device));
-  HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
-  int64_t grid = cus;  // one 1024-lane workgroup per compute unit
+  int64_t grid = cus;  // one workgroup per compute unit (LDS holds the table once)
   if (grid > tiles) grid = tiles;
   int nctrl = kCtrlHeader + tokens;
   zero_words_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl);
-  moe_prepared_kernel<<<static_cast<unsigned>(grid), kThreads, lds, s>>>(a);
+  moe_prepared_kernel<<<static_cast<unsigned>(grid), 64 * waves, lds, s>>>(a);
   HIP_TRY(hipGetLastError());
   return SUB1_OK;
 }
