@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 counter runs of this same
 # command (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a 1 GiB device copy reads on
 # those counters); the summaries are under profiles/.  None where no run was made.
-MEASURED_TRAFFIC = {'c2048-sweep': 4.85e9 + 0.234e9}
+MEASURED_TRAFFIC = {'c2048-sweep': 4.78e9 + 0.208e9}
 
 WORKLOADS = {
     # name: (shape key, experts, p_zero, description)
@@ -226,16 +226,45 @@ def main():
     _, us_ref = time_launches(lambda: stack.forward(x, route, y2), 3, 1, stream_ptr)
     also['reference_layout_kernel_us'] = round(us_ref, 1)
     also['prepared_equals_reference_layout'] = bool(torch.equal(y, y2))
+    # batched decode: 64 tokens routed top-1 by a seeded softmax router (skewed counts)
+    t5 = 64
+    x5 = synthetic.activations(t5, d_model, args.seed + 3)
+    r5 = synthetic.softmax_router(t5, experts, args.seed + 4)
+    y5 = torch.empty_like(x5)
+    _, us5 = time_launches(lambda: prep.forward(x5, r5, y5), 100, 10, stream_ptr)
+    y5b = stack.forward(x5, r5)
+    also['routed_64_tokens'] = {'us_per_layer': round(us5, 2),
+                                'experts_hit': int(torch.unique(r5).numel()),
+                                'equals_reference_layout_kernel': bool(torch.equal(y5, y5b))}
     if not args.no_dense:
         n = min(experts, 128)
         d_us = dense_gemv_us(stack, x, n)
         also['dense_bf16_gemv'] = {'us_per_expert_ffn': round(d_us, 2), 'experts_timed': n,
                                    'us_per_layer_extrapolated': round(d_us * experts, 1),
                                    'sub1_us_per_expert_ffn': round(us_launch / experts, 2)}
+    if not args.experts and args.workload == 'c2048-sweep':
+        # the two smaller layers of the configuration list; their compressed stacks
+        # (57 MB, 110 MB) fit the 256 MB last-level cache, so these are not HBM rates
+        for name in ('base128', 'large128'):
+            shp, n_e, p_z, _ = WORKLOADS[name]
+            dm, df = synthetic.SHAPES[shp]
+            st = synthetic.build_stack(n_e, dm, df, p_z, args.seed + 10)
+            pr = st.prepare()
+            xs = synthetic.activations(n_e, dm, args.seed + 11)
+            rt = torch.arange(n_e, dtype=torch.int32, device='cuda')
+            ys = torch.empty_like(xs)
+            _, us_s = time_launches(lambda: pr.forward(xs, rt, ys), 100, 10, stream_ptr)
+            ab = algorithmic_bytes(st, range(n_e))
+            entry = {'us_per_layer': round(us_s, 2), 'algorithmic_bytes': ab,
+                     'GBps_cache_resident': round(ab / us_s / 1e3, 1)}
+            if name == 'large128' and not args.no_dense:
+                entry['dense_bf16_gemv_us_per_layer'] = round(dense_gemv_us(st, xs, n_e) * n_e, 1)
+            also[name] = entry
+            del st, pr
     out['also'] = also
 
     if not args.no_cpu:
-        done, spent = cpu_baseline(stack, x, min(experts, 64))
+        done, spent = cpu_baseline(stack, x, min(experts, 512))
         out['cpu_baseline'] = {
             'value': round(spent / done * experts * 1e6, 1), 'unit': 'us/layer', 'cores': 1,
             'kind': 'port',

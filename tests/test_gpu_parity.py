@@ -344,3 +344,29 @@ def test_large_stack_paths_agree_and_match_oracle(gpu, oracle):
                 for l in (wi, wo)]
         want, _ = oracle.expert_ffn(host[0], host[1], xs[e], order=1)
         assert np.array_equal(got[e], want), e
+
+
+def test_routed_batch_equals_per_token_products(gpu):
+    """64 tokens routed top-1 by a softmax router over c-2048-shaped experts
+    (skewed per-expert counts, experts with no token): the one-launch result
+    must equal what the per-token calls of the reference's loop give
+    (sub1.py:139-142 and 315-317: wi product, ReLU, wo product per token)."""
+    from qmoe_amd import sub1, sub1_hip, synthetic
+    experts, d_model, d_ff, tokens = 48, 2080, 6144, 64
+    stack = synthetic.build_stack(experts, d_model, d_ff, 0.9, seed=5)
+    prep = stack.prepare()
+    x = synthetic.activations(tokens, d_model, seed=6)
+    route = synthetic.softmax_router(tokens, experts, seed=7)
+    counts = torch.bincount(route.long(), minlength=experts)
+    assert counts.max() >= 2 and (counts == 0).any()        # skewed, some experts idle
+    y = prep.forward(x, route)
+    assert torch.equal(y, stack.forward(x, route))
+    dec = sub1.DEC[0]
+    for t in range(tokens):
+        wi, wo = synthetic.expert_layers(stack, int(route[t]))
+        h = torch.zeros(d_ff, dtype=torch.bfloat16, device='cuda')
+        sub1_hip.sub1matvec(dec, wi[0], wi[1], wi[2], x[t], h)
+        h = torch.relu(h)
+        out = torch.zeros(d_model, dtype=torch.bfloat16, device='cuda')
+        sub1_hip.sub1matvec(dec, wo[0], wo[1], wo[2], h, out)
+        assert torch.equal(out, y[t]), t
