@@ -14,7 +14,7 @@
  *   sub1o_decode         sub1_cuda_kernel.cu:186-192, test.py:103-115
  *   sub1o_dequant        test.py:110, sub1_cuda_kernel.cu:156-157,170-171
  *   sub1o_matvec_lanes   sub1_cuda_kernel.cu:143-201 (lane order, tree, y +=)
- *   sub1o_matvec_seq     same sums, taken per symbol in stream order
+ *   sub1o_matvec_seq     same sums, taken per symbol, in groups of 32 codes
  *   sub1o_matvec_f64     textbook GEMV in double on the decoded matrix
  *   sub1o_expert_ffn     sub1.py:132-143 twice with ReLU between (the
  *                        DenseActDense call made at sub1.py:317)
@@ -328,25 +328,35 @@ void sub1o_matvec_lanes(const int32_t *dec, const uint16_t *codes,
   free(xs);
 }
 
-/* Same product with the summation taken per symbol in stream order: s1 = sum
- * of x over the weights with symbol 1, s2 likewise for symbol 2, both in fp32
- * walking the row left to right, then res = fma(min, s1, max*s2), bf16, +=.
- * A second fp32 ordering of the same sum, used to check kernels that add
- * activations rather than multiply. */
+/* Same product in the order the HIP kernels add: s1 = sum of x over the weights
+ * with symbol 1, s2 likewise for symbol 2, both in fp32.  A row's codes are
+ * taken in groups of SUB1O_GROUP consecutive codes; within a group the
+ * activations are added left to right onto a partial sum that starts at zero,
+ * and the partial sums are added, first group first, onto the row's sum.  Then
+ * res = fma(min, s1, max*s2), bf16, +=.  A second fp32 ordering of the same
+ * sum as sub1o_matvec_lanes. */
+#define SUB1O_GROUP 32
+
 void sub1o_matvec_seq(const int32_t *dec, const uint16_t *codes,
                       const int32_t *row_off, const uint16_t *ter_minmax,
                       const uint16_t *x, uint16_t *y, int height, int width) {
   for (int r = 0; r < height; r++) {
     float s[3] = {0.f, 0.f, 0.f};
     int idx = 0;
-    for (int c = row_off[r]; c < row_off[r + 1]; c++) {
-      int e = codes[c];
-      int n = 2 * (dec[2 * e] & 0xf);
-      for (int d = 0; d < n && idx + d < width; d++) {
-        int t = entry_digit(dec, e, d);
-        if (t) s[t] += bf16_to_f32(x[idx + d]);
+    for (int c0 = row_off[r]; c0 < row_off[r + 1]; c0 += SUB1O_GROUP) {
+      float p[3] = {0.f, 0.f, 0.f};
+      int c1 = c0 + SUB1O_GROUP < row_off[r + 1] ? c0 + SUB1O_GROUP : row_off[r + 1];
+      for (int c = c0; c < c1; c++) {
+        int e = codes[c];
+        int n = 2 * (dec[2 * e] & 0xf);
+        for (int d = 0; d < n && idx + d < width; d++) {
+          int t = entry_digit(dec, e, d);
+          if (t) p[t] += bf16_to_f32(x[idx + d]);
+        }
+        idx += n;
       }
-      idx += n;
+      s[1] += p[1];
+      s[2] += p[2];
     }
     float res = fmaf(bf16_to_f32(ter_minmax[2 * r]), s[1],
                      bf16_to_f32(ter_minmax[2 * r + 1]) * s[2]);

@@ -127,13 +127,17 @@ __device__ __forceinline__ void load_codes8(const uint16_t *p, uint32_t (&w)[4])
   __builtin_memcpy(w, p, 16);
 }
 
-// Sum of activations under the symbol-1 and symbol-2 weights of one row, each
-// in fp32 in column order.
+// Sum of activations under the symbol-1 and symbol-2 weights of one row, in
+// fp32, in the library's canonical order: the row's codes in groups of 32, a
+// partial sum per group taken left to right from zero, the partial sums added
+// first group first.  (The grouping lets the prepared kernels split a row
+// between wavefronts without changing a bit of the result.)
 __device__ __forceinline__ void row_sums(const uint32_t *__restrict__ tab,
                                          const uint16_t *__restrict__ codes, int len,
                                          const float *M, float &s1, float &s2) {
   s1 = 0.f;
   s2 = 0.f;
+  float p1 = 0.f, p2 = 0.f;
   int colw = 0;
   int i = 0;
   uint32_t w[4];
@@ -148,7 +152,13 @@ __device__ __forceinline__ void row_sums(const uint32_t *__restrict__ tab,
       e[2 * j + 1] = tab[cur[j] >> 16];
     }
 #pragma unroll
-    for (int j = 0; j < 8; j++) add_codeword(e[j], M, colw, s1, s2);
+    for (int j = 0; j < 8; j++) add_codeword(e[j], M, colw, p1, p2);
+    if (((i + 8) & 31) == 0) {   // a group of 32 codes is complete
+      s1 += p1;
+      s2 += p2;
+      p1 = 0.f;
+      p2 = 0.f;
+    }
   }
   int rem = len - i;
   if (rem > 0) {
@@ -161,12 +171,14 @@ __device__ __forceinline__ void row_sums(const uint32_t *__restrict__ tab,
         uint32_t code = (j & 1) ? (w[j / 2] >> 16) : (w[j / 2] & 0xffffu);
         uint32_t e = tab[code];
         if (j < skip) e = 0u;  // entry 0 of the slot form: nothing, no advance
-        add_codeword(e, M, colw, s1, s2);
+        add_codeword(e, M, colw, p1, p2);
       }
     } else {
-      for (int j = 0; j < rem; j++) add_codeword(tab[codes[j]], M, colw, s1, s2);
+      for (int j = 0; j < rem; j++) add_codeword(tab[codes[j]], M, colw, p1, p2);
     }
   }
+  s1 += p1;   // the last, possibly partial, group (adds +0 if it was just folded)
+  s2 += p2;
 }
 
 // ------------------------------------------------------------- matvec ------

@@ -39,7 +39,8 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kMaxThreads = 1024;      // the launch picks 8..16 wavefronts per workgroup
 constexpr int kChunk = 4;            // codes per lane per chunk
-constexpr int kRing = 4;             // chunks in flight per lane
+constexpr int kRing = 4;             // chunks in flight per lane (2 KB per wavefront)
+constexpr int kGroupChunks = 8;      // chunks (32 codes) per partial sum, a multiple of kRing
 constexpr int kMaxLen = 4096;        // codes per row: one per column pair at most
 constexpr int kCtrlHeader = 4;       // ctrl[0] ticket, [1] wait-limit hits, [2] bad expert ids
 constexpr uint32_t kIdleWord = 0x00040404u;  // three empty slots, no advance
@@ -353,45 +354,63 @@ __device__ __forceinline__ SliceWalk load_slice(const PreparedArgs &a, const Kin
   return w;
 }
 
-// The two sums of this lane's row.
+// kRing chunks starting at chunk c added onto the partial sums p1, p2.
+// kChecked: compare every code with the lane's own count.
+template <bool kChecked>
+__device__ __forceinline__ void run_chunks(SliceWalk &w, int c, uint32_t shift2,
+                                           const uint32_t *tab, const uint32_t *xa, int &colw,
+                                           float &p1, float &p2, const DotConsts &dk) {
+  const uint2 *p = w.p;
+  const int nch = w.nch;
+#pragma unroll
+  for (int i = 0; i < kRing; i++) {
+    if (!kChecked || c + i < nch) {
+      const uint2 cw = w.ring[i];
+      if (c + i + kRing < nch) w.ring[i] = p[(c + i + kRing) * 64];
+      uint32_t e[4];
+      lookup4(tab, cw, shift2, e);
+      const int j = kChunk * (c + i);
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+        add_codeword(!kChecked || j + q < w.len ? e[q] : kIdleWord, xa, colw, p1, p2, dk);
+    }
+  }
+}
+
+// The two sums of this lane's row, in the library's canonical order: groups of
+// 32 codes (kGroupChunks chunks), a partial sum per group from zero, the
+// partial sums added first group first.  Starts at chunk c0 (a multiple of
+// kGroupChunks) with column offset colw and stops before chunk c_end.
 __device__ __forceinline__ void run_slice(SliceWalk &w, int group_shift, const uint32_t *tab,
                                           const uint32_t *xa, float &s1, float &s2) {
   const DotConsts dk = dot_consts();
   const uint32_t shift2 = static_cast<uint32_t>(group_shift) * 0x00010001u;
-  const int nch = w.nch, nfull = w.nfull, len = w.len;
-  const uint2 *p = w.p;
   s1 = 0.f;
   s2 = 0.f;
+  float p1 = 0.f, p2 = 0.f;
   int colw = 0;
   int c = 0;
   // chunks every lane of the slice has in full: no per-code checks
-  for (; c + kRing <= nfull; c += kRing) {
-#pragma unroll
-    for (int i = 0; i < kRing; i++) {
-      const uint2 cw = w.ring[i];
-      if (c + kRing + i < nch) w.ring[i] = p[(c + kRing + i) * 64];
-      uint32_t e[4];
-      lookup4(tab, cw, shift2, e);
-#pragma unroll
-      for (int q = 0; q < 4; q++) add_codeword(e[q], xa, colw, s1, s2, dk);
+  for (; c + kRing <= w.nfull; c += kRing) {
+    run_chunks<false>(w, c, shift2, tab, xa, colw, p1, p2, dk);
+    if ((c + kRing) % kGroupChunks == 0) {
+      s1 += p1;
+      s2 += p2;
+      p1 = 0.f;
+      p2 = 0.f;
     }
   }
-  // the rest, each code checked against the lane's own count
-  for (; c < nch; c += kRing) {
-#pragma unroll
-    for (int i = 0; i < kRing; i++) {
-      if (c + i < nch) {
-        const uint2 cw = w.ring[i];
-        if (c + kRing + i < nch) w.ring[i] = p[(c + kRing + i) * 64];
-        uint32_t e[4];
-        lookup4(tab, cw, shift2, e);
-        const int j = kChunk * (c + i);
-#pragma unroll
-        for (int q = 0; q < 4; q++)
-          add_codeword(j + q < len ? e[q] : kIdleWord, xa, colw, s1, s2, dk);
-      }
+  for (; c < w.nch; c += kRing) {
+    run_chunks<true>(w, c, shift2, tab, xa, colw, p1, p2, dk);
+    if ((c + kRing) % kGroupChunks == 0) {
+      s1 += p1;
+      s2 += p2;
+      p1 = 0.f;
+      p2 = 0.f;
     }
   }
+  s1 += p1;   // the last, partial group (+0 if it was just folded)
+  s2 += p2;
 }
 
 // Persistent grid.  A tile is (token, projection, part): the slices of one
