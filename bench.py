@@ -174,9 +174,11 @@ def main():
     tick = time.perf_counter()
     prep = stack.prepare()
     torch.cuda.synchronize()
-    print('prepared in %.2f s: %.3f GB of interleaved codes (%.3f x the packed stream)' %
-          (time.perf_counter() - tick, prep.code_bytes / 1e9,
-           prep.code_bytes / (2.0 * stack.w_comp.numel())), file=sys.stderr)
+    print('prepared in %.2f s: %.3f GB of interleaved codes (%.3f x the packed stream) + %.3f GB '
+          'of column checkpoints' %
+          (time.perf_counter() - tick, prep.stream_bytes / 1e9,
+           prep.stream_bytes / (2.0 * stack.w_comp.numel()),
+           (prep.code_bytes - prep.stream_bytes) / 1e9), file=sys.stderr)
 
     x = synthetic.activations(experts, d_model, args.seed + 1)
     route = torch.arange(experts, dtype=torch.int32, device='cuda')

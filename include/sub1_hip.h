@@ -174,16 +174,18 @@ int sub1_moe_grouped(const sub1_moe_stack *stack, const int32_t *token_expert,
  * compared with it, once) and 1 <= d_model, d_ff <= SUB1_PREPARED_MAX_WIDTH.
  *
  *   meta_bytes = sub1_moe_prepared_meta_bytes(experts, d_model, d_ff);
- *   sub1_moe_prepare_layout(stack, meta, meta_bytes, &code_bytes, stream);   // synchronises
- *   sub1_moe_prepare_codes(stack, meta, codes, code_bytes, stream);
- *   sub1_moe_prepared p = {meta, codes, meta_bytes, code_bytes, experts, d_model, d_ff};
+ *   sub1_moe_prepared p;
+ *   sub1_moe_prepare_layout(stack, meta, meta_bytes, &p, stream);   // synchronises; sets p.code_bytes
+ *   p.codes = <device buffer of p.code_bytes bytes>;
+ *   sub1_moe_prepare_codes(stack, &p, stream);
  *   sub1_moe_grouped_prepared(&p, token_expert, x, y, tokens, workspace, bytes, stream);
  *
  * meta and codes are device buffers the caller owns, 256-byte aligned; the
  * original stack is not referenced after sub1_moe_prepare_codes has run.
  * sub1_moe_grouped_prepared has the semantics of sub1_moe_grouped and the same
  * workspace; every row's sums are taken in the same order, so outputs are
- * identical.
+ * identical.  With few tokens several wavefronts share a row slice (the code
+ * buffer carries column checkpoints for that); the results do not change.
  */
 #define SUB1_PREPARED_MAX_WIDTH 8192
 
@@ -192,18 +194,20 @@ typedef struct sub1_moe_prepared {
   const void *codes;
   int64_t meta_bytes;
   int64_t code_bytes;
+  int64_t total_chunks;    /* 512-byte chunk rows of the code stream; checkpoints follow */
   int32_t experts;
   int32_t d_model;
   int32_t d_ff;
+  int32_t max_chunks[2];   /* longest 64-row slice of wi, wo in chunks */
 } sub1_moe_prepared;
 
 int64_t sub1_moe_prepared_meta_bytes(int experts, int d_model, int d_ff);
 
 int sub1_moe_prepare_layout(const sub1_moe_stack *stack, void *meta, int64_t meta_bytes,
-                            int64_t *code_bytes, void *stream);
+                            sub1_moe_prepared *prepared, void *stream);
 
-int sub1_moe_prepare_codes(const sub1_moe_stack *stack, const void *meta, void *codes,
-                           int64_t code_bytes, void *stream);
+int sub1_moe_prepare_codes(const sub1_moe_stack *stack, const sub1_moe_prepared *prepared,
+                           void *stream);
 
 int sub1_moe_grouped_prepared(const sub1_moe_prepared *prepared, const int32_t *token_expert,
                               const void *x, void *y, int tokens, void *workspace,

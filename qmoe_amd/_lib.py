@@ -28,8 +28,9 @@ class MoeStack(ctypes.Structure):
 class MoePrepared(ctypes.Structure):
     """struct sub1_moe_prepared"""
     _fields_ = [('meta', _vp), ('codes', _vp), ('meta_bytes', _i64), ('code_bytes', _i64),
-                ('experts', ctypes.c_int32), ('d_model', ctypes.c_int32),
-                ('d_ff', ctypes.c_int32)]
+                ('total_chunks', _i64), ('experts', ctypes.c_int32),
+                ('d_model', ctypes.c_int32), ('d_ff', ctypes.c_int32),
+                ('max_chunks', ctypes.c_int32 * 2)]
 
 
 # every symbol include/sub1_hip.h declares, with its prototype
@@ -48,8 +49,9 @@ PROTOTYPES = {
                                 _i64, _vp]),
     'sub1_moe_prepared_meta_bytes': (_i64, [_int, _int, _int]),
     'sub1_moe_prepare_layout': (_int, [ctypes.POINTER(MoeStack), _vp, _i64,
-                                       ctypes.POINTER(_i64), _vp]),
-    'sub1_moe_prepare_codes': (_int, [ctypes.POINTER(MoeStack), _vp, _vp, _i64, _vp]),
+                                       ctypes.POINTER(MoePrepared), _vp]),
+    'sub1_moe_prepare_codes': (_int, [ctypes.POINTER(MoeStack), ctypes.POINTER(MoePrepared),
+                                      _vp]),
     'sub1_moe_grouped_prepared': (_int, [ctypes.POINTER(MoePrepared), _vp, _vp, _vp, _int,
                                          _vp, _i64, _vp]),
     'sub1_timing_begin': (_int, [_vp]),

@@ -63,7 +63,8 @@ struct KindMeta {
 struct MetaLayout {
   KindMeta k[2];
   int64_t counts;       // i32 [E*S0 + E*S1 + 1] chunk counts, scanned in place
-  int64_t status;       // i32 [4]: [0] rows with a bad code count
+  int64_t status;       // i32 [4]: [0] rows with a bad code count, [1], [2] longest slice
+                        // of wi / wo in chunks
   int64_t bytes;
 };
 
@@ -111,7 +112,7 @@ __global__ __launch_bounds__(256) void order_rows_kernel(
     uint16_t *__restrict__ row_len, uint16_t *__restrict__ row_idx,
     uint32_t *__restrict__ minmax_sorted, uint16_t *__restrict__ slice_nch,
     uint16_t *__restrict__ slice_nfull, int32_t *__restrict__ counts,
-    int32_t *__restrict__ status, int height, int width, int slices) {
+    int32_t *__restrict__ status, int height, int width, int slices, int kind) {
   __shared__ int hist[kMaxLen + 2];
   const int e = blockIdx.x;
   const int32_t *ro = row_off_all + static_cast<int64_t>(e) * (height + 1);
@@ -160,6 +161,7 @@ __global__ __launch_bounds__(256) void order_rows_kernel(
     slice_nch[g] = static_cast<uint16_t>(nch);
     slice_nfull[g] = static_cast<uint16_t>(nfull);
     counts[g + 1] = nch;
+    atomicMax(&status[1 + kind], nch);
   }
 }
 
@@ -219,6 +221,39 @@ __global__ __launch_bounds__(256) void interleave_codes_kernel(
   }
 }
 
+// Column checkpoints.  For every slice and every group of kGroupChunks chunks,
+// the column offset (in dwords of the LDS activation array, 6 per column pair)
+// at which each lane's row stands when the group begins: 64 x u16 per group,
+// groups of slice g stored from entry slice_base[g]/kGroupChunks + g on.  With
+// them a wavefront can start in the middle of a slice, which is how a small
+// batch is spread over the GPU.  One wavefront per slice walks its codes.
+__device__ __forceinline__ int64_t checkpoint_entry(uint32_t slice_base, int64_t slice) {
+  return static_cast<int64_t>(slice_base / kGroupChunks) + slice;
+}
+
+__global__ __launch_bounds__(256) void checkpoint_kernel(
+    const uint16_t *__restrict__ codes, const uint32_t *__restrict__ table,
+    const uint32_t *__restrict__ slice_base, const uint16_t *__restrict__ slice_nch,
+    uint16_t *__restrict__ ckpt, int64_t first_slice, int64_t nslices, int group_shift) {
+  const int64_t sl = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / 64;
+  if (sl >= nslices) return;
+  const int lane = threadIdx.x & 63;
+  const int nch = slice_nch[sl];
+  const uint2 *p = reinterpret_cast<const uint2 *>(codes + static_cast<int64_t>(slice_base[sl]) * 256) + lane;
+  uint16_t *out = ckpt + checkpoint_entry(slice_base[sl], first_slice + sl) * 64 + lane;
+  uint32_t colw = 0;
+  for (int c = 0; c < nch; c++) {
+    if (c % kGroupChunks == 0) out[(c / kGroupChunks) * 64] = static_cast<uint16_t>(colw);
+    const uint2 w = p[c * 64];
+    const uint32_t cs[4] = {w.x & 0xffffu, w.x >> 16, w.y & 0xffffu, w.y >> 16};
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      uint32_t idx = min(cs[q], (cs[q] >> 3) + static_cast<uint32_t>(group_shift));
+      colw += table[idx] >> 24;
+    }
+  }
+}
+
 __global__ void zero_words_kernel(int32_t *p, int n) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0;
@@ -234,11 +269,15 @@ struct KindArgs {
   const uint16_t *row_idx;
   const uint32_t *minmax;
   int slices, height, width, parts;
+  int split;            // wavefronts that share one slice (1 = a slice per wavefront)
+  int groups_max;       // most 32-code groups in a slice of this kind
+  int64_t first_slice;  // global index of the kind's first slice (checkpoint addressing)
 };
 
 struct PreparedArgs {
   const uint32_t *table;      // kernel decode table (global copy, staged into LDS)
   const uint16_t *codes;
+  const uint16_t *ckpt;       // column checkpoints, behind the code stream
   KindArgs k[2];
   const int32_t *token_expert;
   const uint16_t *x;
@@ -413,6 +452,80 @@ __device__ __forceinline__ void run_slice(SliceWalk &w, int group_shift, const u
   s2 += p2;
 }
 
+// Small-batch form of a tile: `split` wavefronts share each slice, every one
+// taking a run of the slice's 32-code groups (it starts from the column
+// checkpoint of its first group) and leaving one partial-sum pair per group in
+// LDS; after a barrier the slice's first wavefront adds the groups in order,
+// which is the canonical order, so the result is the same to the bit as with a
+// wavefront per slice.
+__device__ __forceinline__ void split_tile(const PreparedArgs &a, const KindArgs &k, int e,
+                                           int s_lo, int s_hi, const uint32_t *tab,
+                                           const uint32_t *xa, uint16_t *dst, bool relu) {
+  float2 *part = reinterpret_cast<float2 *>(const_cast<uint32_t *>(xa) + a.xdwords);
+  const int waves = blockDim.x >> 6;
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int per_pass = waves / k.split;      // slices a pass of the workgroup covers
+  const int sub = wave % k.split;
+  const int local = wave / k.split;
+  const DotConsts dk = dot_consts();
+  const uint32_t shift2 = static_cast<uint32_t>(a.group_shift) * 0x00010001u;
+  for (int s0 = s_lo; s0 < s_hi; s0 += per_pass) {
+    const int s = s0 + local;
+    const bool mine = s < s_hi && local < per_pass;
+    const int64_t sl = static_cast<int64_t>(e) * k.slices + s;
+    int ngroups = 0;
+    if (mine) {
+      const int nch_all = __builtin_amdgcn_readfirstlane(k.slice_nch[sl]);
+      ngroups = (nch_all + kGroupChunks - 1) / kGroupChunks;
+      const int g_lo = sub * ngroups / k.split;
+      const int g_hi = (sub + 1) * ngroups / k.split;
+      if (g_lo < g_hi) {
+        SliceWalk w;
+        const uint32_t base = k.slice_base[sl];
+        w.nfull = __builtin_amdgcn_readfirstlane(k.slice_nfull[sl]);
+        w.len = k.row_len[sl * 64 + lane];
+        w.p = reinterpret_cast<const uint2 *>(a.codes + static_cast<int64_t>(base) * 256) + lane;
+        const int c_lo = g_lo * kGroupChunks;
+        w.nch = min(g_hi * kGroupChunks, nch_all);   // this wavefront's last chunk + 1
+        int colw = 0;
+        if (g_lo)
+          colw = a.ckpt[(checkpoint_entry(base, k.first_slice + sl) + g_lo) * 64 + lane];
+#pragma unroll
+        for (int i = 0; i < kRing; i++)
+          if (c_lo + i < w.nch) w.ring[i] = w.p[(c_lo + i) * 64];
+        for (int g = g_lo; g < g_hi; g++) {
+          float p1 = 0.f, p2 = 0.f;
+          const int c_end = min((g + 1) * kGroupChunks, w.nch);
+          for (int c = g * kGroupChunks; c < c_end; c += kRing) {
+            if (c + kRing <= w.nfull)
+              run_chunks<false>(w, c, shift2, tab, xa, colw, p1, p2, dk);
+            else
+              run_chunks<true>(w, c, shift2, tab, xa, colw, p1, p2, dk);
+          }
+          part[(local * k.groups_max + g) * 64 + lane] = make_float2(p1, p2);
+        }
+      }
+    }
+    __syncthreads();
+    if (mine && sub == 0) {
+      float s1 = 0.f, s2 = 0.f;
+      for (int g = 0; g < ngroups; g++) {
+        float2 v = part[(local * k.groups_max + g) * 64 + lane];
+        s1 += v.x;
+        s2 += v.y;
+      }
+      const int ridx = k.row_idx[sl * 64 + lane];
+      if (ridx != 0xffff) {
+        uint16_t out = f32_to_bf16(row_result(k.minmax[sl * 64 + lane], s1, s2));
+        if (relu && (out & 0x8000u)) out = 0;
+        dst[ridx] = out;
+      }
+    }
+    __syncthreads();
+  }
+}
+
 // Persistent grid.  A tile is (token, projection, part): the slices of one
 // matrix, or of one of `parts` equal ranges of them when there are too few
 // tokens to occupy the GPU otherwise; a workgroup stages the token's
@@ -478,7 +591,8 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
       // the first slice's loads go out before the wait and the staging
       int s = s_lo + wave;
       SliceWalk cur;
-      if (s < s_hi) cur = load_slice(a, k, static_cast<int64_t>(e) * k.slices + s);
+      if (k.split == 1 && s < s_hi)
+        cur = load_slice(a, k, static_cast<int64_t>(e) * k.slices + s);
       if (kind == 1) {
         if (threadIdx.x == 0) {
           int spins = 0;
@@ -498,6 +612,10 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
       stage_activations(xa, src + static_cast<int64_t>(t) * k.width, k.width);
       __syncthreads();
       uint16_t *dst = (kind ? a.y : a.h) + static_cast<int64_t>(t) * k.height;
+      if (k.split > 1) {
+        split_tile(a, k, e, s_lo, s_hi, tab, xa, dst, kind == 0);
+        s = s_hi;
+      }
       for (; s < s_hi; s += waves) {
         const bool more = s + waves < s_hi;
         SliceWalk nxt;
@@ -615,10 +733,10 @@ extern "C" int64_t sub1_moe_prepared_meta_bytes(int experts, int d_model, int d_
 }
 
 extern "C" int sub1_moe_prepare_layout(const sub1_moe_stack *st, void *meta, int64_t meta_bytes,
-                                       int64_t *code_bytes, void *stream) {
+                                       sub1_moe_prepared *out, void *stream) {
   int rc = check_stack(st, "sub1_moe_prepare_layout");
   if (rc) return rc;
-  if (!meta || !code_bytes) return fail(SUB1_ERR_NULL, "sub1_moe_prepare_layout: NULL argument");
+  if (!meta || !out) return fail(SUB1_ERR_NULL, "sub1_moe_prepare_layout: NULL argument");
   if (misaligned(meta, 256)) return fail(SUB1_ERR_ALIGN, "sub1_moe_prepare_layout: meta must be 256-byte aligned");
   const MetaLayout m = meta_layout(st->experts, st->d_model, st->d_ff);
   if (meta_bytes < m.bytes)
@@ -643,56 +761,75 @@ extern "C" int sub1_moe_prepare_layout(const sub1_moe_stack *st, void *meta, int
         reinterpret_cast<uint32_t *>(base + k.minmax),
         reinterpret_cast<uint16_t *>(base + k.slice_nch),
         reinterpret_cast<uint16_t *>(base + k.slice_nfull), counts + slice0, status, k.height,
-        k.width, k.slices);
+        k.width, k.slices, i);
     slice0 += static_cast<int64_t>(st->experts) * k.slices;
   }
   scan_counts_kernel<<<1, 1024, 0, s>>>(counts, static_cast<int>(slice0));
   HIP_TRY(hipGetLastError());
-  int32_t host[2] = {0, 0};
-  HIP_TRY(hipMemcpyAsync(&host[0], status, 4, hipMemcpyDeviceToHost, s));
-  HIP_TRY(hipMemcpyAsync(&host[1], counts + slice0, 4, hipMemcpyDeviceToHost, s));
+  int32_t host[4] = {0, 0, 0, 0};
+  int32_t total = 0;
+  HIP_TRY(hipMemcpyAsync(host, status, sizeof host, hipMemcpyDeviceToHost, s));
+  HIP_TRY(hipMemcpyAsync(&total, counts + slice0, 4, hipMemcpyDeviceToHost, s));
   HIP_TRY(hipStreamSynchronize(s));
   if (host[0])
     return fail(SUB1_ERR_SHAPE,
                 "sub1_moe_prepare_layout: %d rows have a code count outside 1..width/2", host[0]);
-  if (host[1] < 0) return fail(SUB1_ERR_SHAPE, "sub1_moe_prepare_layout: stream too large");
-  *code_bytes = static_cast<int64_t>(host[1]) * 512;
+  if (total < 0) return fail(SUB1_ERR_SHAPE, "sub1_moe_prepare_layout: stream too large");
+  out->meta = meta;
+  out->codes = nullptr;
+  out->meta_bytes = m.bytes;
+  out->total_chunks = total;
+  // the code stream, then one 128-byte checkpoint entry per group of chunks
+  out->code_bytes = static_cast<int64_t>(total) * 512 +
+                    (static_cast<int64_t>(total) / kGroupChunks + slice0 + 1) * 128;
+  out->experts = st->experts;
+  out->d_model = st->d_model;
+  out->d_ff = st->d_ff;
+  out->max_chunks[0] = host[1];
+  out->max_chunks[1] = host[2];
   return SUB1_OK;
 }
 
-extern "C" int sub1_moe_prepare_codes(const sub1_moe_stack *st, const void *meta, void *codes,
-                                      int64_t code_bytes, void *stream) {
+extern "C" int sub1_moe_prepare_codes(const sub1_moe_stack *st, const sub1_moe_prepared *p,
+                                      void *stream) {
   int rc = check_stack(st, "sub1_moe_prepare_codes");
   if (rc) return rc;
-  if (!meta || !codes) return fail(SUB1_ERR_NULL, "sub1_moe_prepare_codes: NULL argument");
-  if (misaligned(meta, 256) || misaligned(codes, 256))
+  if (!p || !p->meta || !p->codes)
+    return fail(SUB1_ERR_NULL, "sub1_moe_prepare_codes: NULL argument");
+  if (misaligned(p->meta, 256) || misaligned(p->codes, 256))
     return fail(SUB1_ERR_ALIGN, "sub1_moe_prepare_codes: buffers must be 256-byte aligned");
+  if (p->experts != st->experts || p->d_model != st->d_model || p->d_ff != st->d_ff)
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_prepare_codes: the layout belongs to another stack");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const DeviceTables *t = nullptr;
   rc = device_tables(s, &t);
   if (rc) return rc;
   const MetaLayout m = meta_layout(st->experts, st->d_model, st->d_ff);
-  const char *base = static_cast<const char *>(meta);
-  // the layout pass left the total in the last count; make sure the buffer holds it
-  int64_t nslices = static_cast<int64_t>(st->experts) * (m.k[0].slices + m.k[1].slices);
-  int32_t total = 0;
-  HIP_TRY(hipMemcpyAsync(&total, reinterpret_cast<const int32_t *>(base + m.counts) + nslices, 4,
-                         hipMemcpyDeviceToHost, s));
-  HIP_TRY(hipStreamSynchronize(s));
-  if (code_bytes < static_cast<int64_t>(total) * 512)
-    return fail(SUB1_ERR_SHAPE, "sub1_moe_prepare_codes: code buffer needs %lld bytes",
-                static_cast<long long>(total) * 512);
+  const char *base = static_cast<const char *>(p->meta);
+  const int64_t nslices = static_cast<int64_t>(st->experts) * (m.k[0].slices + m.k[1].slices);
+  if (p->total_chunks < 0 ||
+      p->code_bytes < p->total_chunks * 512 + (p->total_chunks / kGroupChunks + nslices + 1) * 128)
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_prepare_codes: code buffer smaller than the layout needs");
+  uint16_t *codes = static_cast<uint16_t *>(const_cast<void *>(p->codes));
+  uint16_t *ckpt = codes + p->total_chunks * 256;
   const int64_t *code_base[2] = {st->wi_code_base, st->wo_code_base};
   const int32_t *row_off[2] = {st->wi_row_off, st->wo_row_off};
+  const int group_shift = t->single_codes - t->single_codes / 8;
+  int64_t first_slice = 0;
   for (int i = 0; i < 2; i++) {
     const KindMeta &k = m.k[i];
-    int64_t lanes = static_cast<int64_t>(st->experts) * k.slices * 64;
+    const int64_t kslices = static_cast<int64_t>(st->experts) * k.slices;
+    const int64_t lanes = kslices * 64;
     interleave_codes_kernel<<<static_cast<unsigned>((lanes + 3) / 4), 256, 0, s>>>(
         reinterpret_cast<const uint16_t *>(st->w_comp), code_base[i], row_off[i], t->recode,
         reinterpret_cast<const uint32_t *>(base + k.slice_base),
         reinterpret_cast<const uint16_t *>(base + k.slice_nch),
-        reinterpret_cast<const uint16_t *>(base + k.row_idx), static_cast<uint16_t *>(codes),
-        k.height, k.slices, lanes);
+        reinterpret_cast<const uint16_t *>(base + k.row_idx), codes, k.height, k.slices, lanes);
+    checkpoint_kernel<<<static_cast<unsigned>((kslices + 3) / 4), 256, 0, s>>>(
+        codes, t->table, reinterpret_cast<const uint32_t *>(base + k.slice_base),
+        reinterpret_cast<const uint16_t *>(base + k.slice_nch), ckpt, first_slice, kslices,
+        group_shift);
+    first_slice += kslices;
   }
   HIP_TRY(hipGetLastError());
   return SUB1_OK;
@@ -748,14 +885,7 @@ extern "C" int sub1_moe_grouped_prepared(const sub1_moe_prepared *p, const int32
   int device = 0, cus = 0;
   HIP_TRY(hipGetDevice(&device));
   HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
-  // Whole matrices per tile when the tokens alone give every compute unit two
-  // tiles; otherwise each matrix is cut into parts, down to one slice per
-  // wavefront.
-  for (int i = 0; i < 2; i++) {
-    int max_parts = (a.k[i].slices + waves - 1) / waves;
-    int want = (2 * cus + 2 * tokens - 1) / (2 * tokens);
-    a.k[i].parts = want < 1 ? 1 : (want > max_parts ? max_parts : want);
-  }
+  a.ckpt = a.codes + p->total_chunks * 256;
   a.token_expert = token_expert;
   a.x = static_cast<const uint16_t *>(x);
   a.y = static_cast<uint16_t *>(y);
@@ -767,16 +897,48 @@ extern "C" int sub1_moe_grouped_prepared(const sub1_moe_prepared *p, const int32
   a.table_words = t->words;
   a.single_codes = t->single_codes;
   a.group_shift = t->single_codes - t->single_codes / 8;
-  int wmax = p->d_model > p->d_ff ? p->d_model : p->d_ff;
+  const int wmax = p->d_model > p->d_ff ? p->d_model : p->d_ff;
   a.xdwords = activation_dwords(wmax);
   a.spin_limit = 1 << 24;
+  const size_t lds_limit = 160 * 1024 - 64;
+  const size_t lds_base = (static_cast<size_t>(a.table_words) + a.xdwords) * 4;
+  if (lds_base > lds_limit)
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: width %d does not fit LDS", wmax);
+  // Tiles.  Whole matrices when the tokens alone keep every compute unit busy;
+  // otherwise each matrix is cut into parts, down to one slice per wavefront;
+  // and when even that leaves compute units idle (a handful of tokens), several
+  // wavefronts share a slice, each starting from a column checkpoint.
+  const int want = (cus + tokens - 1) / tokens;   // tiles per token and projection
+  size_t lds_partials = 0;
+  int64_t first_slice = 0;
+  for (int i = 0; i < 2; i++) {
+    KindArgs &k = a.k[i];
+    k.first_slice = first_slice;
+    first_slice += static_cast<int64_t>(p->experts) * k.slices;
+    k.groups_max = (p->max_chunks[i] + kGroupChunks - 1) / kGroupChunks;
+    k.split = 1;
+    const int max_parts = (k.slices + waves - 1) / waves;
+    k.parts = want > max_parts ? max_parts : want;
+    if (want > max_parts) {
+      int split = 1;
+      while (split * 2 <= waves && split * 2 <= k.groups_max &&
+             (k.slices + waves / split - 1) / (waves / split) < want)
+        split *= 2;
+      while (split > 1 &&
+             lds_base + static_cast<size_t>(waves / split) * k.groups_max * 512 > lds_limit)
+        split /= 2;
+      if (split > 1) {
+        k.split = split;
+        k.parts = (k.slices + waves / split - 1) / (waves / split);
+        size_t need = static_cast<size_t>(waves / split) * k.groups_max * 512;
+        if (need > lds_partials) lds_partials = need;
+      }
+    }
+  }
   int64_t tiles = static_cast<int64_t>(tokens) * (a.k[0].parts + a.k[1].parts);
   if (tiles > INT32_MAX - (1 << 20))
     return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: too many tiles");
-
-  size_t lds = (static_cast<size_t>(a.table_words) + a.xdwords) * 4;
-  if (lds > 160 * 1024 - 64)
-    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: width %d does not fit LDS", wmax);
+  const size_t lds = lds_base + lds_partials;
   HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(moe_prepared_kernel),
                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
   int64_t grid = cus;  // one workgroup per compute unit (LDS holds the table once)

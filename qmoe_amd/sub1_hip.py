@@ -233,17 +233,16 @@ class PreparedStack:
         if meta_bytes <= 0:
             raise ValueError('bad stack dimensions')
         self.meta = torch.empty(meta_bytes, dtype=torch.uint8, device=dev)
-        code_bytes = ctypes.c_int64()
+        self._c = _lib.MoePrepared()
         with torch.cuda.device(dev):
             _lib.check(lib.sub1_moe_prepare_layout(ctypes.byref(stack._c), self.meta.data_ptr(),
-                                                   meta_bytes, ctypes.byref(code_bytes), _stream()))
-            self.codes = torch.empty(max(code_bytes.value, 256), dtype=torch.uint8, device=dev)
-            _lib.check(lib.sub1_moe_prepare_codes(ctypes.byref(stack._c), self.meta.data_ptr(),
-                                                  self.codes.data_ptr(), code_bytes.value,
+                                                   meta_bytes, ctypes.byref(self._c), _stream()))
+            self.code_bytes = self._c.code_bytes
+            self.stream_bytes = self._c.total_chunks * 512     # without the checkpoints
+            self.codes = torch.empty(max(self.code_bytes, 256), dtype=torch.uint8, device=dev)
+            self._c.codes = self.codes.data_ptr()
+            _lib.check(lib.sub1_moe_prepare_codes(ctypes.byref(stack._c), ctypes.byref(self._c),
                                                   _stream()))
-        self.code_bytes = code_bytes.value
-        self._c = _lib.MoePrepared(self.meta.data_ptr(), self.codes.data_ptr(), meta_bytes,
-                                   code_bytes.value, stack.experts, stack.d_model, stack.d_ff)
         self._ws = None
 
     def workspace(self, tokens):

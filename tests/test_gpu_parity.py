@@ -370,3 +370,33 @@ def test_routed_batch_equals_per_token_products(gpu):
         out = torch.zeros(d_model, dtype=torch.bfloat16, device='cuda')
         sub1_hip.sub1matvec(dec, wo[0], wo[1], wo[2], h, out)
         assert torch.equal(out, y[t]), t
+
+
+def test_every_tiling_mode_gives_the_same_bits(gpu, oracle):
+    """The prepared kernel tiles differently with the batch size: whole
+    matrices per workgroup (many tokens), parts of a matrix (fewer), several
+    wavefronts sharing one row slice from column checkpoints (a handful).
+    The same token must come out identical in all of them, and equal to the
+    oracle."""
+    from qmoe_amd import synthetic
+    experts, d_model, d_ff = 3, 2080, 6144
+    stack = synthetic.build_stack(experts, d_model, d_ff, 0.9, seed=11)
+    prep = stack.prepare()
+    x1 = synthetic.activations(1, d_model, seed=12)
+    want = None
+    for tokens in (1, 2, 5, 40, 300, 700):
+        x = x1.repeat(tokens, 1).contiguous()
+        route = torch.full((tokens,), 2, dtype=torch.int32, device='cuda')
+        route[0] = 1
+        y = prep.forward(x, route)
+        assert prep.launch_faults(tokens) == (0, 0)
+        if want is None:
+            want = y[0].clone()
+            wi, wo = synthetic.expert_layers(stack, 1)
+            host = [tuple(bits_host(t) if t.dtype != torch.int32 else t.cpu().numpy() for t in l)
+                    for l in (wi, wo)]
+            ref, _ = oracle.expert_ffn(host[0], host[1], bits_host(x1[0]), order=1)
+            assert np.array_equal(bits_host(want), ref)
+        assert torch.equal(y[0], want), tokens
+        if tokens > 1:
+            assert torch.equal(y[1], y[tokens - 1])
