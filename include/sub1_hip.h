@@ -214,6 +214,55 @@ int sub1_moe_grouped_prepared(const sub1_moe_prepared *prepared, const int32_t *
                               int64_t workspace_bytes, void *stream);
 
 /*
+ * The same preparation for plain products: `count` matrices of one shape
+ * (count = 1: one Sub1Linear), then
+ *     y[t, :] += W_m x[t, :],   m = token_matrix[t]  (NULL: matrix 0 for all),
+ * the semantics of sub1_matvec_tokens, in one launch without a workspace.
+ * Tokens whose matrix index is negative or >= count are left alone.
+ *
+ *   meta_bytes = sub1_matrix_prepared_meta_bytes(count, height, width);
+ *   sub1_matrix_prepared p;
+ *   sub1_matrix_prepare_layout(&set, meta, meta_bytes, &p, stream);   // synchronises
+ *   p.codes = <device buffer of p.code_bytes bytes>;
+ *   sub1_matrix_prepare_codes(&set, &p, stream);
+ *   sub1_matvec_prepared(&p, NULL, x, ldx, y, ldy, tokens, stream);
+ */
+typedef struct sub1_matrix_set {
+  const int32_t *dec;
+  const int16_t *w_comp;       /* all streams in one buffer */
+  const int64_t *code_base;    /* int64 [count] first codeword of each matrix; NULL if count == 1 */
+  const int32_t *row_off;      /* int32 [count, height+1], each row starts at 0 */
+  const void *ter_minmax;      /* bf16  [count, 2*height] */
+  int32_t count;
+  int32_t height;
+  int32_t width;
+} sub1_matrix_set;
+
+typedef struct sub1_matrix_prepared {
+  const void *meta;
+  const void *codes;
+  int64_t meta_bytes;
+  int64_t code_bytes;
+  int64_t total_chunks;
+  int32_t count;
+  int32_t height;
+  int32_t width;
+  int32_t max_chunks;
+} sub1_matrix_prepared;
+
+int64_t sub1_matrix_prepared_meta_bytes(int count, int height, int width);
+
+int sub1_matrix_prepare_layout(const sub1_matrix_set *set, void *meta, int64_t meta_bytes,
+                               sub1_matrix_prepared *prepared, void *stream);
+
+int sub1_matrix_prepare_codes(const sub1_matrix_set *set, const sub1_matrix_prepared *prepared,
+                              void *stream);
+
+int sub1_matvec_prepared(const sub1_matrix_prepared *prepared, const int32_t *token_matrix,
+                         const void *x, int64_t ldx, void *y, int64_t ldy, int tokens,
+                         void *stream);
+
+/*
  * Average duration in microseconds of the most recent launches, measured with
  * HIP events on the launch stream: call sub1_timing_begin(stream) before and
  * sub1_timing_end(stream, &us) after a run of launches (end synchronises).

@@ -33,6 +33,20 @@ class MoePrepared(ctypes.Structure):
                 ('max_chunks', ctypes.c_int32 * 2)]
 
 
+class MatrixSet(ctypes.Structure):
+    """struct sub1_matrix_set"""
+    _fields_ = [('dec', _vp), ('w_comp', _vp), ('code_base', _vp), ('row_off', _vp),
+                ('ter_minmax', _vp), ('count', ctypes.c_int32), ('height', ctypes.c_int32),
+                ('width', ctypes.c_int32)]
+
+
+class MatrixPrepared(ctypes.Structure):
+    """struct sub1_matrix_prepared"""
+    _fields_ = [('meta', _vp), ('codes', _vp), ('meta_bytes', _i64), ('code_bytes', _i64),
+                ('total_chunks', _i64), ('count', ctypes.c_int32), ('height', ctypes.c_int32),
+                ('width', ctypes.c_int32), ('max_chunks', ctypes.c_int32)]
+
+
 # every symbol include/sub1_hip.h declares, with its prototype
 PROTOTYPES = {
     'sub1_last_error': (ctypes.c_char_p, []),
@@ -54,6 +68,13 @@ PROTOTYPES = {
                                       _vp]),
     'sub1_moe_grouped_prepared': (_int, [ctypes.POINTER(MoePrepared), _vp, _vp, _vp, _int,
                                          _vp, _i64, _vp]),
+    'sub1_matrix_prepared_meta_bytes': (_i64, [_int, _int, _int]),
+    'sub1_matrix_prepare_layout': (_int, [ctypes.POINTER(MatrixSet), _vp, _i64,
+                                          ctypes.POINTER(MatrixPrepared), _vp]),
+    'sub1_matrix_prepare_codes': (_int, [ctypes.POINTER(MatrixSet),
+                                         ctypes.POINTER(MatrixPrepared), _vp]),
+    'sub1_matvec_prepared': (_int, [ctypes.POINTER(MatrixPrepared), _vp, _vp, _i64, _vp, _i64,
+                                    _int, _vp]),
     'sub1_timing_begin': (_int, [_vp]),
     'sub1_timing_end': (_int, [_vp, ctypes.POINTER(ctypes.c_double)]),
 }

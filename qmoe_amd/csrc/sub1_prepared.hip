@@ -50,7 +50,7 @@ constexpr uint32_t kIdleWord = 0x00040404u;  // three empty slots, no advance
 // One block of device memory, arrays back to back, each 256-byte aligned.
 // Kind 0 = wi (rows d_ff, width d_model), kind 1 = wo.
 struct KindMeta {
-  int64_t slice_base;   // u32 [E*S + 1]   (only kind 0 holds the shared array)
+  int64_t slice_base;   // u32 [E*S] (+1): this kind's part of the scanned counts
   int64_t slice_nch;    // u16 [E*S]
   int64_t slice_nfull;  // u16 [E*S]
   int64_t row_len;      // u16 [E*S*64]
@@ -62,32 +62,36 @@ struct KindMeta {
 
 struct MetaLayout {
   KindMeta k[2];
-  int64_t counts;       // i32 [E*S0 + E*S1 + 1] chunk counts, scanned in place
+  int kinds;
+  int64_t counts;       // i32 [all slices + 1] chunk counts, scanned in place
   int64_t status;       // i32 [4]: [0] rows with a bad code count, [1], [2] longest slice
-                        // of wi / wo in chunks
+                        // of kind 0 / 1 in chunks
   int64_t bytes;
 };
 
 int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 
-MetaLayout meta_layout(int experts, int d_model, int d_ff) {
+// kinds = 2: an expert stack (kind 0 = wi, rows d_ff; kind 1 = wo);
+// kinds = 1: `experts` matrices of one shape.
+MetaLayout meta_layout(int experts, int kinds, const int height[2], const int width[2]) {
   MetaLayout m;
+  m.kinds = kinds;
   int64_t off = 0;
   auto take = [&](int64_t bytes) {
     int64_t o = off;
     off += align256(bytes);
     return o;
   };
-  const int h[2] = {d_ff, d_model}, w[2] = {d_model, d_ff};
   int64_t nslices = 0;
-  for (int i = 0; i < 2; i++) {
+  int64_t first[2] = {0, 0};
+  for (int i = 0; i < kinds; i++) {
     KindMeta &k = m.k[i];
-    k.height = h[i];
-    k.width = w[i];
-    k.slices = (h[i] + 63) / 64;
+    k.height = height[i];
+    k.width = width[i];
+    k.slices = (height[i] + 63) / 64;
     int64_t es = static_cast<int64_t>(experts) * k.slices;
+    first[i] = nslices;
     nslices += es;
-    k.slice_base = 0;  // set below
     k.slice_nch = take(es * 2);
     k.slice_nfull = take(es * 2);
     k.row_len = take(es * 64 * 2);
@@ -95,11 +99,20 @@ MetaLayout meta_layout(int experts, int d_model, int d_ff) {
     k.minmax = take(es * 64 * 4);
   }
   m.counts = take((nslices + 1) * 4);
-  m.k[0].slice_base = m.counts;
-  m.k[1].slice_base = m.counts + static_cast<int64_t>(experts) * m.k[0].slices * 4;
+  for (int i = 0; i < kinds; i++) m.k[i].slice_base = m.counts + first[i] * 4;
   m.status = take(16);
   m.bytes = off;
   return m;
+}
+
+MetaLayout moe_layout(int experts, int d_model, int d_ff) {
+  const int h[2] = {d_ff, d_model}, w[2] = {d_model, d_ff};
+  return meta_layout(experts, 2, h, w);
+}
+
+MetaLayout matrix_layout(int count, int height, int width) {
+  const int h[2] = {height, 0}, w[2] = {width, 0};
+  return meta_layout(count, 1, h, w);
 }
 
 // ---------------------------------------------------------- prepare kernels --
@@ -211,7 +224,7 @@ __global__ __launch_bounds__(256) void interleave_codes_kernel(
   const uint16_t *s = src;
   if (ridx != 0xffff) {
     const int32_t *ro = row_off_all + static_cast<int64_t>(e) * (height + 1);
-    s = src + code_base[e] + ro[ridx];
+    s = src + (code_base ? code_base[e] : 0) + ro[ridx];   // one matrix: no base array
     len = min(max(ro[ridx + 1] - ro[ridx], 0), padded);
   }
   for (int j = lane; j < padded; j += 64) {
@@ -279,11 +292,13 @@ struct PreparedArgs {
   const uint16_t *codes;
   const uint16_t *ckpt;       // column checkpoints, behind the code stream
   KindArgs k[2];
-  const int32_t *token_expert;
+  const int32_t *token_expert;   // NULL: every token uses matrix 0
   const uint16_t *x;
   uint16_t *y;
-  uint16_t *h;
-  int32_t *ctrl;
+  uint16_t *h;                   // kinds == 2 only
+  int32_t *ctrl;                 // NULL: no dependencies between tiles, static tile order
+  int64_t ldx, ldy;              // element strides between tokens of x and y
+  int kinds;                     // 2: y = wo(relu(wi x));  1: y += W x
   int tokens, experts;
   int table_words, single_codes, group_shift;  // group_shift = single_codes - single_codes/8
   int xdwords;                                 // LDS dwords reserved for the activations
@@ -452,6 +467,23 @@ __device__ __forceinline__ void run_slice(SliceWalk &w, int group_shift, const u
   s2 += p2;
 }
 
+// How a row's result leaves the kernel.
+enum OutMode { kStoreRelu = 0, kStore = 1, kAccumulate = 2 };
+
+__device__ __forceinline__ void write_row(uint16_t *dst, int ridx, uint32_t minmax, float s1,
+                                          float s2, int mode) {
+  if (ridx == 0xffff) return;   // padding lane
+  float res = row_result(minmax, s1, s2);
+  uint16_t out = f32_to_bf16(res);
+  if (mode == kStoreRelu) {
+    if (out & 0x8000u) out = 0;   // relu between the projections, on the bf16 value
+  } else if (mode == kAccumulate) {
+    // reference sub1_cuda_kernel.cu:200: y[row] += bf16(res), the sum in bf16
+    out = f32_to_bf16(bf16_to_f32(dst[ridx]) + bf16_to_f32(out));
+  }
+  dst[ridx] = out;
+}
+
 // Small-batch form of a tile: `split` wavefronts share each slice, every one
 // taking a run of the slice's 32-code groups (it starts from the column
 // checkpoint of its first group) and leaving one partial-sum pair per group in
@@ -460,7 +492,7 @@ __device__ __forceinline__ void run_slice(SliceWalk &w, int group_shift, const u
 // wavefront per slice.
 __device__ __forceinline__ void split_tile(const PreparedArgs &a, const KindArgs &k, int e,
                                            int s_lo, int s_hi, const uint32_t *tab,
-                                           const uint32_t *xa, uint16_t *dst, bool relu) {
+                                           const uint32_t *xa, uint16_t *dst, int mode) {
   float2 *part = reinterpret_cast<float2 *>(const_cast<uint32_t *>(xa) + a.xdwords);
   const int waves = blockDim.x >> 6;
   const int wave = threadIdx.x >> 6;
@@ -515,12 +547,7 @@ __device__ __forceinline__ void split_tile(const PreparedArgs &a, const KindArgs
         s1 += v.x;
         s2 += v.y;
       }
-      const int ridx = k.row_idx[sl * 64 + lane];
-      if (ridx != 0xffff) {
-        uint16_t out = f32_to_bf16(row_result(k.minmax[sl * 64 + lane], s1, s2));
-        if (relu && (out & 0x8000u)) out = 0;
-        dst[ridx] = out;
-      }
+      write_row(dst, k.row_idx[sl * 64 + lane], k.minmax[sl * 64 + lane], s1, s2, mode);
     }
     __syncthreads();
   }
@@ -546,23 +573,31 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
   const int waves = threads >> 6;
   for (int i = threadIdx.x; i < a.table_words; i += threads) tab[i] = a.table[i];
   const int n_wi = a.tokens * a.k[0].parts;
-  const int n_all = n_wi + a.tokens * a.k[1].parts;
+  const int n_all = n_wi + (a.kinds == 2 ? a.tokens * a.k[1].parts : 0);
   const int wave = threadIdx.x >> 6;
-  // thread 0 keeps one ticket ahead so that the atomic's round trip overlaps a tile
-  int next_ticket = 0;
-  if (threadIdx.x == 0)
+  const bool dynamic = a.ctrl != nullptr;
+  // dynamic order: thread 0 keeps one ticket ahead so that the atomic's round
+  // trip overlaps a tile; static order: tile = workgroup index + k * grid
+  int next_ticket = blockIdx.x;
+  if (dynamic && threadIdx.x == 0)
     next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
                                          __HIP_MEMORY_SCOPE_AGENT);
   for (;;) {
     __syncthreads();
-    if (threadIdx.x == 0) {
-      s_ticket = next_ticket;
-      if (next_ticket < n_all)
-        next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
-                                             __HIP_MEMORY_SCOPE_AGENT);
+    int ticket;
+    if (dynamic) {
+      if (threadIdx.x == 0) {
+        s_ticket = next_ticket;
+        if (next_ticket < n_all)
+          next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __syncthreads();
+      ticket = s_ticket;
+    } else {
+      ticket = next_ticket;
+      next_ticket += gridDim.x;
     }
-    __syncthreads();
-    const int ticket = s_ticket;
     if (ticket >= n_all) break;
     const int kind = ticket < n_wi ? 0 : 1;
     const KindArgs &k = a.k[kind];
@@ -572,19 +607,17 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
     // slices [s_lo, s_hi) of the matrix
     const int s_lo = static_cast<int>(static_cast<int64_t>(k.slices) * part / k.parts);
     const int s_hi = static_cast<int>(static_cast<int64_t>(k.slices) * (part + 1) / k.parts);
-    int e = a.token_expert[t];
+    int e = a.token_expert ? a.token_expert[t] : 0;
     if (e >= a.experts) {
-      if (kind == 1 && part == 0 && threadIdx.x == 0)
+      if (dynamic && kind == a.kinds - 1 && part == 0 && threadIdx.x == 0)
         __hip_atomic_fetch_add(&a.ctrl[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       e = -1;
     }
-    if (kind == 1 && e < 0) {
+    if (a.kinds == 2 && kind == 1 && e < 0) {
       // a dropped token keeps its input (reference sub1.py:312)
       const int r_lo = min(64 * s_lo, k.height), r_hi = min(64 * s_hi, k.height);
-      for (int i = r_lo + threadIdx.x; i < r_hi; i += threads) {
-        int64_t g = static_cast<int64_t>(t) * k.height + i;
-        a.y[g] = a.x[g];
-      }
+      for (int i = r_lo + threadIdx.x; i < r_hi; i += threads)
+        a.y[static_cast<int64_t>(t) * a.ldy + i] = a.x[static_cast<int64_t>(t) * a.ldx + i];
       continue;
     }
     if (e >= 0) {
@@ -608,12 +641,21 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
         }
         __syncthreads();  // thread 0's acquire now covers the whole workgroup
       }
-      const uint16_t *src = kind ? a.h : a.x;
-      stage_activations(xa, src + static_cast<int64_t>(t) * k.width, k.width);
+      const uint16_t *src = kind ? a.h + static_cast<int64_t>(t) * k.width
+                                 : a.x + static_cast<int64_t>(t) * a.ldx;
+      stage_activations(xa, src, k.width);
       __syncthreads();
-      uint16_t *dst = (kind ? a.y : a.h) + static_cast<int64_t>(t) * k.height;
+      uint16_t *dst;
+      int mode;
+      if (a.kinds == 2 && kind == 0) {
+        dst = a.h + static_cast<int64_t>(t) * k.height;
+        mode = kStoreRelu;
+      } else {
+        dst = a.y + static_cast<int64_t>(t) * a.ldy;
+        mode = a.kinds == 2 ? kStore : kAccumulate;
+      }
       if (k.split > 1) {
-        split_tile(a, k, e, s_lo, s_hi, tab, xa, dst, kind == 0);
+        split_tile(a, k, e, s_lo, s_hi, tab, xa, dst, mode);
         s = s_hi;
       }
       for (; s < s_hi; s += waves) {
@@ -622,15 +664,11 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
         if (more) nxt = load_slice(a, k, static_cast<int64_t>(e) * k.slices + s + waves);
         float s1, s2;
         run_slice(cur, a.group_shift, tab, xa, s1, s2);
-        if (cur.ridx != 0xffff) {
-          uint16_t out = f32_to_bf16(row_result(cur.minmax, s1, s2));
-          if (kind == 0 && (out & 0x8000u)) out = 0;  // relu between the projections
-          dst[cur.ridx] = out;
-        }
+        write_row(dst, cur.ridx, cur.minmax, s1, s2, mode);
         if (more) cur = nxt;
       }
     }
-    if (kind == 0) {
+    if (a.kinds == 2 && kind == 0) {
       sub1::drain_stores();   // this wavefront's h stores are in L2 ...
       __syncthreads();        // ... so are everyone's, and thread 0's release publishes them
       if (threadIdx.x == 0)
@@ -703,66 +741,116 @@ int check_dec(const int32_t *dec, hipStream_t stream) {
   return SUB1_OK;
 }
 
-int check_stack(const sub1_moe_stack *st, const char *who) {
-  if (!st) return fail(SUB1_ERR_NULL, "%s: NULL stack", who);
-  if (!st->dec || !st->w_comp || !st->wi_code_base || !st->wo_code_base || !st->wi_row_off ||
-      !st->wo_row_off || !st->wi_minmax || !st->wo_minmax)
-    return fail(SUB1_ERR_NULL, "%s: NULL pointer in the stack", who);
-  if (st->experts < 1 || st->d_model < 1 || st->d_ff < 1 ||
-      st->d_model > SUB1_PREPARED_MAX_WIDTH || st->d_ff > SUB1_PREPARED_MAX_WIDTH)
-    return fail(SUB1_ERR_SHAPE, "%s: experts %d d_model %d d_ff %d (sizes 1..%d)", who,
-                st->experts, st->d_model, st->d_ff, SUB1_PREPARED_MAX_WIDTH);
-  if (static_cast<int64_t>(st->experts) * ((st->d_ff + 63) / 64 + (st->d_model + 63) / 64) >
-      (1 << 24))
-    return fail(SUB1_ERR_SHAPE, "%s: too many 64-row slices", who);
-  if (misaligned(st->dec, 4) || misaligned(st->w_comp, 2) || misaligned(st->wi_code_base, 8) ||
-      misaligned(st->wo_code_base, 8) || misaligned(st->wi_row_off, 4) ||
-      misaligned(st->wo_row_off, 4) || misaligned(st->wi_minmax, 4) ||
-      misaligned(st->wo_minmax, 4))
-    return fail(SUB1_ERR_ALIGN, "%s: misaligned pointer in the stack", who);
+// What the prepare passes read: `kinds` groups of `count` matrices each.
+struct Source {
+  const int32_t *dec;
+  const uint16_t *w_comp;
+  const int64_t *code_base[2];   // [count] first codeword of each matrix, NULL = 0
+  const int32_t *row_off[2];     // [count, height+1]
+  const uint32_t *minmax[2];     // [count, height]
+  int kinds, count;
+  int height[2], width[2];
+};
+
+int check_source(const Source &src, const char *who) {
+  if (!src.dec || !src.w_comp) return fail(SUB1_ERR_NULL, "%s: NULL pointer", who);
+  if (src.count < 1) return fail(SUB1_ERR_SHAPE, "%s: %d matrices", who, src.count);
+  int64_t slices = 0;
+  for (int i = 0; i < src.kinds; i++) {
+    if (!src.row_off[i] || !src.minmax[i] || (src.count > 1 && !src.code_base[i]))
+      return fail(SUB1_ERR_NULL, "%s: NULL pointer", who);
+    if (src.height[i] < 1 || src.height[i] > 65534 || src.width[i] < 1 ||
+        src.width[i] > SUB1_PREPARED_MAX_WIDTH)
+      return fail(SUB1_ERR_SHAPE, "%s: matrix %d x %d (height 1..65534, width 1..%d)", who,
+                  src.height[i], src.width[i], SUB1_PREPARED_MAX_WIDTH);
+    if (misaligned(src.row_off[i], 4) || misaligned(src.minmax[i], 4) ||
+        misaligned(src.code_base[i], 8))
+      return fail(SUB1_ERR_ALIGN, "%s: misaligned pointer", who);
+    slices += static_cast<int64_t>(src.count) * ((src.height[i] + 63) / 64);
+  }
+  if (slices > (1 << 24)) return fail(SUB1_ERR_SHAPE, "%s: too many 64-row slices", who);
+  if (misaligned(src.dec, 4) || misaligned(src.w_comp, 2))
+    return fail(SUB1_ERR_ALIGN, "%s: misaligned pointer", who);
   return SUB1_OK;
 }
 
-}  // namespace
-
-// ================================================================ C ABI =====
-
-extern "C" int64_t sub1_moe_prepared_meta_bytes(int experts, int d_model, int d_ff) {
-  if (experts < 1 || d_model < 1 || d_ff < 1) return 0;
-  return meta_layout(experts, d_model, d_ff).bytes;
+Source moe_source(const sub1_moe_stack *st) {
+  Source src;
+  src.dec = st->dec;
+  src.w_comp = reinterpret_cast<const uint16_t *>(st->w_comp);
+  src.code_base[0] = st->wi_code_base;
+  src.code_base[1] = st->wo_code_base;
+  src.row_off[0] = st->wi_row_off;
+  src.row_off[1] = st->wo_row_off;
+  src.minmax[0] = static_cast<const uint32_t *>(st->wi_minmax);
+  src.minmax[1] = static_cast<const uint32_t *>(st->wo_minmax);
+  src.kinds = 2;
+  src.count = st->experts;
+  src.height[0] = st->d_ff;
+  src.width[0] = st->d_model;
+  src.height[1] = st->d_model;
+  src.width[1] = st->d_ff;
+  return src;
 }
 
-extern "C" int sub1_moe_prepare_layout(const sub1_moe_stack *st, void *meta, int64_t meta_bytes,
-                                       sub1_moe_prepared *out, void *stream) {
-  int rc = check_stack(st, "sub1_moe_prepare_layout");
-  if (rc) return rc;
-  if (!meta || !out) return fail(SUB1_ERR_NULL, "sub1_moe_prepare_layout: NULL argument");
-  if (misaligned(meta, 256)) return fail(SUB1_ERR_ALIGN, "sub1_moe_prepare_layout: meta must be 256-byte aligned");
-  const MetaLayout m = meta_layout(st->experts, st->d_model, st->d_ff);
+Source matrix_source(const sub1_matrix_set *ms) {
+  Source src;
+  src.dec = ms->dec;
+  src.w_comp = reinterpret_cast<const uint16_t *>(ms->w_comp);
+  src.code_base[0] = ms->code_base;
+  src.code_base[1] = nullptr;
+  src.row_off[0] = ms->row_off;
+  src.row_off[1] = nullptr;
+  src.minmax[0] = static_cast<const uint32_t *>(ms->ter_minmax);
+  src.minmax[1] = nullptr;
+  src.kinds = 1;
+  src.count = ms->count;
+  src.height[0] = ms->height;
+  src.width[0] = ms->width;
+  src.height[1] = 0;
+  src.width[1] = 0;
+  return src;
+}
+
+// What a prepared buffer pair holds, in the terms of the kernels.
+struct Prepared {
+  const void *meta;
+  const void *codes;
+  int64_t meta_bytes, code_bytes, total_chunks;
+  int kinds, count;
+  int height[2], width[2];
+  int max_chunks[2];
+};
+
+struct LayoutResult {
+  int64_t meta_bytes, code_bytes, total_chunks;
+  int max_chunks[2];
+};
+
+int prepare_layout(const Source &src, void *meta, int64_t meta_bytes, LayoutResult *out,
+                   hipStream_t s, const char *who) {
+  if (!meta || !out) return fail(SUB1_ERR_NULL, "%s: NULL argument", who);
+  if (misaligned(meta, 256)) return fail(SUB1_ERR_ALIGN, "%s: meta must be 256-byte aligned", who);
+  const MetaLayout m = meta_layout(src.count, src.kinds, src.height, src.width);
   if (meta_bytes < m.bytes)
-    return fail(SUB1_ERR_SHAPE, "sub1_moe_prepare_layout: meta needs %lld bytes",
-                static_cast<long long>(m.bytes));
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  rc = check_dec(st->dec, s);
+    return fail(SUB1_ERR_SHAPE, "%s: meta needs %lld bytes", who, static_cast<long long>(m.bytes));
+  int rc = check_dec(src.dec, s);
   if (rc) return rc;
   char *base = static_cast<char *>(meta);
   int32_t *status = reinterpret_cast<int32_t *>(base + m.status);
   int32_t *counts = reinterpret_cast<int32_t *>(base + m.counts);
   zero_words_kernel<<<1, 64, 0, s>>>(status, 4);
-  const int32_t *row_off[2] = {st->wi_row_off, st->wo_row_off};
-  const void *minmax[2] = {st->wi_minmax, st->wo_minmax};
   int64_t slice0 = 0;
-  for (int i = 0; i < 2; i++) {
+  for (int i = 0; i < src.kinds; i++) {
     const KindMeta &k = m.k[i];
-    order_rows_kernel<<<st->experts, 256, 0, s>>>(
-        row_off[i], static_cast<const uint32_t *>(minmax[i]),
-        reinterpret_cast<uint16_t *>(base + k.row_len),
+    order_rows_kernel<<<src.count, 256, 0, s>>>(
+        src.row_off[i], src.minmax[i], reinterpret_cast<uint16_t *>(base + k.row_len),
         reinterpret_cast<uint16_t *>(base + k.row_idx),
         reinterpret_cast<uint32_t *>(base + k.minmax),
         reinterpret_cast<uint16_t *>(base + k.slice_nch),
         reinterpret_cast<uint16_t *>(base + k.slice_nfull), counts + slice0, status, k.height,
         k.width, k.slices, i);
-    slice0 += static_cast<int64_t>(st->experts) * k.slices;
+    slice0 += static_cast<int64_t>(src.count) * k.slices;
   }
   scan_counts_kernel<<<1, 1024, 0, s>>>(counts, static_cast<int>(slice0));
   HIP_TRY(hipGetLastError());
@@ -772,56 +860,42 @@ extern "C" int sub1_moe_prepare_layout(const sub1_moe_stack *st, void *meta, int
   HIP_TRY(hipMemcpyAsync(&total, counts + slice0, 4, hipMemcpyDeviceToHost, s));
   HIP_TRY(hipStreamSynchronize(s));
   if (host[0])
-    return fail(SUB1_ERR_SHAPE,
-                "sub1_moe_prepare_layout: %d rows have a code count outside 1..width/2", host[0]);
-  if (total < 0) return fail(SUB1_ERR_SHAPE, "sub1_moe_prepare_layout: stream too large");
-  out->meta = meta;
-  out->codes = nullptr;
+    return fail(SUB1_ERR_SHAPE, "%s: %d rows have a code count outside 1..width/2", who, host[0]);
+  if (total < 0) return fail(SUB1_ERR_SHAPE, "%s: stream too large", who);
   out->meta_bytes = m.bytes;
   out->total_chunks = total;
   // the code stream, then one 128-byte checkpoint entry per group of chunks
   out->code_bytes = static_cast<int64_t>(total) * 512 +
                     (static_cast<int64_t>(total) / kGroupChunks + slice0 + 1) * 128;
-  out->experts = st->experts;
-  out->d_model = st->d_model;
-  out->d_ff = st->d_ff;
   out->max_chunks[0] = host[1];
   out->max_chunks[1] = host[2];
   return SUB1_OK;
 }
 
-extern "C" int sub1_moe_prepare_codes(const sub1_moe_stack *st, const sub1_moe_prepared *p,
-                                      void *stream) {
-  int rc = check_stack(st, "sub1_moe_prepare_codes");
-  if (rc) return rc;
-  if (!p || !p->meta || !p->codes)
-    return fail(SUB1_ERR_NULL, "sub1_moe_prepare_codes: NULL argument");
-  if (misaligned(p->meta, 256) || misaligned(p->codes, 256))
-    return fail(SUB1_ERR_ALIGN, "sub1_moe_prepare_codes: buffers must be 256-byte aligned");
-  if (p->experts != st->experts || p->d_model != st->d_model || p->d_ff != st->d_ff)
-    return fail(SUB1_ERR_SHAPE, "sub1_moe_prepare_codes: the layout belongs to another stack");
-  hipStream_t s = static_cast<hipStream_t>(stream);
+int prepare_codes(const Source &src, const Prepared &p, hipStream_t s, const char *who) {
+  if (!p.meta || !p.codes) return fail(SUB1_ERR_NULL, "%s: NULL argument", who);
+  if (misaligned(p.meta, 256) || misaligned(p.codes, 256))
+    return fail(SUB1_ERR_ALIGN, "%s: buffers must be 256-byte aligned", who);
   const DeviceTables *t = nullptr;
-  rc = device_tables(s, &t);
+  int rc = device_tables(s, &t);
   if (rc) return rc;
-  const MetaLayout m = meta_layout(st->experts, st->d_model, st->d_ff);
-  const char *base = static_cast<const char *>(p->meta);
-  const int64_t nslices = static_cast<int64_t>(st->experts) * (m.k[0].slices + m.k[1].slices);
-  if (p->total_chunks < 0 ||
-      p->code_bytes < p->total_chunks * 512 + (p->total_chunks / kGroupChunks + nslices + 1) * 128)
-    return fail(SUB1_ERR_SHAPE, "sub1_moe_prepare_codes: code buffer smaller than the layout needs");
-  uint16_t *codes = static_cast<uint16_t *>(const_cast<void *>(p->codes));
-  uint16_t *ckpt = codes + p->total_chunks * 256;
-  const int64_t *code_base[2] = {st->wi_code_base, st->wo_code_base};
-  const int32_t *row_off[2] = {st->wi_row_off, st->wo_row_off};
+  const MetaLayout m = meta_layout(src.count, src.kinds, src.height, src.width);
+  const char *base = static_cast<const char *>(p.meta);
+  int64_t nslices = 0;
+  for (int i = 0; i < src.kinds; i++) nslices += static_cast<int64_t>(src.count) * m.k[i].slices;
+  if (p.total_chunks < 0 || p.meta_bytes < m.bytes ||
+      p.code_bytes < p.total_chunks * 512 + (p.total_chunks / kGroupChunks + nslices + 1) * 128)
+    return fail(SUB1_ERR_SHAPE, "%s: buffers smaller than the layout needs", who);
+  uint16_t *codes = static_cast<uint16_t *>(const_cast<void *>(p.codes));
+  uint16_t *ckpt = codes + p.total_chunks * 256;
   const int group_shift = t->single_codes - t->single_codes / 8;
   int64_t first_slice = 0;
-  for (int i = 0; i < 2; i++) {
+  for (int i = 0; i < src.kinds; i++) {
     const KindMeta &k = m.k[i];
-    const int64_t kslices = static_cast<int64_t>(st->experts) * k.slices;
+    const int64_t kslices = static_cast<int64_t>(src.count) * k.slices;
     const int64_t lanes = kslices * 64;
     interleave_codes_kernel<<<static_cast<unsigned>((lanes + 3) / 4), 256, 0, s>>>(
-        reinterpret_cast<const uint16_t *>(st->w_comp), code_base[i], row_off[i], t->recode,
+        src.w_comp, src.code_base[i], src.row_off[i], t->recode,
         reinterpret_cast<const uint32_t *>(base + k.slice_base),
         reinterpret_cast<const uint16_t *>(base + k.slice_nch),
         reinterpret_cast<const uint16_t *>(base + k.row_idx), codes, k.height, k.slices, lanes);
@@ -835,48 +909,58 @@ extern "C" int sub1_moe_prepare_codes(const sub1_moe_stack *st, const sub1_moe_p
   return SUB1_OK;
 }
 
-extern "C" int sub1_moe_grouped_prepared(const sub1_moe_prepared *p, const int32_t *token_expert,
-                                         const void *x, void *y, int tokens, void *workspace,
-                                         int64_t workspace_bytes, void *stream) {
-  if (!p) return fail(SUB1_ERR_NULL, "sub1_moe_grouped_prepared: NULL argument");
-  if (tokens == 0) return SUB1_OK;
-  if (!p->meta || !p->codes || !token_expert || !x || !y)
-    return fail(SUB1_ERR_NULL, "sub1_moe_grouped_prepared: NULL argument");
-  if (p->experts < 1 || p->d_model < 1 || p->d_ff < 1 ||
-      p->d_model > SUB1_PREPARED_MAX_WIDTH || p->d_ff > SUB1_PREPARED_MAX_WIDTH)
-    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: experts %d d_model %d d_ff %d",
-                p->experts, p->d_model, p->d_ff);
+// Launch of the prepared kernel.  kinds == 2: y = wo(relu(wi x)) per token,
+// workspace required; kinds == 1: y += W x per token, no workspace.
+int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *x, int64_t ldx,
+                    void *y, int64_t ldy, int tokens, void *workspace, int64_t workspace_bytes,
+                    hipStream_t s, const char *who) {
+  if (!p.meta || !p.codes || !x || !y) return fail(SUB1_ERR_NULL, "%s: NULL argument", who);
+  if (p.kinds == 2 && !token_matrix) return fail(SUB1_ERR_NULL, "%s: NULL token_expert", who);
   if (tokens < 0 || tokens > (1 << 20))
-    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: tokens %d outside 0..2^20", tokens);
-  if (!workspace || workspace_bytes < sub1_moe_workspace_bytes(tokens, p->d_ff))
-    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: workspace of %lld bytes needed",
-                static_cast<long long>(sub1_moe_workspace_bytes(tokens, p->d_ff)));
-  if (misaligned(workspace, 256) || misaligned(p->meta, 256) || misaligned(p->codes, 256) ||
-      misaligned(token_expert, 4) || misaligned(x, 2) || misaligned(y, 2))
-    return fail(SUB1_ERR_ALIGN, "sub1_moe_grouped_prepared: misaligned pointer");
-  hipStream_t s = static_cast<hipStream_t>(stream);
+    return fail(SUB1_ERR_SHAPE, "%s: tokens %d outside 0..2^20", who, tokens);
+  if (ldx < p.width[0] || ldy < (p.kinds == 2 ? p.height[1] : p.height[0]))
+    return fail(SUB1_ERR_SHAPE, "%s: token strides smaller than the rows", who);
+  if (misaligned(p.meta, 256) || misaligned(p.codes, 256) || misaligned(token_matrix, 4) ||
+      misaligned(x, 2) || misaligned(y, 2))
+    return fail(SUB1_ERR_ALIGN, "%s: misaligned pointer", who);
+  const int d_ff = p.kinds == 2 ? p.height[0] : 0;
+  if (p.kinds == 2) {
+    if (!workspace || workspace_bytes < sub1_moe_workspace_bytes(tokens, d_ff))
+      return fail(SUB1_ERR_SHAPE, "%s: workspace of %lld bytes needed", who,
+                  static_cast<long long>(sub1_moe_workspace_bytes(tokens, d_ff)));
+    if (misaligned(workspace, 256)) return fail(SUB1_ERR_ALIGN, "%s: misaligned workspace", who);
+  }
   const DeviceTables *t = nullptr;
   int rc = device_tables(s, &t);
   if (rc) return rc;
-  const MetaLayout m = meta_layout(p->experts, p->d_model, p->d_ff);
-  if (p->meta_bytes < m.bytes)
-    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: meta smaller than its layout");
-  const char *base = static_cast<const char *>(p->meta);
+  const MetaLayout m = meta_layout(p.count, p.kinds, p.height, p.width);
+  if (p.meta_bytes < m.bytes) return fail(SUB1_ERR_SHAPE, "%s: meta smaller than its layout", who);
+  const char *base = static_cast<const char *>(p.meta);
 
   PreparedArgs a;
   a.table = t->table;
-  a.codes = static_cast<const uint16_t *>(p->codes);
+  a.codes = static_cast<const uint16_t *>(p.codes);
+  a.ckpt = a.codes + p.total_chunks * 256;
+  a.kinds = p.kinds;
+  int wmax = 0;
   for (int i = 0; i < 2; i++) {
+    KindArgs &ka = a.k[i];
+    if (i >= p.kinds) {
+      ka = a.k[0];
+      ka.parts = 0;
+      continue;
+    }
     const KindMeta &k = m.k[i];
-    a.k[i].slice_base = reinterpret_cast<const uint32_t *>(base + k.slice_base);
-    a.k[i].slice_nch = reinterpret_cast<const uint16_t *>(base + k.slice_nch);
-    a.k[i].slice_nfull = reinterpret_cast<const uint16_t *>(base + k.slice_nfull);
-    a.k[i].row_len = reinterpret_cast<const uint16_t *>(base + k.row_len);
-    a.k[i].row_idx = reinterpret_cast<const uint16_t *>(base + k.row_idx);
-    a.k[i].minmax = reinterpret_cast<const uint32_t *>(base + k.minmax);
-    a.k[i].slices = k.slices;
-    a.k[i].height = k.height;
-    a.k[i].width = k.width;
+    ka.slice_base = reinterpret_cast<const uint32_t *>(base + k.slice_base);
+    ka.slice_nch = reinterpret_cast<const uint16_t *>(base + k.slice_nch);
+    ka.slice_nfull = reinterpret_cast<const uint16_t *>(base + k.slice_nfull);
+    ka.row_len = reinterpret_cast<const uint16_t *>(base + k.row_len);
+    ka.row_idx = reinterpret_cast<const uint16_t *>(base + k.row_idx);
+    ka.minmax = reinterpret_cast<const uint32_t *>(base + k.minmax);
+    ka.slices = k.slices;
+    ka.height = k.height;
+    ka.width = k.width;
+    if (k.width > wmax) wmax = k.width;
   }
   // 16 wavefronts per workgroup.  A count that divides the slice counts better
   // (11 for the c-2048 shapes) leaves fewer idle wavefront slots but measured
@@ -885,25 +969,28 @@ extern "C" int sub1_moe_grouped_prepared(const sub1_moe_prepared *p, const int32
   int device = 0, cus = 0;
   HIP_TRY(hipGetDevice(&device));
   HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
-  a.ckpt = a.codes + p->total_chunks * 256;
-  a.token_expert = token_expert;
+  a.token_expert = token_matrix;
   a.x = static_cast<const uint16_t *>(x);
   a.y = static_cast<uint16_t *>(y);
-  a.ctrl = static_cast<int32_t *>(workspace);
-  int64_t ctrl_bytes = (static_cast<int64_t>(kCtrlHeader + tokens) * 4 + 255) / 256 * 256;
-  a.h = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + ctrl_bytes);
+  a.ldx = ldx;
+  a.ldy = ldy;
+  a.ctrl = nullptr;
+  a.h = nullptr;
+  if (p.kinds == 2) {
+    a.ctrl = static_cast<int32_t *>(workspace);
+    int64_t ctrl_bytes = (static_cast<int64_t>(kCtrlHeader + tokens) * 4 + 255) / 256 * 256;
+    a.h = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + ctrl_bytes);
+  }
   a.tokens = tokens;
-  a.experts = p->experts;
+  a.experts = p.count;
   a.table_words = t->words;
   a.single_codes = t->single_codes;
   a.group_shift = t->single_codes - t->single_codes / 8;
-  const int wmax = p->d_model > p->d_ff ? p->d_model : p->d_ff;
   a.xdwords = activation_dwords(wmax);
   a.spin_limit = 1 << 24;
   const size_t lds_limit = 160 * 1024 - 64;
   const size_t lds_base = (static_cast<size_t>(a.table_words) + a.xdwords) * 4;
-  if (lds_base > lds_limit)
-    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: width %d does not fit LDS", wmax);
+  if (lds_base > lds_limit) return fail(SUB1_ERR_SHAPE, "%s: width %d does not fit LDS", who, wmax);
   // Tiles.  Whole matrices when the tokens alone keep every compute unit busy;
   // otherwise each matrix is cut into parts, down to one slice per wavefront;
   // and when even that leaves compute units idle (a handful of tokens), several
@@ -911,11 +998,12 @@ extern "C" int sub1_moe_grouped_prepared(const sub1_moe_prepared *p, const int32
   const int want = (cus + tokens - 1) / tokens;   // tiles per token and projection
   size_t lds_partials = 0;
   int64_t first_slice = 0;
-  for (int i = 0; i < 2; i++) {
+  int64_t tiles = 0;
+  for (int i = 0; i < p.kinds; i++) {
     KindArgs &k = a.k[i];
     k.first_slice = first_slice;
-    first_slice += static_cast<int64_t>(p->experts) * k.slices;
-    k.groups_max = (p->max_chunks[i] + kGroupChunks - 1) / kGroupChunks;
+    first_slice += static_cast<int64_t>(p.count) * k.slices;
+    k.groups_max = (p.max_chunks[i] + kGroupChunks - 1) / kGroupChunks;
     k.split = 1;
     const int max_parts = (k.slices + waves - 1) / waves;
     k.parts = want > max_parts ? max_parts : want;
@@ -934,18 +1022,179 @@ extern "C" int sub1_moe_grouped_prepared(const sub1_moe_prepared *p, const int32
         if (need > lds_partials) lds_partials = need;
       }
     }
+    tiles += static_cast<int64_t>(tokens) * k.parts;
   }
-  int64_t tiles = static_cast<int64_t>(tokens) * (a.k[0].parts + a.k[1].parts);
-  if (tiles > INT32_MAX - (1 << 20))
-    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: too many tiles");
+  if (tiles > INT32_MAX - (1 << 20)) return fail(SUB1_ERR_SHAPE, "%s: too many tiles", who);
   const size_t lds = lds_base + lds_partials;
   HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(moe_prepared_kernel),
                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
   int64_t grid = cus;  // one workgroup per compute unit (LDS holds the table once)
   if (grid > tiles) grid = tiles;
-  int nctrl = kCtrlHeader + tokens;
-  zero_words_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl);
+  if (a.ctrl) {
+    int nctrl = kCtrlHeader + tokens;
+    zero_words_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl);
+  }
   moe_prepared_kernel<<<static_cast<unsigned>(grid), 64 * waves, lds, s>>>(a);
   HIP_TRY(hipGetLastError());
   return SUB1_OK;
+}
+
+int check_moe_stack(const sub1_moe_stack *st, const char *who) {
+  if (!st) return fail(SUB1_ERR_NULL, "%s: NULL stack", who);
+  if (st->experts < 1 || st->d_model < 1 || st->d_ff < 1)
+    return fail(SUB1_ERR_SHAPE, "%s: experts %d d_model %d d_ff %d", who, st->experts,
+                st->d_model, st->d_ff);
+  return check_source(moe_source(st), who);
+}
+
+int check_matrix_set(const sub1_matrix_set *ms, const char *who) {
+  if (!ms) return fail(SUB1_ERR_NULL, "%s: NULL matrix set", who);
+  return check_source(matrix_source(ms), who);
+}
+
+}  // namespace
+
+// ================================================================ C ABI =====
+
+extern "C" int64_t sub1_moe_prepared_meta_bytes(int experts, int d_model, int d_ff) {
+  if (experts < 1 || d_model < 1 || d_ff < 1) return 0;
+  return moe_layout(experts, d_model, d_ff).bytes;
+}
+
+extern "C" int sub1_moe_prepare_layout(const sub1_moe_stack *st, void *meta, int64_t meta_bytes,
+                                       sub1_moe_prepared *out, void *stream) {
+  int rc = check_moe_stack(st, "sub1_moe_prepare_layout");
+  if (rc) return rc;
+  if (!out) return fail(SUB1_ERR_NULL, "sub1_moe_prepare_layout: NULL argument");
+  LayoutResult r;
+  rc = prepare_layout(moe_source(st), meta, meta_bytes, &r, static_cast<hipStream_t>(stream),
+                      "sub1_moe_prepare_layout");
+  if (rc) return rc;
+  out->meta = meta;
+  out->codes = nullptr;
+  out->meta_bytes = r.meta_bytes;
+  out->code_bytes = r.code_bytes;
+  out->total_chunks = r.total_chunks;
+  out->experts = st->experts;
+  out->d_model = st->d_model;
+  out->d_ff = st->d_ff;
+  out->max_chunks[0] = r.max_chunks[0];
+  out->max_chunks[1] = r.max_chunks[1];
+  return SUB1_OK;
+}
+
+namespace {
+Prepared from_moe(const sub1_moe_prepared *p) {
+  Prepared q;
+  q.meta = p->meta;
+  q.codes = p->codes;
+  q.meta_bytes = p->meta_bytes;
+  q.code_bytes = p->code_bytes;
+  q.total_chunks = p->total_chunks;
+  q.kinds = 2;
+  q.count = p->experts;
+  q.height[0] = p->d_ff;
+  q.width[0] = p->d_model;
+  q.height[1] = p->d_model;
+  q.width[1] = p->d_ff;
+  q.max_chunks[0] = p->max_chunks[0];
+  q.max_chunks[1] = p->max_chunks[1];
+  return q;
+}
+
+Prepared from_matrix(const sub1_matrix_prepared *p) {
+  Prepared q;
+  q.meta = p->meta;
+  q.codes = p->codes;
+  q.meta_bytes = p->meta_bytes;
+  q.code_bytes = p->code_bytes;
+  q.total_chunks = p->total_chunks;
+  q.kinds = 1;
+  q.count = p->count;
+  q.height[0] = p->height;
+  q.width[0] = p->width;
+  q.height[1] = 0;
+  q.width[1] = 0;
+  q.max_chunks[0] = p->max_chunks;
+  q.max_chunks[1] = 0;
+  return q;
+}
+
+bool bad_dims(int count, int h, int w) {
+  return count < 1 || h < 1 || w < 1 || h > 65534 || w > SUB1_PREPARED_MAX_WIDTH;
+}
+}  // namespace
+
+extern "C" int sub1_moe_prepare_codes(const sub1_moe_stack *st, const sub1_moe_prepared *p,
+                                      void *stream) {
+  int rc = check_moe_stack(st, "sub1_moe_prepare_codes");
+  if (rc) return rc;
+  if (!p) return fail(SUB1_ERR_NULL, "sub1_moe_prepare_codes: NULL argument");
+  if (p->experts != st->experts || p->d_model != st->d_model || p->d_ff != st->d_ff)
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_prepare_codes: the layout belongs to another stack");
+  return prepare_codes(moe_source(st), from_moe(p), static_cast<hipStream_t>(stream),
+                       "sub1_moe_prepare_codes");
+}
+
+extern "C" int sub1_moe_grouped_prepared(const sub1_moe_prepared *p, const int32_t *token_expert,
+                                         const void *x, void *y, int tokens, void *workspace,
+                                         int64_t workspace_bytes, void *stream) {
+  if (!p) return fail(SUB1_ERR_NULL, "sub1_moe_grouped_prepared: NULL argument");
+  if (tokens == 0) return SUB1_OK;
+  if (bad_dims(p->experts, p->d_ff, p->d_model) || bad_dims(p->experts, p->d_model, p->d_ff))
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped_prepared: experts %d d_model %d d_ff %d",
+                p->experts, p->d_model, p->d_ff);
+  return launch_prepared(from_moe(p), token_expert, x, p->d_model, y, p->d_model, tokens,
+                         workspace, workspace_bytes, static_cast<hipStream_t>(stream),
+                         "sub1_moe_grouped_prepared");
+}
+
+extern "C" int64_t sub1_matrix_prepared_meta_bytes(int count, int height, int width) {
+  if (count < 1 || height < 1 || width < 1) return 0;
+  return matrix_layout(count, height, width).bytes;
+}
+
+extern "C" int sub1_matrix_prepare_layout(const sub1_matrix_set *ms, void *meta,
+                                          int64_t meta_bytes, sub1_matrix_prepared *out,
+                                          void *stream) {
+  int rc = check_matrix_set(ms, "sub1_matrix_prepare_layout");
+  if (rc) return rc;
+  if (!out) return fail(SUB1_ERR_NULL, "sub1_matrix_prepare_layout: NULL argument");
+  LayoutResult r;
+  rc = prepare_layout(matrix_source(ms), meta, meta_bytes, &r, static_cast<hipStream_t>(stream),
+                      "sub1_matrix_prepare_layout");
+  if (rc) return rc;
+  out->meta = meta;
+  out->codes = nullptr;
+  out->meta_bytes = r.meta_bytes;
+  out->code_bytes = r.code_bytes;
+  out->total_chunks = r.total_chunks;
+  out->count = ms->count;
+  out->height = ms->height;
+  out->width = ms->width;
+  out->max_chunks = r.max_chunks[0];
+  return SUB1_OK;
+}
+
+extern "C" int sub1_matrix_prepare_codes(const sub1_matrix_set *ms,
+                                         const sub1_matrix_prepared *p, void *stream) {
+  int rc = check_matrix_set(ms, "sub1_matrix_prepare_codes");
+  if (rc) return rc;
+  if (!p) return fail(SUB1_ERR_NULL, "sub1_matrix_prepare_codes: NULL argument");
+  if (p->count != ms->count || p->height != ms->height || p->width != ms->width)
+    return fail(SUB1_ERR_SHAPE, "sub1_matrix_prepare_codes: the layout belongs to other matrices");
+  return prepare_codes(matrix_source(ms), from_matrix(p), static_cast<hipStream_t>(stream),
+                       "sub1_matrix_prepare_codes");
+}
+
+extern "C" int sub1_matvec_prepared(const sub1_matrix_prepared *p, const int32_t *token_matrix,
+                                    const void *x, int64_t ldx, void *y, int64_t ldy,
+                                    int tokens, void *stream) {
+  if (!p) return fail(SUB1_ERR_NULL, "sub1_matvec_prepared: NULL argument");
+  if (tokens == 0) return SUB1_OK;
+  if (bad_dims(p->count, p->height, p->width))
+    return fail(SUB1_ERR_SHAPE, "sub1_matvec_prepared: %d matrices of %d x %d", p->count,
+                p->height, p->width);
+  return launch_prepared(from_matrix(p), token_matrix, x, ldx, y, ldy, tokens, nullptr, 0,
+                         static_cast<hipStream_t>(stream), "sub1_matvec_prepared");
 }

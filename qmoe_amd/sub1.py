@@ -7,7 +7,8 @@ Differences from the reference that a caller can observe:
   * importing works without a GPU (the reference indexes GPUS[-1] at import,
     sub1.py:107-111); the device tables are then empty until a GPU exists;
   * `Sub1Linear.forward` runs all tokens in one launch (the reference loops
-    over tokens, sub1.py:137-142);
+    over tokens, sub1.py:137-142), from a copy of the codes in a GPU-friendly
+    layout that it makes on first use (`Sub1Linear.fast`);
   * any (height, width) works, not only the six Switch shapes.
 """
 import torch
@@ -55,15 +56,35 @@ class Sub1Linear(nn.Module):
         self.register_buffer('ter_minmax', torch.zeros(2 * height, dtype=torch.bfloat16))
         self.register_buffer('weight', torch.zeros(0, dtype=torch.bfloat16))
 
+    # forward() goes through a copy of the codes in the layout the GPU streams
+    # fastest, made on first use (it costs about as much memory again as w_comp
+    # and is remade when a buffer is replaced or written in place).  Set to
+    # False to run straight from the packed buffers instead.
+    fast = True
+
+    def _prepared(self, width):
+        key = tuple((t.data_ptr(), t._version, t.numel())
+                    for t in (self.w_comp, self.row_off, self.ter_minmax)) + (width,)
+        cached = getattr(self, '_prepared_cache', None)
+        if cached is None or cached[0] != key:
+            table = DEC[self.w_comp.device.index]
+            cached = (key, sub1_hip.PreparedMatrix(table, self.w_comp, self.row_off,
+                                                   self.ter_minmax, width))
+            self._prepared_cache = cached
+        return cached[1]
+
     def forward(self, x):
         """x bf16 [T, width] -> bf16 [T, height] (reference sub1.py:132-143)."""
         height = self.row_off.shape[0] - 1
         y = torch.zeros((x.shape[0], height), dtype=torch.bfloat16, device=x.device)
         if x.shape[0] == 0:
             return y
-        table = DEC[self.w_comp.device.index]
-        sub1_hip.sub1matvec_tokens(table, self.w_comp, self.row_off, self.ter_minmax,
-                                   x.contiguous(), y)
+        x = x.contiguous()
+        if self.fast and x.shape[1] <= sub1_hip.PREPARED_MAX_WIDTH:
+            self._prepared(x.shape[1]).matvec_tokens(x, y)
+        else:
+            table = DEC[self.w_comp.device.index]
+            sub1_hip.sub1matvec_tokens(table, self.w_comp, self.row_off, self.ter_minmax, x, y)
         return y
 
     @staticmethod

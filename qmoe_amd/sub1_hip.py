@@ -17,6 +17,7 @@ import torch
 from . import _lib
 
 DICT_ENTRIES = _lib.DICT_ENTRIES
+PREPARED_MAX_WIDTH = _lib.PREPARED_MAX_WIDTH
 
 
 def _stream():
@@ -273,3 +274,44 @@ class PreparedStack:
     def launch_faults(self, tokens):
         ctrl = self.workspace(tokens)[:16].view(torch.int32).tolist()
         return ctrl[1], ctrl[2]
+
+
+class PreparedMatrix:
+    """One compressed matrix (the three buffers of a Sub1Linear) copied into
+    the fast layout; `matvec_tokens(x, y)` does y[t] += W x[t] like
+    sub1matvec_tokens, in one launch with the decode table in LDS."""
+
+    def __init__(self, dec, w_comp, row_off, ter_minmax, width):
+        lib = _lib.load()
+        dev = dec.device
+        height = row_off.numel() - 1
+        self.device, self.height, self.width = dev, height, width
+        src = _lib.MatrixSet(
+            _need(dec, torch.int32, 'dec', numel=_lib.DEC_WORDS),
+            _need(w_comp, torch.int16, 'w_comp', dev), None,
+            _need(row_off, torch.int32, 'row_off', dev),
+            _need(ter_minmax, torch.bfloat16, 'ter_minmax', dev, numel=2 * height),
+            1, height, width)
+        meta_bytes = lib.sub1_matrix_prepared_meta_bytes(1, height, width)
+        self.meta = torch.empty(meta_bytes, dtype=torch.uint8, device=dev)
+        self._c = _lib.MatrixPrepared()
+        with torch.cuda.device(dev):
+            _lib.check(lib.sub1_matrix_prepare_layout(ctypes.byref(src), self.meta.data_ptr(),
+                                                      meta_bytes, ctypes.byref(self._c), _stream()))
+            self.codes = torch.empty(max(self._c.code_bytes, 256), dtype=torch.uint8, device=dev)
+            self._c.codes = self.codes.data_ptr()
+            _lib.check(lib.sub1_matrix_prepare_codes(ctypes.byref(src), ctypes.byref(self._c),
+                                                     _stream()))
+
+    def matvec_tokens(self, x, y):
+        dev = self.device
+        p_x = _need(x, torch.bfloat16, 'x', dev, dim=2)
+        p_y = _need(y, torch.bfloat16, 'y', dev, dim=2)
+        tokens = x.shape[0]
+        if x.shape[1] != self.width or y.shape != (tokens, self.height):
+            raise ValueError('x must be [T, %d] and y [T, %d]' % (self.width, self.height))
+        if tokens == 0:
+            return
+        with torch.cuda.device(dev):
+            _lib.check(_lib.load().sub1_matvec_prepared(
+                ctypes.byref(self._c), None, p_x, self.width, p_y, self.height, tokens, _stream()))

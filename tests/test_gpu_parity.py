@@ -400,3 +400,41 @@ def test_every_tiling_mode_gives_the_same_bits(gpu, oracle):
         assert torch.equal(y[0], want), tokens
         if tokens > 1:
             assert torch.equal(y[1], y[tokens - 1])
+
+
+@pytest.mark.parametrize('height,width,p0', SWITCH_SHAPES + [(77, 333, 0.7), (5, 1, 0.5),
+                                                             (130, 15, 0.9), (300, 8192, 0.99)])
+def test_prepared_matrix_product(gpu, oracle, height, width, p0):
+    """The single-matrix fast path (what Sub1Linear.forward uses): y += W x for
+    several tokens, bit-exact against the oracle, accumulating like sub1matvec."""
+    sub1, op = gpu
+    c = dev_case(oracle, height, width, p0, seed=11 * height + width)
+    pm = op.PreparedMatrix(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], width)
+    tokens = 3
+    xs = np.stack([c['x']] + [so.synthetic_activation(width, 900 + i) for i in range(tokens - 1)])
+    pre = so.f32_to_bf16_bits(np.random.default_rng(1).standard_normal((tokens, height)).astype(np.float32))
+    y = bf16_dev(pre).clone()
+    pm.matvec_tokens(bf16_dev(xs), y)
+    got = bits_host(y)
+    for i in range(tokens):
+        want = oracle.matvec_seq(c['codes'], c['row_off'], c['mm'], xs[i], y=pre[i])
+        assert np.array_equal(got[i], want), i
+    y0 = torch.zeros((1, height), dtype=torch.bfloat16, device='cuda')
+    pm.matvec_tokens(c['x_d'].reshape(1, -1), y0)
+    check_product(oracle, c, bits_host(y0[0]))
+
+
+def test_sub1linear_fast_and_packed_paths_agree(gpu, oracle):
+    sub1, op = gpu
+    t, mm = so.synthetic_ternary(3072, 768, 0.9, seed=77)
+    w = bf16_dev(oracle.dequant(t.astype(np.uint8), mm))
+    lin = sub1.Sub1Linear.make(w)
+    x = torch.randn((4, 768), generator=torch.Generator().manual_seed(3)).bfloat16().cuda()
+    y_fast = lin(x)
+    lin.fast = False
+    y_packed = lin(x)
+    assert torch.equal(y_fast, y_packed)
+    # replacing a buffer invalidates the prepared copy
+    lin.fast = True
+    lin.ter_minmax = (lin.ter_minmax.float() * 2).bfloat16()
+    assert torch.equal(lin(x).float(), 2 * y_fast.float())
