@@ -13,11 +13,15 @@
 //   * codes are renumbered (sub1_build_kernel_tables) so that the decode table
 //     is 61.5 KB and lives in LDS next to the activations.
 //
-// moe_prepared_kernel then walks 64 rows per wavefront: per codeword one LDS
-// table read and three LDS activation reads, each folded into two running
-// sums (activations under row-min weights, under row-max weights) with
+// The kernels then walk 64 rows per wavefront: per codeword one LDS table read
+// and three LDS activation reads, each folded into two running sums
+// (activations under row-min weights, under row-max weights) with
 // v_dot2c_f32_bf16 on (x,0)/(0,x) bf16 pairs; no cross-lane traffic at all.
-// It computes what reference sub1_cuda_kernel.cu:163-201 computes per row.
+// They compute what reference sub1_cuda_kernel.cu:163-201 computes per row.
+// moe_prepared_kernel is the streaming form (persistent grid, a wavefront per
+// slice, the next slice's loads in flight); moe_prepared_small_kernel is the
+// latency form for a handful of tokens (one tile per workgroup, wavefronts
+// share a slice from column checkpoints).  Both give the same bits.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -37,10 +41,11 @@ using sub1::row_result;
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kMaxThreads = 1024;      // the launch picks 8..16 wavefronts per workgroup
+constexpr int kMaxThreads = 1024;    // 16 wavefronts per workgroup
 constexpr int kChunk = 4;            // codes per lane per chunk
 constexpr int kRing = 4;             // chunks in flight per lane (2 KB per wavefront)
 constexpr int kGroupChunks = 8;      // chunks (32 codes) per partial sum, a multiple of kRing
+constexpr int kSplitRing = 8;        // chunks in flight per lane where wavefronts share a slice
 constexpr int kMaxLen = 4096;        // codes per row: one per column pair at most
 constexpr int kCtrlHeader = 4;       // ctrl[0] ticket, [1] wait-limit hits, [2] bad expert ids
 constexpr uint32_t kIdleWord = 0x00040404u;  // three empty slots, no advance
@@ -314,18 +319,59 @@ __host__ __device__ constexpr int activation_dwords(int width) {
   return 6 * ((width + 28 + 1) / 2 + 1);
 }
 
+// Every load of a thread is in flight before its first LDS store, so a tile
+// pays one memory round trip for its activations, not one per pass.
 __device__ __forceinline__ void stage_activations(uint32_t *xa, const uint16_t *x, int width) {
   const int npairs = (width + 28 + 1) / 2 + 1;
-  for (int m = threadIdx.x; m < npairs; m += blockDim.x) {
-    uint32_t xe = 2 * m < width ? x[2 * m] : 0u;
-    uint32_t xo = 2 * m + 1 < width ? x[2 * m + 1] : 0u;
-    uint32_t *p = xa + 6 * m;
-    p[0] = xe;
-    p[1] = xe << 16;
-    p[2] = xo;
-    p[3] = xo << 16;
-    p[4] = 0u;
-    p[5] = 0u;
+  const int step = blockDim.x;
+  const bool aligned = (reinterpret_cast<uintptr_t>(x) & 3u) == 0;
+  for (int m0 = threadIdx.x; m0 < npairs; m0 += 4 * step) {
+    uint32_t v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const int m = m0 + u * step;
+      v[u] = 0u;
+      if (aligned && 2 * m + 1 < width) {
+        v[u] = *reinterpret_cast<const uint32_t *>(x + 2 * m);
+      } else {
+        if (2 * m < width) v[u] = x[2 * m];
+        if (2 * m + 1 < width) v[u] |= static_cast<uint32_t>(x[2 * m + 1]) << 16;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const int m = m0 + u * step;
+      if (m < npairs) {
+        uint32_t *p = xa + 6 * m;
+        p[0] = v[u] & 0xffffu;
+        p[1] = v[u] << 16;
+        p[2] = v[u] >> 16;
+        p[3] = v[u] & 0xffff0000u;
+        p[4] = 0u;
+        p[5] = 0u;
+      }
+    }
+  }
+}
+
+// The decode table into LDS with 16-byte loads, all of a thread's loads in
+// flight before its first store.  `words` is a multiple of 4 and the global
+// copy is padded to it.
+__device__ __forceinline__ void stage_table(uint32_t *tab, const uint32_t *src, int words) {
+  const uint4 *s4 = reinterpret_cast<const uint4 *>(src);
+  uint4 *d4 = reinterpret_cast<uint4 *>(tab);
+  const int n4 = words >> 2;
+  const int step = blockDim.x;
+  for (int i0 = threadIdx.x; i0 < n4; i0 += 4 * step) {
+    const int i1 = i0 + step, i2 = i1 + step, i3 = i2 + step;
+    const uint4 v0 = s4[i0];   // indices clamped: every load is valid and unconditional
+    const uint4 v1 = s4[min(i1, n4 - 1)];
+    const uint4 v2 = s4[min(i2, n4 - 1)];
+    const uint4 v3 = s4[min(i3, n4 - 1)];
+    d4[i0] = v0;
+    if (i1 < n4) d4[i1] = v1;
+    if (i2 < n4) d4[i2] = v2;
+    if (i3 < n4) d4[i3] = v3;
   }
 }
 
@@ -384,12 +430,14 @@ __device__ __forceinline__ void add_codeword(uint32_t e, const uint32_t *xa, int
 // What a lane needs to walk its row of one slice; load_slice issues the loads
 // of the first chunks, so calling it for the NEXT slice before walking the
 // current one hides their latency.
-struct SliceWalk {
+template <int R>
+struct Walk {
   const uint2 *p;
   int nch, nfull, len, ridx;
   uint32_t minmax;
-  uint2 ring[kRing];
+  uint2 ring[R];
 };
+typedef Walk<kRing> SliceWalk;
 
 __device__ __forceinline__ SliceWalk load_slice(const PreparedArgs &a, const KindArgs &k,
                                                 int64_t sl) {
@@ -408,19 +456,19 @@ __device__ __forceinline__ SliceWalk load_slice(const PreparedArgs &a, const Kin
   return w;
 }
 
-// kRing chunks starting at chunk c added onto the partial sums p1, p2.
-// kChecked: compare every code with the lane's own count.
-template <bool kChecked>
-__device__ __forceinline__ void run_chunks(SliceWalk &w, int c, uint32_t shift2,
+// R chunks (the depth of the walk's ring) starting at chunk c added onto the
+// partial sums p1, p2.  kChecked: compare every code with the lane's own count.
+template <bool kChecked, int R>
+__device__ __forceinline__ void run_chunks(Walk<R> &w, int c, uint32_t shift2,
                                            const uint32_t *tab, const uint32_t *xa, int &colw,
                                            float &p1, float &p2, const DotConsts &dk) {
   const uint2 *p = w.p;
   const int nch = w.nch;
 #pragma unroll
-  for (int i = 0; i < kRing; i++) {
+  for (int i = 0; i < R; i++) {
     if (!kChecked || c + i < nch) {
       const uint2 cw = w.ring[i];
-      if (c + i + kRing < nch) w.ring[i] = p[(c + i + kRing) * 64];
+      if (c + i + R < nch) w.ring[i] = p[(c + i + R) * 64];
       uint32_t e[4];
       lookup4(tab, cw, shift2, e);
       const int j = kChunk * (c + i);
@@ -428,6 +476,9 @@ __device__ __forceinline__ void run_chunks(SliceWalk &w, int c, uint32_t shift2,
       for (int q = 0; q < 4; q++)
         add_codeword(!kChecked || j + q < w.len ? e[q] : kIdleWord, xa, colw, p1, p2, dk);
     }
+    // a deep ring is for latency: keep the scheduler from also hoisting every
+    // chunk's table words, which would not fit the registers
+    if (R > kRing) __builtin_amdgcn_sched_barrier(0);
   }
 }
 
@@ -489,68 +540,178 @@ __device__ __forceinline__ void write_row(uint16_t *dst, int ridx, uint32_t minm
 // checkpoint of its first group) and leaving one partial-sum pair per group in
 // LDS; after a barrier the slice's first wavefront adds the groups in order,
 // which is the canonical order, so the result is the same to the bit as with a
-// wavefront per slice.
-__device__ __forceinline__ void split_tile(const PreparedArgs &a, const KindArgs &k, int e,
-                                           int s_lo, int s_hi, const uint32_t *tab,
-                                           const uint32_t *xa, uint16_t *dst, int mode) {
-  float2 *part = reinterpret_cast<float2 *>(const_cast<uint32_t *>(xa) + a.xdwords);
-  const int waves = blockDim.x >> 6;
-  const int wave = threadIdx.x >> 6;
+// wavefront per slice.  Built for latency: split_begin puts the loads of a
+// whole group in flight, and the kernel calls it before it waits for and
+// stages the activations.
+struct SplitWalk {
+  Walk<kSplitRing> w;   // w.nch: this wavefront's last chunk + 1
+  int g_lo, g_hi, ngroups, colw;
+  int64_t sl;
+  bool mine;
+};
+
+// Everything but len, colw and the ring is the same in all lanes and is kept
+// in scalar registers (the wavefront index goes through readfirstlane).  The
+// ring loads are unconditional, with the chunk index clamped to the wavefront's
+// last chunk, so that they all leave at once.
+__device__ __forceinline__ SplitWalk split_begin(const PreparedArgs &a, const KindArgs &k, int e,
+                                                 int s0, int s_hi) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
-  const int per_pass = waves / k.split;      // slices a pass of the workgroup covers
   const int sub = wave % k.split;
+  const int s = s0 + wave / k.split;
+  SplitWalk r;
+  r.mine = s < s_hi;
+  r.ngroups = 0;
+  r.g_lo = 0;
+  r.g_hi = 0;
+  r.colw = 0;
+  r.sl = static_cast<int64_t>(e) * k.slices + s;
+  if (r.mine) {
+    const int nch_all = __builtin_amdgcn_readfirstlane(k.slice_nch[r.sl]);
+    r.ngroups = (nch_all + kGroupChunks - 1) / kGroupChunks;
+    r.g_lo = sub * r.ngroups / k.split;
+    r.g_hi = (sub + 1) * r.ngroups / k.split;
+    if (sub == 0) {   // the wavefront that will write the slice's rows
+      r.w.ridx = k.row_idx[r.sl * 64 + lane];
+      r.w.minmax = k.minmax[r.sl * 64 + lane];
+    }
+    if (r.g_lo < r.g_hi) {
+      const uint32_t base = __builtin_amdgcn_readfirstlane(k.slice_base[r.sl]);
+      r.w.nfull = __builtin_amdgcn_readfirstlane(k.slice_nfull[r.sl]);
+      r.w.len = k.row_len[r.sl * 64 + lane];
+      r.w.p = reinterpret_cast<const uint2 *>(a.codes + static_cast<int64_t>(base) * 256) + lane;
+      const int c_lo = r.g_lo * kGroupChunks;
+      r.w.nch = min(r.g_hi * kGroupChunks, nch_all);
+      if (r.g_lo)
+        r.colw = a.ckpt[(checkpoint_entry(base, k.first_slice + r.sl) + r.g_lo) * 64 + lane];
+#pragma unroll
+      for (int i = 0; i < kSplitRing; i++)
+        r.w.ring[i] = r.w.p[min(c_lo + i, r.w.nch - 1) * 64];
+    }
+  }
+  return r;
+}
+
+// The groups of a tile; contains a workgroup barrier.  A wavefront that
+// has its slice to itself (split 1) adds the groups in registers, in the same
+// order, and leaves the partial-sum area alone.
+__device__ __forceinline__ void split_run(const PreparedArgs &a, const KindArgs &k, SplitWalk &r,
+                                          const uint32_t *tab, const uint32_t *xa, uint16_t *dst,
+                                          int mode) {
+  float2 *part = reinterpret_cast<float2 *>(const_cast<uint32_t *>(xa) + a.xdwords);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
   const int local = wave / k.split;
+  const bool alone = k.split == 1;
   const DotConsts dk = dot_consts();
   const uint32_t shift2 = static_cast<uint32_t>(a.group_shift) * 0x00010001u;
-  for (int s0 = s_lo; s0 < s_hi; s0 += per_pass) {
-    const int s = s0 + local;
-    const bool mine = s < s_hi && local < per_pass;
-    const int64_t sl = static_cast<int64_t>(e) * k.slices + s;
-    int ngroups = 0;
-    if (mine) {
-      const int nch_all = __builtin_amdgcn_readfirstlane(k.slice_nch[sl]);
-      ngroups = (nch_all + kGroupChunks - 1) / kGroupChunks;
-      const int g_lo = sub * ngroups / k.split;
-      const int g_hi = (sub + 1) * ngroups / k.split;
-      if (g_lo < g_hi) {
-        SliceWalk w;
-        const uint32_t base = k.slice_base[sl];
-        w.nfull = __builtin_amdgcn_readfirstlane(k.slice_nfull[sl]);
-        w.len = k.row_len[sl * 64 + lane];
-        w.p = reinterpret_cast<const uint2 *>(a.codes + static_cast<int64_t>(base) * 256) + lane;
-        const int c_lo = g_lo * kGroupChunks;
-        w.nch = min(g_hi * kGroupChunks, nch_all);   // this wavefront's last chunk + 1
-        int colw = 0;
-        if (g_lo)
-          colw = a.ckpt[(checkpoint_entry(base, k.first_slice + sl) + g_lo) * 64 + lane];
-#pragma unroll
-        for (int i = 0; i < kRing; i++)
-          if (c_lo + i < w.nch) w.ring[i] = w.p[(c_lo + i) * 64];
-        for (int g = g_lo; g < g_hi; g++) {
-          float p1 = 0.f, p2 = 0.f;
-          const int c_end = min((g + 1) * kGroupChunks, w.nch);
-          for (int c = g * kGroupChunks; c < c_end; c += kRing) {
-            if (c + kRing <= w.nfull)
-              run_chunks<false>(w, c, shift2, tab, xa, colw, p1, p2, dk);
-            else
-              run_chunks<true>(w, c, shift2, tab, xa, colw, p1, p2, dk);
-          }
-          part[(local * k.groups_max + g) * 64 + lane] = make_float2(p1, p2);
-        }
-      }
+  int colw = r.colw;
+  float s1 = 0.f, s2 = 0.f;
+  for (int g = r.g_lo; g < r.g_hi; g++) {
+    float p1 = 0.f, p2 = 0.f;
+    const int c_end = min((g + 1) * kGroupChunks, r.w.nch);
+    for (int c = g * kGroupChunks; c < c_end; c += kSplitRing) {
+      if (c + kSplitRing <= r.w.nfull)
+        run_chunks<false>(r.w, c, shift2, tab, xa, colw, p1, p2, dk);
+      else
+        run_chunks<true>(r.w, c, shift2, tab, xa, colw, p1, p2, dk);
     }
-    __syncthreads();
-    if (mine && sub == 0) {
-      float s1 = 0.f, s2 = 0.f;
-      for (int g = 0; g < ngroups; g++) {
+    if (alone) {
+      s1 += p1;
+      s2 += p2;
+    } else {
+      part[(local * k.groups_max + g) * 64 + lane] = make_float2(p1, p2);
+    }
+  }
+  __syncthreads();
+  if (r.mine && wave % k.split == 0) {
+    if (!alone)
+      for (int g = 0; g < r.ngroups; g++) {
         float2 v = part[(local * k.groups_max + g) * 64 + lane];
         s1 += v.x;
         s2 += v.y;
       }
-      write_row(dst, k.row_idx[sl * 64 + lane], k.minmax[sl * 64 + lane], s1, s2, mode);
+    write_row(dst, r.w.ridx, r.w.minmax, s1, s2, mode);
+  }
+}
+
+// A wo tile waits until its token's wi tiles have published h (bounded spin of
+// one lane, then a barrier that extends its acquire to the workgroup); then the
+// tile's activations go into LDS.  Ends with a barrier.
+__device__ __forceinline__ void await_activations(const PreparedArgs &a, const KindArgs &k,
+                                                  int kind, int t, uint32_t *xa) {
+  if (kind == 1) {
+    if (threadIdx.x == 0) {
+      int spins = 0;
+      while (__hip_atomic_load(&a.ctrl[kCtrlHeader + t], __ATOMIC_ACQUIRE,
+                               __HIP_MEMORY_SCOPE_AGENT) < a.k[0].parts) {
+        if (++spins > a.spin_limit) {
+          __hip_atomic_fetch_add(&a.ctrl[1], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(8);
+      }
     }
     __syncthreads();
   }
+  const uint16_t *src = kind ? a.h + static_cast<int64_t>(t) * k.width
+                             : a.x + static_cast<int64_t>(t) * a.ldx;
+  stage_activations(xa, src, k.width);
+  __syncthreads();
+}
+
+// What a ticket stands for.  Every field is the same in all lanes.
+struct Tile {
+  int kind, t, s_lo, s_hi, e;   // e < 0: no matrix (token dropped or index out of range)
+};
+
+__device__ __forceinline__ Tile decode_tile(const PreparedArgs &a, int ticket, bool count_faults) {
+  const int n_wi = a.tokens * a.k[0].parts;
+  Tile tile;
+  tile.kind = ticket < n_wi ? 0 : 1;
+  const KindArgs &k = a.k[tile.kind];
+  const int rel = tile.kind ? ticket - n_wi : ticket;
+  tile.t = rel / k.parts;
+  const int part = rel - tile.t * k.parts;
+  // slices [s_lo, s_hi) of the matrix
+  tile.s_lo = static_cast<int>(static_cast<int64_t>(k.slices) * part / k.parts);
+  tile.s_hi = static_cast<int>(static_cast<int64_t>(k.slices) * (part + 1) / k.parts);
+  tile.e = a.token_expert ? __builtin_amdgcn_readfirstlane(a.token_expert[tile.t]) : 0;
+  if (tile.e >= a.experts) {
+    if (count_faults && tile.kind == a.kinds - 1 && part == 0 && threadIdx.x == 0)
+      __hip_atomic_fetch_add(&a.ctrl[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    tile.e = -1;
+  }
+  return tile;
+}
+
+// A dropped token keeps its input (reference sub1.py:312).
+__device__ __forceinline__ void pass_through(const PreparedArgs &a, const KindArgs &k, int t,
+                                             int s_lo, int s_hi) {
+  const int r_lo = min(64 * s_lo, k.height), r_hi = min(64 * s_hi, k.height);
+  for (int i = r_lo + threadIdx.x; i < r_hi; i += blockDim.x)
+    a.y[static_cast<int64_t>(t) * a.ldy + i] = a.x[static_cast<int64_t>(t) * a.ldx + i];
+}
+
+__device__ __forceinline__ uint16_t *tile_output(const PreparedArgs &a, const KindArgs &k,
+                                                 int kind, int t, int &mode) {
+  if (a.kinds == 2 && kind == 0) {
+    mode = kStoreRelu;
+    return a.h + static_cast<int64_t>(t) * k.height;
+  }
+  mode = a.kinds == 2 ? kStore : kAccumulate;
+  return a.y + static_cast<int64_t>(t) * a.ldy;
+}
+
+// h of a token's wi tile becomes visible to the wo tiles: every wavefront
+// drains its own stores, the barrier collects them, one release publishes.
+__device__ __forceinline__ void publish_h(const PreparedArgs &a, int t) {
+  sub1::drain_stores();
+  __syncthreads();
+  if (threadIdx.x == 0)
+    __hip_atomic_fetch_add(&a.ctrl[kCtrlHeader + t], 1, __ATOMIC_RELEASE,
+                           __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Persistent grid.  A tile is (token, projection, part): the slices of one
@@ -565,20 +726,21 @@ __device__ __forceinline__ void split_tile(const PreparedArgs &a, const KindArgs
 // fence costs an L2 write-back on this part, which is why the lanes do not fence
 // individually.
 __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs a) {
-  extern __shared__ uint32_t lds[];
+  extern __shared__ __align__(16) uint32_t lds[];
   __shared__ int s_ticket;
   uint32_t *tab = lds;
   uint32_t *xa = lds + a.table_words;
   const int threads = blockDim.x;
   const int waves = threads >> 6;
-  for (int i = threadIdx.x; i < a.table_words; i += threads) tab[i] = a.table[i];
+  stage_table(tab, a.table, a.table_words);
   const int n_wi = a.tokens * a.k[0].parts;
   const int n_all = n_wi + (a.kinds == 2 ? a.tokens * a.k[1].parts : 0);
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const bool dynamic = a.ctrl != nullptr;
   // dynamic order: thread 0 keeps one ticket ahead so that the atomic's round
   // trip overlaps a tile; static order: tile = workgroup index + k * grid
-  int next_ticket = blockIdx.x;
+  int static_ticket = blockIdx.x;   // the same in every lane, unlike thread 0's next_ticket
+  int next_ticket = 0;
   if (dynamic && threadIdx.x == 0)
     next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
                                          __HIP_MEMORY_SCOPE_AGENT);
@@ -593,89 +755,80 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
                                                __HIP_MEMORY_SCOPE_AGENT);
       }
       __syncthreads();
-      ticket = s_ticket;
+      ticket = __builtin_amdgcn_readfirstlane(s_ticket);   // the same in every lane: scalar
     } else {
-      ticket = next_ticket;
-      next_ticket += gridDim.x;
+      ticket = static_ticket;
+      static_ticket += gridDim.x;
     }
     if (ticket >= n_all) break;
-    const int kind = ticket < n_wi ? 0 : 1;
+    const Tile tile = decode_tile(a, ticket, dynamic);
+    const int kind = tile.kind, t = tile.t, s_lo = tile.s_lo, s_hi = tile.s_hi, e = tile.e;
     const KindArgs &k = a.k[kind];
-    const int rel = kind ? ticket - n_wi : ticket;
-    const int t = rel / k.parts;
-    const int part = rel - t * k.parts;
-    // slices [s_lo, s_hi) of the matrix
-    const int s_lo = static_cast<int>(static_cast<int64_t>(k.slices) * part / k.parts);
-    const int s_hi = static_cast<int>(static_cast<int64_t>(k.slices) * (part + 1) / k.parts);
-    int e = a.token_expert ? a.token_expert[t] : 0;
-    if (e >= a.experts) {
-      if (dynamic && kind == a.kinds - 1 && part == 0 && threadIdx.x == 0)
-        __hip_atomic_fetch_add(&a.ctrl[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      e = -1;
-    }
     if (a.kinds == 2 && kind == 1 && e < 0) {
-      // a dropped token keeps its input (reference sub1.py:312)
-      const int r_lo = min(64 * s_lo, k.height), r_hi = min(64 * s_hi, k.height);
-      for (int i = r_lo + threadIdx.x; i < r_hi; i += threads)
-        a.y[static_cast<int64_t>(t) * a.ldy + i] = a.x[static_cast<int64_t>(t) * a.ldx + i];
+      pass_through(a, k, t, s_lo, s_hi);
       continue;
     }
     if (e >= 0) {
-      // the first slice's loads go out before the wait and the staging
-      int s = s_lo + wave;
-      SliceWalk cur;
-      if (k.split == 1 && s < s_hi)
-        cur = load_slice(a, k, static_cast<int64_t>(e) * k.slices + s);
-      if (kind == 1) {
-        if (threadIdx.x == 0) {
-          int spins = 0;
-          while (__hip_atomic_load(&a.ctrl[kCtrlHeader + t], __ATOMIC_ACQUIRE,
-                                   __HIP_MEMORY_SCOPE_AGENT) < a.k[0].parts) {
-            if (++spins > a.spin_limit) {
-              __hip_atomic_fetch_add(&a.ctrl[1], 1, __ATOMIC_RELAXED,
-                                     __HIP_MEMORY_SCOPE_AGENT);
-              break;
-            }
-            __builtin_amdgcn_s_sleep(8);
-          }
-        }
-        __syncthreads();  // thread 0's acquire now covers the whole workgroup
-      }
-      const uint16_t *src = kind ? a.h + static_cast<int64_t>(t) * k.width
-                                 : a.x + static_cast<int64_t>(t) * a.ldx;
-      stage_activations(xa, src, k.width);
-      __syncthreads();
-      uint16_t *dst;
       int mode;
-      if (a.kinds == 2 && kind == 0) {
-        dst = a.h + static_cast<int64_t>(t) * k.height;
-        mode = kStoreRelu;
-      } else {
-        dst = a.y + static_cast<int64_t>(t) * a.ldy;
-        mode = a.kinds == 2 ? kStore : kAccumulate;
-      }
-      if (k.split > 1) {
-        split_tile(a, k, e, s_lo, s_hi, tab, xa, dst, mode);
-        s = s_hi;
-      }
-      for (; s < s_hi; s += waves) {
-        const bool more = s + waves < s_hi;
-        SliceWalk nxt;
-        if (more) nxt = load_slice(a, k, static_cast<int64_t>(e) * k.slices + s + waves);
-        float s1, s2;
-        run_slice(cur, a.group_shift, tab, xa, s1, s2);
-        write_row(dst, cur.ridx, cur.minmax, s1, s2, mode);
-        if (more) cur = nxt;
+      uint16_t *dst = tile_output(a, k, kind, t, mode);
+      // the first loads of the codes go out before the wait and the staging
+      {
+        int s = s_lo + wave;
+        SliceWalk cur;
+        if (s < s_hi) cur = load_slice(a, k, static_cast<int64_t>(e) * k.slices + s);
+        await_activations(a, k, kind, t, xa);
+        for (; s < s_hi; s += waves) {
+          const bool more = s + waves < s_hi;
+          SliceWalk nxt;
+          if (more) nxt = load_slice(a, k, static_cast<int64_t>(e) * k.slices + s + waves);
+          float s1, s2;
+          run_slice(cur, a.group_shift, tab, xa, s1, s2);
+          write_row(dst, cur.ridx, cur.minmax, s1, s2, mode);
+          if (more) cur = nxt;
+        }
       }
     }
-    if (a.kinds == 2 && kind == 0) {
-      sub1::drain_stores();   // this wavefront's h stores are in L2 ...
-      __syncthreads();        // ... so are everyone's, and thread 0's release publishes them
-      if (threadIdx.x == 0)
-        __hip_atomic_fetch_add(&a.ctrl[kCtrlHeader + t], 1, __ATOMIC_RELEASE,
-                               __HIP_MEMORY_SCOPE_AGENT);
-    }
+    if (a.kinds == 2 && kind == 0) publish_h(a, t);
   }
+}
+
+// One tile per workgroup, for the batches too small to occupy the GPU with a
+// wavefront per slice: built for latency.  `split` wavefronts share a slice
+// (split_begin / split_run), all of a wavefront's loads leave before anything
+// waits, and nothing loops.  Tiles are taken by ticket like in the persistent
+// kernel, so a wo tile's wait for its token's wi tiles ends for the same reason.
+__global__ __launch_bounds__(kMaxThreads) void moe_prepared_small_kernel(PreparedArgs a) {
+  extern __shared__ __align__(16) uint32_t lds[];
+  __shared__ int s_ticket;
+  uint32_t *tab = lds;
+  uint32_t *xa = lds + a.table_words;
+  const bool dynamic = a.ctrl != nullptr;
+  int ticket = blockIdx.x;
+  if (dynamic && threadIdx.x == 0)
+    s_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  stage_table(tab, a.table, a.table_words);
+  if (dynamic) {
+    __syncthreads();
+    ticket = __builtin_amdgcn_readfirstlane(s_ticket);
+  }
+  const int n_all = a.tokens * (a.k[0].parts + (a.kinds == 2 ? a.k[1].parts : 0));
+  if (ticket >= n_all) return;
+  const Tile tile = decode_tile(a, ticket, dynamic);
+  const int kind = tile.kind, t = tile.t, e = tile.e;
+  const KindArgs &k = a.k[kind];
+  if (a.kinds == 2 && kind == 1 && e < 0) {
+    pass_through(a, k, t, tile.s_lo, tile.s_hi);
+    return;
+  }
+  if (e >= 0) {
+    int mode;
+    uint16_t *dst = tile_output(a, k, kind, t, mode);
+    // the launch cuts the matrices so that a tile has at most waves / split slices
+    SplitWalk walk = split_begin(a, k, e, tile.s_lo, tile.s_hi);
+    await_activations(a, k, kind, t, xa);
+    split_run(a, k, walk, tab, xa, dst, mode);
+  }
+  if (a.kinds == 2 && kind == 0) publish_h(a, t);
 }
 
 // ------------------------------------------------------ per-device tables --
@@ -911,6 +1064,77 @@ int prepare_codes(const Source &src, const Prepared &p, hipStream_t s, const cha
 
 // Launch of the prepared kernel.  kinds == 2: y = wo(relu(wi x)) per token,
 // workspace required; kinds == 1: y += W x per token, no workspace.
+// Cut of the matrices for a batch that cannot occupy the GPU with a wavefront
+// per slice.  Per projection: a workgroup takes per_wg slices (16 = no sharing)
+// and waves / per_wg wavefronts share each slice, at most one per 32-code group.
+// The choice minimises an estimate of the kernel time in microseconds: a round
+// of workgroups costs a fixed part (table, activations, first loads: they do
+// not overlap with the previous round, LDS admits one workgroup per compute
+// unit) plus the groups that the busiest SIMD walks one after the other.
+// Sets split and parts of every projection; returns the LDS bytes for partial
+// sums, 0 if sharing nothing is estimated best (then nothing is changed).
+// The two constants come from timing every cut of the Switch base and c-2048
+// layers at 1 to 64 tokens on an MI355X.
+constexpr double kRoundFixedUs = 8.0;   // a round of workgroups before its first codeword
+constexpr double kGroupUs = 1.5;        // one 32-code group on a SIMD
+size_t plan_small(PreparedArgs &a, int kinds, int tokens, int cus, int waves, size_t lds_room) {
+  struct Option {
+    int split, parts;
+    int64_t tiles;
+    double round_us;
+    size_t partials;
+  };
+  Option opt[2][5];
+  int nopt[2] = {0, 0};
+  for (int i = 0; i < kinds; i++) {
+    const KindArgs &k = a.k[i];
+    int groups_pow2 = 1;
+    while (groups_pow2 < k.groups_max) groups_pow2 *= 2;
+    for (int per_wg = 1; per_wg <= waves; per_wg *= 2) {
+      Option o;
+      o.split = waves / per_wg < groups_pow2 ? waves / per_wg : groups_pow2;
+      o.partials = o.split > 1 ? static_cast<size_t>(per_wg) * k.groups_max * 512 : 0;
+      if (o.partials > lds_room) continue;
+      if (o.split == 1 && per_wg != waves) continue;
+      o.parts = (k.slices + per_wg - 1) / per_wg;
+      o.tiles = static_cast<int64_t>(tokens) * o.parts;
+      const int busy = per_wg * (o.split < k.groups_max ? o.split : k.groups_max);
+      const int serial = ((busy + 3) / 4) * ((k.groups_max + o.split - 1) / o.split);
+      o.round_us = kRoundFixedUs + kGroupUs * serial;
+      opt[i][nopt[i]++] = o;
+    }
+  }
+  double best = 1e30;
+  int pick[2] = {-1, -1};
+  for (int i0 = 0; i0 < nopt[0]; i0++)
+    for (int i1 = 0; i1 < (kinds == 2 ? nopt[1] : 1); i1++) {
+      const Option &o0 = opt[0][i0];
+      double us = std::max(1.0, static_cast<double>(o0.tiles) / cus) * o0.round_us;
+      if (kinds == 2) {
+        const Option &o1 = opt[1][i1];
+        // wo workgroups that found a free compute unit at the start have their
+        // fixed part behind them when h arrives
+        const bool resident = o0.tiles + o1.tiles <= cus;
+        us += std::max(1.0, static_cast<double>(o1.tiles) / cus) * o1.round_us -
+              (resident ? kRoundFixedUs : 0.0);
+      }
+      if (us < best) {
+        best = us;
+        pick[0] = i0;
+        pick[1] = i1;
+      }
+    }
+  size_t partials = 0;
+  for (int i = 0; i < kinds; i++)
+    if (opt[i][pick[i]].partials > partials) partials = opt[i][pick[i]].partials;
+  if (partials == 0) return 0;
+  for (int i = 0; i < kinds; i++) {
+    a.k[i].split = opt[i][pick[i]].split;
+    a.k[i].parts = opt[i][pick[i]].parts;
+  }
+  return partials;
+}
+
 int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *x, int64_t ldx,
                     void *y, int64_t ldy, int tokens, void *workspace, int64_t workspace_bytes,
                     hipStream_t s, const char *who) {
@@ -983,7 +1207,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   }
   a.tokens = tokens;
   a.experts = p.count;
-  a.table_words = t->words;
+  a.table_words = (t->words + 3) & ~3;   // the device copy is zero-padded to the maximum
   a.single_codes = t->single_codes;
   a.group_shift = t->single_codes - t->single_codes / 8;
   a.xdwords = activation_dwords(wmax);
@@ -992,13 +1216,14 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   const size_t lds_base = (static_cast<size_t>(a.table_words) + a.xdwords) * 4;
   if (lds_base > lds_limit) return fail(SUB1_ERR_SHAPE, "%s: width %d does not fit LDS", who, wmax);
   // Tiles.  Whole matrices when the tokens alone keep every compute unit busy;
-  // otherwise each matrix is cut into parts, down to one slice per wavefront;
-  // and when even that leaves compute units idle (a handful of tokens), several
-  // wavefronts share a slice, each starting from a column checkpoint.
+  // otherwise each matrix is cut into parts, down to one slice per wavefront
+  // (the persistent kernel).  When even that leaves compute units idle (a
+  // handful of tokens), the other kernel runs: a workgroup takes fewer slices
+  // (8, 4, 2 or 1) and the wavefronts this frees share the slices, each
+  // starting from a column checkpoint.  plan_small picks the cut by estimate.
   const int want = (cus + tokens - 1) / tokens;   // tiles per token and projection
-  size_t lds_partials = 0;
   int64_t first_slice = 0;
-  int64_t tiles = 0;
+  bool idle_units = false;
   for (int i = 0; i < p.kinds; i++) {
     KindArgs &k = a.k[i];
     k.first_slice = first_slice;
@@ -1007,34 +1232,32 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     k.split = 1;
     const int max_parts = (k.slices + waves - 1) / waves;
     k.parts = want > max_parts ? max_parts : want;
-    if (want > max_parts) {
-      int split = 1;
-      while (split * 2 <= waves && split * 2 <= k.groups_max &&
-             (k.slices + waves / split - 1) / (waves / split) < want)
-        split *= 2;
-      while (split > 1 &&
-             lds_base + static_cast<size_t>(waves / split) * k.groups_max * 512 > lds_limit)
-        split /= 2;
-      if (split > 1) {
-        k.split = split;
-        k.parts = (k.slices + waves / split - 1) / (waves / split);
-        size_t need = static_cast<size_t>(waves / split) * k.groups_max * 512;
-        if (need > lds_partials) lds_partials = need;
-      }
-    }
-    tiles += static_cast<int64_t>(tokens) * k.parts;
+    if (want > max_parts) idle_units = true;
   }
+  size_t lds_partials = 0;
+  if (idle_units) lds_partials = plan_small(a, p.kinds, tokens, cus, waves, lds_limit - lds_base);
+  const bool small = lds_partials != 0;
+  int64_t tiles = 0;
+  for (int i = 0; i < p.kinds; i++) tiles += static_cast<int64_t>(tokens) * a.k[i].parts;
   if (tiles > INT32_MAX - (1 << 20)) return fail(SUB1_ERR_SHAPE, "%s: too many tiles", who);
   const size_t lds = lds_base + lds_partials;
-  HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(moe_prepared_kernel),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-  int64_t grid = cus;  // one workgroup per compute unit (LDS holds the table once)
-  if (grid > tiles) grid = tiles;
+  // Batches too small to occupy the GPU with a wavefront per slice go to the
+  // one-tile-per-workgroup kernel, everything else to the persistent one with
+  // a workgroup per compute unit (LDS holds the table once).
+  const void *fn = small ? reinterpret_cast<const void *>(moe_prepared_small_kernel)
+                         : reinterpret_cast<const void *>(moe_prepared_kernel);
+  HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(lds)));
   if (a.ctrl) {
     int nctrl = kCtrlHeader + tokens;
     zero_words_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl);
   }
-  moe_prepared_kernel<<<static_cast<unsigned>(grid), 64 * waves, lds, s>>>(a);
+  if (small) {
+    moe_prepared_small_kernel<<<static_cast<unsigned>(tiles), 64 * waves, lds, s>>>(a);
+  } else {
+    const int64_t grid = tiles < cus ? tiles : cus;
+    moe_prepared_kernel<<<static_cast<unsigned>(grid), 64 * waves, lds, s>>>(a);
+  }
   HIP_TRY(hipGetLastError());
   return SUB1_OK;
 }
