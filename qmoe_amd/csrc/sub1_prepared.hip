@@ -307,6 +307,7 @@ struct PreparedArgs {
   int tokens, experts;
   int table_words, single_codes, group_shift;  // group_shift = single_codes - single_codes/8
   int xdwords;                                 // LDS dwords reserved for the activations
+  int hdwords;                                 // fused kernel: LDS dwords of h (wo's activations)
   int spin_limit;
 };
 
@@ -792,6 +793,89 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
   }
 }
 
+// Streaming form for batches of at least one token per compute unit: a tile is
+// a token, and the workgroup runs wi, ReLU and wo back to back with h kept in
+// LDS, already in the layout wo reads its activations from.  No workspace
+// traffic for h, no waiting between workgroups; tickets only balance the load.
+// LDS: table | x (wi's activations) | h (wo's activations).
+__global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(PreparedArgs a) {
+  extern __shared__ __align__(16) uint32_t lds[];
+  __shared__ int s_ticket;
+  uint32_t *tab = lds;
+  uint32_t *xa = lds + a.table_words;
+  uint32_t *ha = xa + a.xdwords;
+  const int threads = blockDim.x;
+  const int waves = threads >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const KindArgs &ki = a.k[0];
+  const KindArgs &ko = a.k[1];
+  stage_table(tab, a.table, a.table_words);
+  // h: the lanes overwrite the two value dwords of their rows; the empty slots
+  // and the columns past d_ff stay zero for the whole launch
+  for (int i = threadIdx.x; i < a.hdwords; i += threads) ha[i] = 0u;
+  int next_ticket = 0;
+  if (threadIdx.x == 0)
+    next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+  for (;;) {
+    __syncthreads();   // the previous token's wo has read h; s_ticket is free
+    if (threadIdx.x == 0) {
+      s_ticket = next_ticket;
+      if (next_ticket < a.tokens)
+        next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    const int t = __builtin_amdgcn_readfirstlane(s_ticket);
+    if (t >= a.tokens) break;
+    int e = __builtin_amdgcn_readfirstlane(a.token_expert[t]);
+    if (e >= a.experts) {
+      if (threadIdx.x == 0)
+        __hip_atomic_fetch_add(&a.ctrl[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      e = -1;
+    }
+    if (e < 0) {
+      pass_through(a, ko, t, 0, ko.slices);
+      continue;
+    }
+    // wi: x -> relu(h) into LDS
+    int s = wave;
+    SliceWalk cur;
+    if (s < ki.slices) cur = load_slice(a, ki, static_cast<int64_t>(e) * ki.slices + s);
+    stage_activations(xa, a.x + static_cast<int64_t>(t) * a.ldx, ki.width);
+    __syncthreads();
+    for (; s < ki.slices; s += waves) {
+      const bool more = s + waves < ki.slices;
+      SliceWalk nxt;
+      if (more) nxt = load_slice(a, ki, static_cast<int64_t>(e) * ki.slices + s + waves);
+      float s1, s2;
+      run_slice(cur, a.group_shift, tab, xa, s1, s2);
+      if (cur.ridx != 0xffff) {
+        uint32_t out = f32_to_bf16(row_result(cur.minmax, s1, s2));
+        if (out & 0x8000u) out = 0;   // relu between the projections, on the bf16 value
+        uint32_t *p = ha + 6 * (cur.ridx >> 1) + 2 * (cur.ridx & 1);
+        p[0] = out;
+        p[1] = out << 16;
+      }
+      if (more) cur = nxt;
+    }
+    // wo: h -> y; its first loads go out before the barrier
+    s = wave;
+    if (s < ko.slices) cur = load_slice(a, ko, static_cast<int64_t>(e) * ko.slices + s);
+    __syncthreads();
+    uint16_t *dst = a.y + static_cast<int64_t>(t) * a.ldy;
+    for (; s < ko.slices; s += waves) {
+      const bool more = s + waves < ko.slices;
+      SliceWalk nxt;
+      if (more) nxt = load_slice(a, ko, static_cast<int64_t>(e) * ko.slices + s + waves);
+      float s1, s2;
+      run_slice(cur, a.group_shift, tab, ha, s1, s2);
+      write_row(dst, cur.ridx, cur.minmax, s1, s2, kStore);
+      if (more) cur = nxt;
+    }
+  }
+}
+
 // One tile per workgroup, for the batches too small to occupy the GPU with a
 // wavefront per slice: built for latency.  `split` wavefronts share a slice
 // (split_begin / split_run), all of a wavefront's loads leave before anything
@@ -1211,6 +1295,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   a.single_codes = t->single_codes;
   a.group_shift = t->single_codes - t->single_codes / 8;
   a.xdwords = activation_dwords(wmax);
+  a.hdwords = 0;
   a.spin_limit = 1 << 24;
   const size_t lds_limit = 160 * 1024 - 64;
   const size_t lds_base = (static_cast<size_t>(a.table_words) + a.xdwords) * 4;
@@ -1240,6 +1325,24 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   int64_t tiles = 0;
   for (int i = 0; i < p.kinds; i++) tiles += static_cast<int64_t>(tokens) * a.k[i].parts;
   if (tiles > INT32_MAX - (1 << 20)) return fail(SUB1_ERR_SHAPE, "%s: too many tiles", who);
+  // At least a token per compute unit: a workgroup takes whole tokens and keeps
+  // h in LDS, if table + x + h fit.
+  const size_t lds_fused = (static_cast<size_t>(a.table_words) + activation_dwords(a.k[0].width) +
+                            activation_dwords(a.k[1].width)) * 4;
+  const bool fused = p.kinds == 2 && !small && a.k[0].parts == 1 && a.k[1].parts == 1 &&
+                     lds_fused <= lds_limit;
+  if (fused) {
+    a.xdwords = activation_dwords(a.k[0].width);
+    a.hdwords = activation_dwords(a.k[1].width);
+    const void *fn = reinterpret_cast<const void *>(moe_prepared_fused_kernel);
+    HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(lds_fused)));
+    zero_words_kernel<<<1, 256, 0, s>>>(a.ctrl, kCtrlHeader);
+    const int grid = tokens < cus ? tokens : cus;
+    moe_prepared_fused_kernel<<<grid, 64 * waves, lds_fused, s>>>(a);
+    HIP_TRY(hipGetLastError());
+    return SUB1_OK;
+  }
   const size_t lds = lds_base + lds_partials;
   // Batches too small to occupy the GPU with a wavefront per slice go to the
   // one-tile-per-workgroup kernel, everything else to the persistent one with

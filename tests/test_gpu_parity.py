@@ -373,9 +373,10 @@ def test_routed_batch_equals_per_token_products(gpu):
 
 
 def test_every_tiling_mode_gives_the_same_bits(gpu, oracle):
-    """The prepared kernel tiles differently with the batch size: whole
-    matrices per workgroup (many tokens), parts of a matrix (fewer), several
-    wavefronts sharing one row slice from column checkpoints (a handful).
+    """The prepared kernels tile differently with the batch size: a token
+    with both its matrices per workgroup (many tokens), whole matrices or
+    parts of a matrix (fewer), several wavefronts sharing one row slice from
+    column checkpoints (a handful).
     The same token must come out identical in all of them, and equal to the
     oracle."""
     from qmoe_amd import synthetic
@@ -400,6 +401,32 @@ def test_every_tiling_mode_gives_the_same_bits(gpu, oracle):
         assert torch.equal(y[0], want), tokens
         if tokens > 1:
             assert torch.equal(y[1], y[tokens - 1])
+
+
+def test_token_per_workgroup_tiles_with_dropped_tokens(gpu, oracle):
+    """At least one token per compute unit: a workgroup then runs both
+    projections of a token with the intermediate activations kept on chip.
+    Dropped tokens pass through, out-of-range expert ids are counted, and the
+    rest equals the small-batch result of the same tokens."""
+    from qmoe_amd import synthetic
+    experts, d_model, d_ff, tokens = 5, 1024, 4096, 520
+    stack = synthetic.build_stack(experts, d_model, d_ff, 0.88, seed=21)
+    prep = stack.prepare()
+    x = synthetic.activations(tokens, d_model, seed=22)
+    route = (torch.arange(tokens, dtype=torch.int32, device='cuda') * 7) % experts
+    route[3] = -1
+    route[400] = -1
+    route[77] = experts
+    route[519] = experts + 100
+    y = prep.forward(x, route)
+    assert prep.launch_faults(tokens) == (0, 2)
+    for t in (3, 400, 77, 519):
+        assert torch.equal(y[t], x[t])
+    keep = [0, 1, 2, 4, 5, 76, 78, 255, 256, 399, 401, 518]
+    idx = torch.tensor(keep, device='cuda')
+    small = prep.forward(x[idx].contiguous(), route[idx].contiguous())
+    assert torch.equal(y[idx], small)
+    assert torch.equal(y, stack.forward(x, route))
 
 
 @pytest.mark.parametrize('height,width,p0', SWITCH_SHAPES + [(77, 333, 0.7), (5, 1, 0.5),
