@@ -408,6 +408,10 @@ __device__ __forceinline__ void lookup2(const uint32_t *tab, uint32_t pair, uint
   uint32_t b_hi = (sym >> 16) * 0x4081u;
   e_lo = (w_lo & ~0x00010101u) | (b_lo & 0x00010101u);
   e_hi = (w_hi & ~0x00010101u) | (b_hi & 0x00010101u);
+  // one v_bfi each; the empty asm keeps the compiler from redoing the merge
+  // for every byte it later extracts
+  asm("" : "+v"(e_lo));
+  asm("" : "+v"(e_hi));
 }
 
 __device__ __forceinline__ void lookup4(const uint32_t *tab, uint2 w, uint32_t shift2,
@@ -428,13 +432,20 @@ __device__ __forceinline__ void add_codeword(uint32_t e, const uint32_t *xa, int
   colw += static_cast<int>(e >> 24);
 }
 
+// This lane's chunk 0 of the slice that starts at chunk `base` of the stream.
+__device__ __forceinline__ const uint2 *chunk_pointer(const uint16_t *codes, uint32_t base) {
+  return reinterpret_cast<const uint2 *>(codes + static_cast<int64_t>(base) * 256) +
+         (threadIdx.x & 63);
+}
+
 // What a lane needs to walk its row of one slice; load_slice issues the loads
 // of the first chunks, so calling it for the NEXT slice before walking the
 // current one hides their latency.
 template <int R>
 struct Walk {
-  const uint2 *p;
-  int nch, nfull, len, ridx;
+  uint32_t base;     // the slice's first chunk, in chunks; the same in every lane,
+  int nch, nfull;    // like the chunk counts
+  int len, ridx;
   uint32_t minmax;
   uint2 ring[R];
 };
@@ -449,27 +460,27 @@ __device__ __forceinline__ SliceWalk load_slice(const PreparedArgs &a, const Kin
   w.len = k.row_len[sl * 64 + lane];
   w.ridx = k.row_idx[sl * 64 + lane];
   w.minmax = k.minmax[sl * 64 + lane];
-  w.p = reinterpret_cast<const uint2 *>(a.codes + static_cast<int64_t>(k.slice_base[sl]) * 256) +
-        lane;
+  w.base = __builtin_amdgcn_readfirstlane(k.slice_base[sl]);
+  const uint2 *p = chunk_pointer(a.codes, w.base);
 #pragma unroll
-  for (int i = 0; i < kRing; i++)
-    if (i < w.nch) w.ring[i] = w.p[i * 64];
+  for (int i = 0; i < kRing; i++) w.ring[i] = p[min(i, w.nch - 1) * 64];
   return w;
 }
 
 // R chunks (the depth of the walk's ring) starting at chunk c added onto the
 // partial sums p1, p2.  kChecked: compare every code with the lane's own count.
 template <bool kChecked, int R>
-__device__ __forceinline__ void run_chunks(Walk<R> &w, int c, uint32_t shift2,
+__device__ __forceinline__ void run_chunks(Walk<R> &w, const uint2 *p, int c, uint32_t shift2,
                                            const uint32_t *tab, const uint32_t *xa, int &colw,
                                            float &p1, float &p2, const DotConsts &dk) {
-  const uint2 *p = w.p;
   const int nch = w.nch;
 #pragma unroll
   for (int i = 0; i < R; i++) {
     if (!kChecked || c + i < nch) {
       const uint2 cw = w.ring[i];
-      if (c + i + R < nch) w.ring[i] = p[(c + i + R) * 64];
+      // unconditional, clamped to the last chunk: the load can target the ring
+      // register itself and the loop needs no wait for it
+      w.ring[i] = p[min(c + i + R, nch - 1) * 64];
       uint32_t e[4];
       lookup4(tab, cw, shift2, e);
       const int j = kChunk * (c + i);
@@ -487,10 +498,17 @@ __device__ __forceinline__ void run_chunks(Walk<R> &w, int c, uint32_t shift2,
 // 32 codes (kGroupChunks chunks), a partial sum per group from zero, the
 // partial sums added first group first.  Starts at chunk c0 (a multiple of
 // kGroupChunks) with column offset colw and stops before chunk c_end.
-__device__ __forceinline__ void run_slice(SliceWalk &w, int group_shift, const uint32_t *tab,
+__device__ __forceinline__ void run_slice(SliceWalk &w, const uint16_t *codes, int group_shift,
+                                          const uint32_t *tab,
                                           const uint32_t *xa, float &s1, float &s2) {
   const DotConsts dk = dot_consts();
   const uint32_t shift2 = static_cast<uint32_t>(group_shift) * 0x00010001u;
+  // a walk that went through `cur = nxt` may sit in vector registers: put what
+  // is the same in all lanes back into scalar ones, for scalar loop control
+  // and scalar address arithmetic
+  w.nch = __builtin_amdgcn_readfirstlane(w.nch);
+  w.nfull = __builtin_amdgcn_readfirstlane(w.nfull);
+  const uint2 *p = chunk_pointer(codes, __builtin_amdgcn_readfirstlane(w.base));
   s1 = 0.f;
   s2 = 0.f;
   float p1 = 0.f, p2 = 0.f;
@@ -498,7 +516,7 @@ __device__ __forceinline__ void run_slice(SliceWalk &w, int group_shift, const u
   int c = 0;
   // chunks every lane of the slice has in full: no per-code checks
   for (; c + kRing <= w.nfull; c += kRing) {
-    run_chunks<false>(w, c, shift2, tab, xa, colw, p1, p2, dk);
+    run_chunks<false>(w, p, c, shift2, tab, xa, colw, p1, p2, dk);
     if ((c + kRing) % kGroupChunks == 0) {
       s1 += p1;
       s2 += p2;
@@ -507,7 +525,7 @@ __device__ __forceinline__ void run_slice(SliceWalk &w, int group_shift, const u
     }
   }
   for (; c < w.nch; c += kRing) {
-    run_chunks<true>(w, c, shift2, tab, xa, colw, p1, p2, dk);
+    run_chunks<true>(w, p, c, shift2, tab, xa, colw, p1, p2, dk);
     if ((c + kRing) % kGroupChunks == 0) {
       s1 += p1;
       s2 += p2;
@@ -568,6 +586,7 @@ __device__ __forceinline__ SplitWalk split_begin(const PreparedArgs &a, const Ki
   r.g_hi = 0;
   r.colw = 0;
   r.sl = static_cast<int64_t>(e) * k.slices + s;
+  r.w.base = 0;
   if (r.mine) {
     const int nch_all = __builtin_amdgcn_readfirstlane(k.slice_nch[r.sl]);
     r.ngroups = (nch_all + kGroupChunks - 1) / kGroupChunks;
@@ -581,14 +600,15 @@ __device__ __forceinline__ SplitWalk split_begin(const PreparedArgs &a, const Ki
       const uint32_t base = __builtin_amdgcn_readfirstlane(k.slice_base[r.sl]);
       r.w.nfull = __builtin_amdgcn_readfirstlane(k.slice_nfull[r.sl]);
       r.w.len = k.row_len[r.sl * 64 + lane];
-      r.w.p = reinterpret_cast<const uint2 *>(a.codes + static_cast<int64_t>(base) * 256) + lane;
+      r.w.base = base;
+      const uint2 *p = chunk_pointer(a.codes, base);
       const int c_lo = r.g_lo * kGroupChunks;
       r.w.nch = min(r.g_hi * kGroupChunks, nch_all);
       if (r.g_lo)
         r.colw = a.ckpt[(checkpoint_entry(base, k.first_slice + r.sl) + r.g_lo) * 64 + lane];
 #pragma unroll
       for (int i = 0; i < kSplitRing; i++)
-        r.w.ring[i] = r.w.p[min(c_lo + i, r.w.nch - 1) * 64];
+        r.w.ring[i] = p[min(c_lo + i, r.w.nch - 1) * 64];
     }
   }
   return r;
@@ -609,14 +629,15 @@ __device__ __forceinline__ void split_run(const PreparedArgs &a, const KindArgs 
   const uint32_t shift2 = static_cast<uint32_t>(a.group_shift) * 0x00010001u;
   int colw = r.colw;
   float s1 = 0.f, s2 = 0.f;
+  const uint2 *p = chunk_pointer(a.codes, r.w.base);
   for (int g = r.g_lo; g < r.g_hi; g++) {
     float p1 = 0.f, p2 = 0.f;
     const int c_end = min((g + 1) * kGroupChunks, r.w.nch);
     for (int c = g * kGroupChunks; c < c_end; c += kSplitRing) {
       if (c + kSplitRing <= r.w.nfull)
-        run_chunks<false>(r.w, c, shift2, tab, xa, colw, p1, p2, dk);
+        run_chunks<false>(r.w, p, c, shift2, tab, xa, colw, p1, p2, dk);
       else
-        run_chunks<true>(r.w, c, shift2, tab, xa, colw, p1, p2, dk);
+        run_chunks<true>(r.w, p, c, shift2, tab, xa, colw, p1, p2, dk);
     }
     if (alone) {
       s1 += p1;
@@ -783,7 +804,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
           SliceWalk nxt;
           if (more) nxt = load_slice(a, k, static_cast<int64_t>(e) * k.slices + s + waves);
           float s1, s2;
-          run_slice(cur, a.group_shift, tab, xa, s1, s2);
+          run_slice(cur, a.codes, a.group_shift, tab, xa, s1, s2);
           write_row(dst, cur.ridx, cur.minmax, s1, s2, mode);
           if (more) cur = nxt;
         }
@@ -849,7 +870,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
       SliceWalk nxt;
       if (more) nxt = load_slice(a, ki, static_cast<int64_t>(e) * ki.slices + s + waves);
       float s1, s2;
-      run_slice(cur, a.group_shift, tab, xa, s1, s2);
+      run_slice(cur, a.codes, a.group_shift, tab, xa, s1, s2);
       if (cur.ridx != 0xffff) {
         uint32_t out = f32_to_bf16(row_result(cur.minmax, s1, s2));
         if (out & 0x8000u) out = 0;   // relu between the projections, on the bf16 value
@@ -869,7 +890,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
       SliceWalk nxt;
       if (more) nxt = load_slice(a, ko, static_cast<int64_t>(e) * ko.slices + s + waves);
       float s1, s2;
-      run_slice(cur, a.group_shift, tab, ha, s1, s2);
+      run_slice(cur, a.codes, a.group_shift, tab, ha, s1, s2);
       write_row(dst, cur.ridx, cur.minmax, s1, s2, kStore);
       if (more) cur = nxt;
     }
