@@ -1,7 +1,8 @@
 """Module surface of the reference's `sub1.py` for the compressed-layer path:
 `setup`, the tables `dec`/`trie`, `GPUS`/`DEV`/`DEC`/`TRIE`, `Sub1Linear`
 (same buffers, `forward(x)`, static `make(w)`), plus `Sub1Experts`, the
-one-launch form of the expert loop in `FasterMLP.forward`.
+one-launch form of the expert loop, and `FasterMLP`, the sparse-MLP module the
+reference wraps around it (router, expert launch, router-probability scaling).
 
 Differences from the reference that a caller can observe:
   * importing works without a GPU (the reference indexes GPUS[-1] at import,
@@ -125,3 +126,72 @@ class Sub1Experts(nn.Module):
 
     def forward(self, x, expert_index):
         return self.stack.forward(x.contiguous(), expert_index.to(torch.int32).contiguous())
+
+
+def _router_outputs(outputs, experts):
+    """(one-hot routing mask [.., E], probabilities [.., 1], logits [.., E])
+    from a Switch top-1 router's 3-tuple, whatever its order: transformers
+    4.28 returns (mask, probs, logits) (reference sub1.py:310), later versions
+    put the probabilities first.  The probabilities are the entry whose last
+    dimension is 1; of the two [.., E] entries the mask is the integer one."""
+    probs = [o for o in outputs if o.shape[-1] == 1 and experts != 1]
+    wide = [o for o in outputs if o.shape[-1] == experts and not any(o is p for p in probs)]
+    if experts == 1:
+        wide = list(outputs)
+        floats = [o for o in wide if o.is_floating_point()]
+        mask = [o for o in wide if not o.is_floating_point()]
+        if len(mask) != 1 or len(floats) != 2:
+            raise ValueError('cannot tell the router outputs apart')
+        # with one expert the top-1 probability is softmax of one logit = 1
+        return mask[0], floats[0], floats[1]
+    mask = [o for o in wide if not o.is_floating_point()]
+    logits = [o for o in wide if o.is_floating_point()]
+    if len(probs) != 1 or len(mask) != 1 or len(logits) != 1:
+        raise ValueError('cannot tell the router outputs apart: shapes %s'
+                         % [tuple(o.shape) for o in outputs])
+    return mask[0], probs[0], logits[0]
+
+
+class FasterMLP(nn.Module):
+    """The sparse MLP of a Switch block around the compressed experts
+    (reference sub1.py:299-321): router, experts, multiplication by the router
+    probability.  `mlp` is the block's `SwitchTransformersSparseMLP`-shaped
+    module: `mlp.router` and `mlp.experts` (a ModuleDict of modules with
+    `wi`/`wo` Sub1Linear layers).
+
+    Differences from the reference: the experts run in one launch (built from
+    the layers' buffers on first use, rebuilt if they are replaced or written);
+    tokens stay on their GPU (one GPU here, the reference moves them to the
+    layer's GPU and back, sub1.py:307-320)."""
+
+    def __init__(self, mlp, gpu=None):
+        super().__init__()
+        if gpu is not None:
+            mlp = mlp.to(gpu)
+        self.router = mlp.router
+        self.experts = nn.ModuleList(mlp.experts.values())
+        self.gpu = gpu
+
+    def _launcher(self):
+        key = tuple((t.data_ptr(), t._version) for e in self.experts for l in (e.wi, e.wo)
+                    for t in (l.w_comp, l.row_off, l.ter_minmax))
+        cached = getattr(self, '_launcher_cache', None)
+        if cached is None or cached[0] != key:
+            stack = Sub1Experts([e.wi for e in self.experts], [e.wo for e in self.experts]).stack
+            cached = (key, stack.prepare() if stack.can_prepare() else stack)
+            self._launcher_cache = cached
+        return cached[1]
+
+    def forward(self, hidden_states):
+        """hidden_states [B, S, d_model] -> (router_probs * expert output,
+        (router_logits, expert_index)); tokens that the router's capacity
+        limit dropped keep their input (reference sub1.py:312-318)."""
+        router_mask, router_probs, router_logits = _router_outputs(
+            self.router(hidden_states), len(self.experts))
+        expert_index = torch.argmax(router_mask, dim=-1)
+        routed = router_mask.sum(dim=-1) > 0
+        route = torch.where(routed, expert_index, torch.full_like(expert_index, -1))
+        x = hidden_states.reshape(-1, hidden_states.shape[-1]).to(torch.bfloat16).contiguous()
+        next_states = self._launcher().forward(x, route.reshape(-1).to(torch.int32).contiguous())
+        hidden_states = router_probs * next_states.view(hidden_states.shape).to(hidden_states.dtype)
+        return hidden_states, (router_logits, expert_index)

@@ -206,6 +206,11 @@ class ExpertStack:
                 ws.numel(), _stream()))
         return y
 
+    def can_prepare(self):
+        """Whether the fast layout takes these shapes (it also wants the fixed
+        dictionary, which prepare() itself checks)."""
+        return max(self.d_model, self.d_ff) <= PREPARED_MAX_WIDTH
+
     def prepare(self):
         """The fast form of this stack (see PreparedStack); the stack itself
         is left as it is and is not referenced by the result."""

@@ -1,0 +1,118 @@
+"""The modules around the kernels: ternary front end -> make -> forward, and
+the sparse-MLP module (router, one-launch experts, probability scaling) against
+the reference's per-expert loop (sub1.py:306-321) restated with per-layer
+calls."""
+import types
+
+import pytest
+import torch
+import torch.nn as nn
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope='module')
+def gpu():
+    from qmoe_amd import sub1
+    assert torch.cuda.is_available(), 'these tests need the GPU'
+    assert sub1.DEC, 'device tables missing'
+    return sub1
+
+
+class Top1Router(nn.Module):
+    """Switch top-1 router with a capacity limit, as HuggingFace's
+    SwitchTransformersTop1Router computes it: fp32 softmax over a linear
+    classifier, one-hot of the argmax, tokens beyond an expert's capacity (in
+    sequence order) lose their expert.  `order` picks the tuple layout of
+    transformers 4.28 ('mask_first') or of later versions ('probs_first')."""
+
+    def __init__(self, d_model, experts, capacity, order):
+        super().__init__()
+        self.classifier = nn.Linear(d_model, experts, bias=False)
+        self.experts, self.capacity, self.order = experts, capacity, order
+
+    def forward(self, hidden):
+        logits = self.classifier(hidden.float())
+        probs = torch.softmax(logits, dim=-1)
+        index = torch.argmax(probs, dim=-1)
+        mask = torch.nn.functional.one_hot(index, self.experts)
+        priority = torch.cumsum(mask, dim=-2)
+        mask = mask * (priority <= self.capacity)
+        top = torch.max(probs, dim=-1).values.unsqueeze(-1).to(hidden.dtype)
+        if self.order == 'mask_first':
+            return mask, top, logits
+        return top, mask, logits
+
+
+class Expert(nn.Module):
+    def __init__(self, wi, wo):
+        super().__init__()
+        self.wi, self.wo = wi, wo
+
+    def forward(self, x):
+        return self.wo(torch.relu(self.wi(x)))
+
+
+def ternary_dense(h, w, p0, gen):
+    from qmoe_amd import synthetic
+    t = synthetic.draw_symbols(h, w, p0, gen, 'cuda')
+    mm = synthetic.draw_minmax(h, gen, 'cuda')
+    lut = torch.stack((torch.zeros(h, device='cuda', dtype=torch.bfloat16), mm[0::2], mm[1::2]), 1)
+    return torch.gather(lut, 1, t.long()).contiguous()
+
+
+def test_ternarize_make_forward(gpu):
+    from qmoe_amd import quant, sub1, sub1_hip
+    g = torch.Generator(device='cuda').manual_seed(31)
+    w = torch.randn((192, 320), generator=g, device='cuda') * 0.05
+    wq = quant.ternarize(w)
+    lin = sub1.Sub1Linear.make(wq)
+    dense = sub1_hip.sub1decode(sub1.DEC[0], lin.w_comp, lin.row_off, lin.ter_minmax, 320,
+                                want_tern=False)[1]
+    assert torch.equal(dense, wq.bfloat16())          # the packed layer holds exactly wq
+    x = torch.randn((5, 320), generator=g, device='cuda').bfloat16()
+    y = lin(x)
+    ref = x.float() @ wq.bfloat16().float().t()
+    assert torch.linalg.norm(y.float() - ref) <= 1e-2 * torch.linalg.norm(ref)
+    # compression: far below 2 bytes per weight
+    assert lin.w_comp.numel() * 2 < 0.2 * w.numel() * 2
+
+
+@pytest.mark.parametrize('order', ['mask_first', 'probs_first'])
+def test_faster_mlp_equals_the_expert_loop(gpu, order):
+    from qmoe_amd import sub1
+    d_model, d_ff, experts, batch, seq = 256, 512, 6, 2, 24
+    g = torch.Generator(device='cuda').manual_seed(41)
+    layers = nn.ModuleDict()
+    for e in range(experts):
+        wi = sub1.Sub1Linear.make(ternary_dense(d_ff, d_model, 0.85, g))
+        wo = sub1.Sub1Linear.make(ternary_dense(d_model, d_ff, 0.85, g))
+        layers['expert_%d' % e] = Expert(wi, wo)
+    router = Top1Router(d_model, experts, capacity=3, order=order).cuda()
+    with torch.no_grad():
+        router.classifier.weight.copy_(torch.randn((experts, d_model), generator=g, device='cuda'))
+    mlp = types.SimpleNamespace(router=router, experts=layers)
+    fast = sub1.FasterMLP(mlp)
+    hidden = torch.randn((batch, seq, d_model), generator=g, device='cuda').bfloat16()
+    out, (logits, index) = fast(hidden)
+
+    # the reference's loop, per expert, on the packed buffers
+    outs = router(hidden)
+    mask, probs = (outs[0], outs[1]) if order == 'mask_first' else (outs[1], outs[0])
+    assert int((mask.sum(-1) == 0).sum()) > 0            # the capacity limit dropped tokens
+    next_states = hidden.clone()
+    for e in torch.nonzero(mask.sum(dim=(0, 1)), as_tuple=True)[0]:
+        sel = mask[:, :, e].bool()
+        expert = layers['expert_%d' % int(e)]
+        saved = sub1.Sub1Linear.fast
+        sub1.Sub1Linear.fast = False
+        try:
+            next_states[sel] = expert(hidden[sel])
+        finally:
+            sub1.Sub1Linear.fast = saved
+    want = probs * next_states
+    assert torch.equal(out, want)
+    assert torch.equal(index, torch.argmax(mask, dim=-1))
+    assert torch.equal(logits, outs[2])
+    # a second call reuses the stacked experts
+    assert torch.equal(fast(hidden)[0], want)
