@@ -116,3 +116,29 @@ def test_faster_mlp_equals_the_expert_loop(gpu, order):
     assert torch.equal(logits, outs[2])
     # a second call reuses the stacked experts
     assert torch.equal(fast(hidden)[0], want)
+
+
+def test_checkpoint_directory_to_one_launch_layer(gpu, tmp_path):
+    """Experts written in the reference's directory format come back as one
+    stacked layer whose output equals the per-expert layers' output."""
+    from qmoe_amd import checkpoint, sub1
+    d_model, d_ff, experts = 128, 320, 4
+    g = torch.Generator(device='cuda').manual_seed(51)
+    mgr = checkpoint.Sub1CheckpointManager(str(tmp_path), config={'d_model': d_model})
+    made = []
+    for j in range(experts):
+        wi = sub1.Sub1Linear.make(ternary_dense(d_ff, d_model, 0.8, g))
+        wo = sub1.Sub1Linear.make(ternary_dense(d_model, d_ff, 0.8, g))
+        made.append(Expert(wi, wo))
+        mgr.add_expert('decoder.block.1.layer.2.mlp.experts.expert_%d' % j, wi, wo)
+    mgr.finalize()
+    stacks = checkpoint.load_expert_stacks(str(tmp_path), 'cuda:0')
+    assert list(stacks) == ['decoder.block.1.layer.2.mlp']
+    layer = stacks['decoder.block.1.layer.2.mlp']
+    x = torch.randn((9, d_model), generator=g, device='cuda').bfloat16()
+    route = torch.tensor([0, 3, 1, 2, 2, -1, 0, 3, 1], dtype=torch.int32, device='cuda')
+    y = layer(x, route)
+    for t in range(9):
+        e = int(route[t])
+        want = x[t:t + 1] if e < 0 else made[e](x[t:t + 1])
+        assert torch.equal(y[t:t + 1], want), t
