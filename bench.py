@@ -69,10 +69,13 @@ def time_launches(fn, steps, warmup, stream_ptr):
     return wall, us.value / steps
 
 
-def cpu_baseline(stack, x, sample_experts, budget_s=12.0):
+def cpu_baseline(stack, x, sample_experts, threads, budget_s=10.0):
     """The CPU oracle's reference-order decode+matvec (a scalar C port of the
-    reference kernel's arithmetic, one core) on the first experts of the same
-    stack, extrapolated to the whole layer."""
+    reference kernel's arithmetic) on the first experts of the same stack:
+    `threads` experts at a time on as many host cores (the C call runs outside
+    the interpreter lock).  Returns (experts done, wall seconds inside the
+    oracle); transfers of the experts to the host are not timed."""
+    import concurrent.futures
     import numpy as np
     import torch
     from oracle import sub1_oracle as so
@@ -80,18 +83,40 @@ def cpu_baseline(stack, x, sample_experts, budget_s=12.0):
     o = so.COracle()
     o.tables()
     done, spent = 0, 0.0
-    for e in range(sample_experts):
-        wi, wo = synthetic.expert_layers(stack, e)
-        host = [tuple(t.view(torch.int16).cpu().numpy().view(np.uint16) if t.dtype != torch.int32
-                      else t.cpu().numpy() for t in l) for l in (wi, wo)]
-        xe = x[e].view(torch.int16).cpu().numpy().view(np.uint16)
-        tick = time.perf_counter()
-        o.expert_ffn(host[0], host[1], xe, order=0)
-        spent += time.perf_counter() - tick
-        done += 1
-        if spent > budget_s:
-            break
+    with concurrent.futures.ThreadPoolExecutor(max_workers=threads) as pool:
+        while done < sample_experts and spent < budget_s:
+            batch = []
+            for e in range(done, min(done + 4 * threads, sample_experts)):
+                wi, wo = synthetic.expert_layers(stack, e)
+                host = [tuple(t.view(torch.int16).cpu().numpy().view(np.uint16)
+                              if t.dtype != torch.int32 else t.cpu().numpy() for t in l)
+                        for l in (wi, wo)]
+                batch.append((host[0], host[1],
+                              x[e].view(torch.int16).cpu().numpy().view(np.uint16)))
+            tick = time.perf_counter()
+            list(pool.map(lambda b: o.expert_ffn(b[0], b[1], b[2], order=0), batch))
+            spent += time.perf_counter() - tick
+            done += len(batch)
     return done, spent
+
+
+def cpu_single_matrix_us(seed):
+    """The first configuration of the list: one Switch-base wi matrix
+    (3072 x 768, P(0) = 0.9), one token, decode + product on one host core
+    through the C oracle in the reference kernel's arithmetic.  Microseconds
+    per product."""
+    from oracle import sub1_oracle as so
+    o = so.COracle()
+    o.tables()
+    t, mm = so.synthetic_ternary(3072, 768, 0.9, seed)
+    codes, row_off = o.encode(t)
+    xv = so.synthetic_activation(768, seed + 1)
+    o.matvec_lanes(codes, row_off, mm, xv)
+    reps = 20
+    tick = time.perf_counter()
+    for _ in range(reps):
+        o.matvec_lanes(codes, row_off, mm, xv)
+    return (time.perf_counter() - tick) / reps * 1e6
 
 
 def dense_gemv_us(stack, x, experts):
@@ -126,6 +151,58 @@ def dense_gemv_us(stack, x, experts):
     return (time.perf_counter() - tick) / reps / experts * 1e6
 
 
+def single_matrix_protocol(seed, stream_ptr):
+    """The reference's own benchmark (test.py:117-126 and 163-186: 100 warm-up
+    + 1000 calls of one product per Switch shape, compressed against dense
+    bf16 torch.matmul) with one token.  Per shape: kernel-side microseconds
+    from HIP events over back-to-back calls for the prepared layout, the
+    packed layout (`sub1matvec`, the drop-in call) and the dense product, and
+    the reference's wall-clock protocol (synchronise after every call) for the
+    drop-in call and the dense product."""
+    import torch
+    from qmoe_amd import sub1, sub1_hip, synthetic
+
+    def sync_each_us(fn, warmup=100, reps=1000):
+        for _ in range(warmup):
+            fn()
+            torch.cuda.synchronize()
+        tick = time.perf_counter()
+        for _ in range(reps):
+            fn()
+            torch.cuda.synchronize()
+        return (time.perf_counter() - tick) / reps * 1e6
+
+    g = torch.Generator(device='cuda')
+    g.manual_seed(seed)
+    dec, trie = sub1.device_tables('cuda:0')
+    rows = {}
+    for name, (h, w, p0) in (('base_wi', (3072, 768, 0.9)), ('base_wo', (768, 3072, 0.9)),
+                             ('large_wi', (4096, 1024, 0.88)), ('large_wo', (1024, 4096, 0.88)),
+                             ('c2048_wi', (6144, 2080, 0.9)), ('c2048_wo', (2080, 6144, 0.9))):
+        t = synthetic.draw_symbols(h, w, p0, g, 'cuda')
+        mm = synthetic.draw_minmax(h, g, 'cuda')
+        lut = torch.stack((torch.zeros(h, device='cuda', dtype=torch.bfloat16), mm[0::2], mm[1::2]), 1)
+        dense = torch.gather(lut, 1, t.long()).contiguous()
+        row_off = torch.zeros(h + 1, dtype=torch.int32, device='cuda')
+        w_comp = sub1_hip.sub1pack(trie, t, row_off)
+        del t
+        x = torch.randn(w, generator=g, device='cuda').bfloat16()
+        y = torch.zeros(h, dtype=torch.bfloat16, device='cuda')
+        x2, y2 = x.reshape(1, -1), torch.zeros((1, h), dtype=torch.bfloat16, device='cuda')
+        xd, yd = x.reshape(-1, 1), torch.zeros((h, 1), dtype=torch.bfloat16, device='cuda')
+        pm = sub1_hip.PreparedMatrix(dec, w_comp, row_off, mm, w)
+        packed = lambda: sub1_hip.sub1matvec(dec, w_comp, row_off, mm, x, y)
+        matmul = lambda: torch.matmul(dense, xd, out=yd)
+        rows[name] = {
+            'prepared_us': round(time_launches(lambda: pm.matvec_tokens(x2, y2), 1000, 100, stream_ptr)[1], 2),
+            'packed_us': round(time_launches(packed, 1000, 100, stream_ptr)[1], 2),
+            'dense_bf16_us': round(time_launches(matmul, 1000, 100, stream_ptr)[1], 2),
+            'sync_each_packed_us': round(sync_each_us(packed), 2),
+            'sync_each_dense_us': round(sync_each_us(matmul), 2),
+            'compressed_bytes': 2 * w_comp.numel(), 'dense_bytes': 2 * h * w}
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -137,6 +214,12 @@ def main():
     ap.add_argument('--no-dense', action='store_true', help='skip the dense bf16 comparison')
     ap.add_argument('--sweep-only', action='store_true',
                     help='only the headline sweep (what a profiler run should see)')
+    ap.add_argument('--small-batch-only', type=int, default=0, metavar='TOKENS',
+                    help='instead of the benchmark, run the expert layer of the workload on '
+                         'this many tokens (1: one token to one expert; more: softmax router) '
+                         '`--steps` times, for a profiler')
+    ap.add_argument('--single-matrix-only', action='store_true',
+                    help='instead of the benchmark, run only the one-product-per-shape protocol')
     ap.add_argument('--seed', type=int, default=20231116)
     ap.add_argument('--calibrate-copy', type=int, default=0, metavar='MIB',
                     help='instead of the benchmark, run a plain device copy of this many MiB '
@@ -159,6 +242,12 @@ def main():
     import torch
     from qmoe_amd import synthetic
 
+    if args.single_matrix_only:
+        torch.cuda.set_device(0)
+        stream_ptr = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        print(json.dumps({'single_matrix_1_token': single_matrix_protocol(args.seed + 30, stream_ptr)}))
+        return
+
     shape, experts, p_zero, desc = WORKLOADS[args.workload]
     if args.experts:
         experts = args.experts
@@ -179,6 +268,20 @@ def main():
           (time.perf_counter() - tick, prep.stream_bytes / 1e9,
            prep.stream_bytes / (2.0 * stack.w_comp.numel()),
            (prep.code_bytes - prep.stream_bytes) / 1e9), file=sys.stderr)
+
+    if args.small_batch_only:
+        t = args.small_batch_only
+        xs = synthetic.activations(t, d_model, args.seed + 3)
+        if t == 1:
+            g = torch.Generator().manual_seed(args.seed + 2)
+            rs = torch.randint(0, experts, (1,), generator=g).to(torch.int32).cuda()
+        else:
+            rs = synthetic.softmax_router(t, experts, args.seed + 4)
+        ys = torch.empty_like(xs)
+        stream_ptr = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        _, us = time_launches(lambda: prep.forward(xs, rs, ys), args.steps, args.warmup, stream_ptr)
+        print(json.dumps({'workload': desc, 'tokens': t, 'us_per_layer': round(us, 2)}))
+        return
 
     x = synthetic.activations(experts, d_model, args.seed + 1)
     route = torch.arange(experts, dtype=torch.int32, device='cuda')
@@ -263,16 +366,23 @@ def main():
                 entry['dense_bf16_gemv_us_per_layer'] = round(dense_gemv_us(st, xs, n_e) * n_e, 1)
             also[name] = entry
             del st, pr
+    if not args.no_dense:
+        also['single_matrix_1_token'] = single_matrix_protocol(args.seed + 30, stream_ptr)
     out['also'] = also
 
     if not args.no_cpu:
-        done, spent = cpu_baseline(stack, x, min(experts, 512))
+        cores = min(16, len(os.sched_getaffinity(0)))
+        done1, spent1 = cpu_baseline(stack, x, min(experts, 64), 1, budget_s=3.0)
+        done, spent = cpu_baseline(stack, x, experts, cores)
         out['cpu_baseline'] = {
-            'value': round(spent / done * experts * 1e6, 1), 'unit': 'us/layer', 'cores': 1,
+            'value': round(spent / done * experts * 1e6, 1), 'unit': 'us/layer', 'cores': cores,
             'kind': 'port',
             'sample': '%d of %d expert FFNs of the same stack through the scalar C oracle in '
-                      'the reference kernel\'s lane order, %.1f s, extrapolated to the layer'
-                      % (done, experts, spent)}
+                      'the reference kernel\'s lane order, %d at a time on %d host threads, '
+                      '%.1f s, extrapolated to the layer' % (done, experts, cores, cores, spent),
+            'one_core_us_per_layer': round(spent1 / done1 * experts * 1e6, 1),
+            'one_core_sample': '%d expert FFNs, %.1f s' % (done1, spent1),
+            'base_wi_3072x768_one_core_us': round(cpu_single_matrix_us(args.seed + 20), 1)}
     print(json.dumps(out))
 
 
