@@ -897,43 +897,63 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
   }
 }
 
-// One tile per workgroup, for the batches too small to occupy the GPU with a
-// wavefront per slice: built for latency.  `split` wavefronts share a slice
-// (split_begin / split_run), all of a wavefront's loads leave before anything
-// waits, and nothing loops.  Tiles are taken by ticket like in the persistent
-// kernel, so a wo tile's wait for its token's wi tiles ends for the same reason.
+// For the batches too small to occupy the GPU with a wavefront per slice: built
+// for latency.  `split` wavefronts share a slice (split_begin / split_run) and
+// all of a wavefront's loads leave before anything waits.  With no more tiles
+// than compute units every workgroup runs one tile; beyond that the grid is
+// persistent and keeps its table.  Tiles are taken by ticket like in the
+// streaming kernel, so a wo tile's wait for its token's wi tiles ends for the
+// same reason.
 __global__ __launch_bounds__(kMaxThreads) void moe_prepared_small_kernel(PreparedArgs a) {
   extern __shared__ __align__(16) uint32_t lds[];
   __shared__ int s_ticket;
   uint32_t *tab = lds;
   uint32_t *xa = lds + a.table_words;
   const bool dynamic = a.ctrl != nullptr;
-  int ticket = blockIdx.x;
-  if (dynamic && threadIdx.x == 0)
-    s_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  stage_table(tab, a.table, a.table_words);
-  if (dynamic) {
-    __syncthreads();
-    ticket = __builtin_amdgcn_readfirstlane(s_ticket);
-  }
   const int n_all = a.tokens * (a.k[0].parts + (a.kinds == 2 ? a.k[1].parts : 0));
-  if (ticket >= n_all) return;
-  const Tile tile = decode_tile(a, ticket, dynamic);
-  const int kind = tile.kind, t = tile.t, e = tile.e;
-  const KindArgs &k = a.k[kind];
-  if (a.kinds == 2 && kind == 1 && e < 0) {
-    pass_through(a, k, t, tile.s_lo, tile.s_hi);
-    return;
+  int static_ticket = blockIdx.x;
+  int next_ticket = 0;
+  if (dynamic && threadIdx.x == 0)
+    next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+  stage_table(tab, a.table, a.table_words);
+  for (;;) {
+    int ticket;
+    if (dynamic) {
+      __syncthreads();   // the previous tile is done with s_ticket, x and the partial sums
+      if (threadIdx.x == 0) {
+        s_ticket = next_ticket;
+        if (next_ticket < n_all && n_all > static_cast<int>(gridDim.x))
+          next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+        else
+          next_ticket = n_all;
+      }
+      __syncthreads();
+      ticket = __builtin_amdgcn_readfirstlane(s_ticket);
+    } else {
+      __syncthreads();
+      ticket = static_ticket;
+      static_ticket += gridDim.x;
+    }
+    if (ticket >= n_all) break;
+    const Tile tile = decode_tile(a, ticket, dynamic);
+    const int kind = tile.kind, t = tile.t, e = tile.e;
+    const KindArgs &k = a.k[kind];
+    if (a.kinds == 2 && kind == 1 && e < 0) {
+      pass_through(a, k, t, tile.s_lo, tile.s_hi);
+      continue;
+    }
+    if (e >= 0) {
+      int mode;
+      uint16_t *dst = tile_output(a, k, kind, t, mode);
+      // the launch cuts the matrices so that a tile has at most waves / split slices
+      SplitWalk walk = split_begin(a, k, e, tile.s_lo, tile.s_hi);
+      await_activations(a, k, kind, t, xa);
+      split_run(a, k, walk, tab, xa, dst, mode);
+    }
+    if (a.kinds == 2 && kind == 0) publish_h(a, t);
   }
-  if (e >= 0) {
-    int mode;
-    uint16_t *dst = tile_output(a, k, kind, t, mode);
-    // the launch cuts the matrices so that a tile has at most waves / split slices
-    SplitWalk walk = split_begin(a, k, e, tile.s_lo, tile.s_hi);
-    await_activations(a, k, kind, t, xa);
-    split_run(a, k, walk, tab, xa, dst, mode);
-  }
-  if (a.kinds == 2 && kind == 0) publish_h(a, t);
 }
 
 // ------------------------------------------------------ per-device tables --
@@ -1377,7 +1397,8 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     zero_words_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl);
   }
   if (small) {
-    moe_prepared_small_kernel<<<static_cast<unsigned>(tiles), 64 * waves, lds, s>>>(a);
+    const int64_t grid = tiles < cus ? tiles : cus;
+    moe_prepared_small_kernel<<<static_cast<unsigned>(grid), 64 * waves, lds, s>>>(a);
   } else {
     const int64_t grid = tiles < cus ? tiles : cus;
     moe_prepared_kernel<<<static_cast<unsigned>(grid), 64 * waves, lds, s>>>(a);
