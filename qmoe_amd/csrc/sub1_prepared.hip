@@ -759,23 +759,23 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
   const int n_all = n_wi + (a.kinds == 2 ? a.tokens * a.k[1].parts : 0);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const bool dynamic = a.ctrl != nullptr;
-  // dynamic order: thread 0 keeps one ticket ahead so that the atomic's round
-  // trip overlaps a tile; static order: tile = workgroup index + k * grid
+  // dynamic order: thread 0 asks for the next ticket when its own part of the
+  // tile is done, so that the atomic's round trip overlaps the tile's tail (any
+  // earlier and the workgroups that start first take tiles away from the last
+  // ones); static order: tile = workgroup index + k * grid
   int static_ticket = blockIdx.x;   // the same in every lane, unlike thread 0's next_ticket
   int next_ticket = 0;
-  if (dynamic && threadIdx.x == 0)
-    next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
-                                         __HIP_MEMORY_SCOPE_AGENT);
+  auto fetch_next = [&]() {
+    if (dynamic && threadIdx.x == 0)
+      next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+  };
+  fetch_next();
   for (;;) {
     __syncthreads();
     int ticket;
     if (dynamic) {
-      if (threadIdx.x == 0) {
-        s_ticket = next_ticket;
-        if (next_ticket < n_all)
-          next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
-                                               __HIP_MEMORY_SCOPE_AGENT);
-      }
+      if (threadIdx.x == 0) s_ticket = next_ticket;
       __syncthreads();
       ticket = __builtin_amdgcn_readfirstlane(s_ticket);   // the same in every lane: scalar
     } else {
@@ -788,6 +788,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
     const KindArgs &k = a.k[kind];
     if (a.kinds == 2 && kind == 1 && e < 0) {
       pass_through(a, k, t, s_lo, s_hi);
+      fetch_next();
       continue;
     }
     if (e >= 0) {
@@ -810,6 +811,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
         }
       }
     }
+    fetch_next();
     if (a.kinds == 2 && kind == 0) publish_h(a, t);
   }
 }
@@ -835,17 +837,15 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
   // and the columns past d_ff stay zero for the whole launch
   for (int i = threadIdx.x; i < a.hdwords; i += threads) ha[i] = 0u;
   int next_ticket = 0;
-  if (threadIdx.x == 0)
-    next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
-                                         __HIP_MEMORY_SCOPE_AGENT);
+  auto fetch_next = [&]() {
+    if (threadIdx.x == 0)
+      next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+  };
+  fetch_next();
   for (;;) {
     __syncthreads();   // the previous token's wo has read h; s_ticket is free
-    if (threadIdx.x == 0) {
-      s_ticket = next_ticket;
-      if (next_ticket < a.tokens)
-        next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
-                                             __HIP_MEMORY_SCOPE_AGENT);
-    }
+    if (threadIdx.x == 0) s_ticket = next_ticket;
     __syncthreads();
     const int t = __builtin_amdgcn_readfirstlane(s_ticket);
     if (t >= a.tokens) break;
@@ -857,6 +857,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
     }
     if (e < 0) {
       pass_through(a, ko, t, 0, ko.slices);
+      fetch_next();
       continue;
     }
     // wi: x -> relu(h) into LDS
@@ -880,6 +881,10 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
       }
       if (more) cur = nxt;
     }
+    // the next token is asked for halfway through this one: early enough to
+    // hide the round trip, late enough that the workgroups that started first
+    // do not take the last tokens away from the others
+    fetch_next();
     // wo: h -> y; its first loads go out before the barrier
     s = wave;
     if (s < ko.slices) cur = load_slice(a, ko, static_cast<int64_t>(e) * ko.slices + s);
@@ -1357,8 +1362,21 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     k.groups_max = (p.max_chunks[i] + kGroupChunks - 1) / kGroupChunks;
     k.split = 1;
     const int max_parts = (k.slices + waves - 1) / waves;
-    k.parts = want > max_parts ? max_parts : want;
     if (want > max_parts) idle_units = true;
+    // Parts per matrix for the streaming kernel: the count that needs the fewest
+    // passes of a workgroup per compute unit (a pass = one slice per wavefront;
+    // 33 slices are 3 passes as one part but 1.5 rounds of 1 pass as three).
+    double best = 1e30;
+    for (int parts = 1; parts <= max_parts; parts++) {
+      const int per_tile = (k.slices + parts - 1) / parts;
+      const int64_t rounds = (static_cast<int64_t>(tokens) * parts + cus - 1) / cus;
+      // a quarter of a pass per tile for staging its activations
+      const double cost = rounds * ((per_tile + waves - 1) / waves + 0.25);
+      if (cost < best - 1e-9) {
+        best = cost;
+        k.parts = parts;
+      }
+    }
   }
   size_t lds_partials = 0;
   if (idle_units) lds_partials = plan_small(a, p.kinds, tokens, cus, waves, lds_limit - lds_base);
