@@ -220,6 +220,9 @@ def main():
                          '`--steps` times, for a profiler')
     ap.add_argument('--single-matrix-only', action='store_true',
                     help='instead of the benchmark, run only the one-product-per-shape protocol')
+    ap.add_argument('--probe-gathers', action='store_true',
+                    help='instead of the benchmark, measure the time per random-gather '
+                         'instruction from LDS and from global tables (the bound of the decode loop)')
     ap.add_argument('--seed', type=int, default=20231116)
     ap.add_argument('--calibrate-copy', type=int, default=0, metavar='MIB',
                     help='instead of the benchmark, run a plain device copy of this many MiB '
@@ -241,6 +244,21 @@ def main():
     import ctypes
     import torch
     from qmoe_amd import synthetic
+
+    if args.probe_gathers:
+        from qmoe_amd import _lib
+        lib = _lib.load()
+        torch.cuda.set_device(0)
+        stream_ptr = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rows = {}
+        for name, from_lds, words in (('lds_16k_words', 1, 16384), ('lds_32k_words', 1, 32768),
+                                      ('global_4KB', 0, 1024), ('global_16KB', 0, 4096),
+                                      ('global_64KB', 0, 16384), ('global_256KB', 0, 65536)):
+            c = ctypes.c_double()
+            _lib.check(lib.sub1_probe_gather(from_lds, words, 4000, ctypes.byref(c), stream_ptr))
+            rows[name] = round(c.value, 3)
+        print(json.dumps({'ns_per_wavefront_gather_per_compute_unit': rows}))
+        return
 
     if args.single_matrix_only:
         torch.cuda.set_device(0)

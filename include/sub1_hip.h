@@ -271,6 +271,16 @@ int sub1_matvec_prepared(const sub1_matrix_prepared *prepared, const int32_t *to
 int sub1_timing_begin(void *stream);
 int sub1_timing_end(void *stream, double *elapsed_us);
 
+/*
+ * Gather-rate probe (no counterpart in the reference; for the benchmark's
+ * bound): nanoseconds a compute unit needs per wavefront instruction that reads one
+ * random dword per lane from a table of `words` dwords (a power of two), held
+ * in LDS (from_lds != 0, words <= 32768) or in global memory, with 16
+ * wavefronts per compute unit and four gathers in flight per lane, as in the
+ * decode loop.  Allocates and frees its own buffers; synchronises.
+ */
+int sub1_probe_gather(int from_lds, int words, int steps, double *ns_per_gather, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -77,6 +77,7 @@ PROTOTYPES = {
                                     _int, _vp]),
     'sub1_timing_begin': (_int, [_vp]),
     'sub1_timing_end': (_int, [_vp, ctypes.POINTER(ctypes.c_double)]),
+    'sub1_probe_gather': (_int, [_int, _int, _int, ctypes.POINTER(ctypes.c_double), _vp]),
 }
 
 _lib = None
