@@ -142,3 +142,35 @@ def test_checkpoint_directory_to_one_launch_layer(gpu, tmp_path):
         e = int(route[t])
         want = x[t:t + 1] if e < 0 else made[e](x[t:t + 1])
         assert torch.equal(y[t:t + 1], want), t
+
+
+def test_layer_launch_replays_from_a_graph(gpu):
+    """The grouped launch allocates nothing and clears its control words with
+    a kernel, so a HIP graph can hold it: replays (with eager launches and
+    synchronisations in between) give the eager result every time."""
+    from qmoe_amd import synthetic
+    d_model, d_ff = synthetic.SHAPES['base']
+    stack = synthetic.build_stack(8, d_model, d_ff, 0.9, seed=61)
+    prep = stack.prepare()
+    for tokens in (1, 12):
+        x = synthetic.activations(tokens, d_model, seed=62)
+        route = (torch.arange(tokens, dtype=torch.int32, device='cuda') * 3) % 8
+        y = torch.empty_like(x)
+        prep.forward(x, route, y)            # first call: tables, workspace
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            prep.forward(x, route, y)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            prep.forward(x, route, y)
+        for rep in range(4):
+            x.copy_(synthetic.activations(tokens, d_model, seed=70 + rep))
+            y.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = y.clone()
+            eager = prep.forward(x, route)   # eager work between the replays
+            torch.cuda.synchronize()
+            assert torch.equal(got, eager), (tokens, rep)
