@@ -429,6 +429,26 @@ def test_token_per_workgroup_tiles_with_dropped_tokens(gpu, oracle):
     assert torch.equal(y, stack.forward(x, route))
 
 
+@pytest.mark.parametrize('d_model,d_ff', [(64, 8192), (8192, 64), (2, 2)])
+def test_extreme_widths_in_every_batch_regime(gpu, oracle, d_model, d_ff):
+    """The widest activations the fast layout takes (8192: table, x and h fill
+    the LDS) and the narrowest, from one token to more tokens than compute
+    units: every regime must equal the packed-layout kernel, and one token
+    must equal the oracle."""
+    stack, wi, wo = small_stack(oracle, 2, d_model, d_ff, 0.95, seed=800)
+    prep = stack.prepare()
+    xs = np.stack([so.synthetic_activation(d_model, 900 + i) for i in range(3)])
+    want, _ = oracle.expert_ffn(wi[1], wo[1], xs[0], order=1)
+    for tokens in (1, 7, 90, 300):
+        x = bf16_dev(np.tile(xs, (tokens // 3 + 1, 1))[:tokens])
+        route = torch.ones(tokens, dtype=torch.int32, device='cuda')
+        route[1::2] = 0
+        y = prep.forward(x, route)
+        assert prep.launch_faults(tokens) == (0, 0)
+        assert torch.equal(y, stack.forward(x, route)), tokens
+        assert np.array_equal(bits_host(y[0]), want), tokens
+
+
 @pytest.mark.parametrize('height,width,p0', SWITCH_SHAPES + [(77, 333, 0.7), (5, 1, 0.5),
                                                              (130, 15, 0.9), (300, 8192, 0.99)])
 def test_prepared_matrix_product(gpu, oracle, height, width, p0):
