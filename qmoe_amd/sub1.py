@@ -64,13 +64,16 @@ class Sub1Linear(nn.Module):
     fast = True
 
     def _prepared(self, width):
-        key = tuple((t.data_ptr(), t._version, t.numel())
-                    for t in (self.w_comp, self.row_off, self.ter_minmax)) + (width,)
+        live = (self.w_comp, self.row_off, self.ter_minmax)
+        key = tuple((t.data_ptr(), t._version, t.numel()) for t in live) + (width,)
         cached = getattr(self, '_prepared_cache', None)
         if cached is None or cached[0] != key:
             table = DEC[self.w_comp.device.index]
+            # the entry keeps the source tensors alive: their addresses are part
+            # of the key and must not be handed out again while it is cached
             cached = (key, sub1_hip.PreparedMatrix(table, self.w_comp, self.row_off,
-                                                   self.ter_minmax, width))
+                                                   self.ter_minmax, width),
+                      [t.detach() for t in live])
             self._prepared_cache = cached
         return cached[1]
 
@@ -173,12 +176,15 @@ class FasterMLP(nn.Module):
         self.gpu = gpu
 
     def _launcher(self):
-        key = tuple((t.data_ptr(), t._version) for e in self.experts for l in (e.wi, e.wo)
-                    for t in (l.w_comp, l.row_off, l.ter_minmax))
+        live = [t for e in self.experts for l in (e.wi, e.wo)
+                for t in (l.w_comp, l.row_off, l.ter_minmax)]
+        key = tuple((t.data_ptr(), t._version, t.numel()) for t in live)
         cached = getattr(self, '_launcher_cache', None)
         if cached is None or cached[0] != key:
             stack = Sub1Experts([e.wi for e in self.experts], [e.wo for e in self.experts]).stack
-            cached = (key, stack.prepare() if stack.can_prepare() else stack)
+            # the aliases keep the keyed addresses from being reused while cached
+            cached = (key, stack.prepare() if stack.can_prepare() else stack,
+                      [t.detach() for t in live])
             self._launcher_cache = cached
         return cached[1]
 

@@ -485,3 +485,38 @@ def test_sub1linear_fast_and_packed_paths_agree(gpu, oracle):
     lin.fast = True
     lin.ter_minmax = (lin.ter_minmax.float() * 2).bfloat16()
     assert torch.equal(lin(x).float(), 2 * y_fast.float())
+
+
+def test_sub1linear_prepared_copy_follows_the_buffers(gpu, oracle):
+    """In-place writes and `.data` replacement (as a checkpoint loader does)
+    must both be seen by the cached fast layout, also when the allocator could
+    hand the old address to the new tensor."""
+    sub1, op = gpu
+    layers = []
+    for seed in (81, 82):
+        t, mm = so.synthetic_ternary(256, 128, 0.8, seed=seed)
+        layers.append(sub1.Sub1Linear.make(bf16_dev(oracle.dequant(t.astype(np.uint8), mm))))
+    a, b = layers
+    x = torch.randn((3, 128), generator=torch.Generator().manual_seed(5)).bfloat16().cuda()
+    ya, yb = a(x).clone(), b(x).clone()
+    assert not torch.equal(ya, yb)
+    # in place: a takes b's min/max (same shape), result changes accordingly
+    saved = a.ter_minmax.clone()
+    a.ter_minmax.copy_(b.ter_minmax)
+    a.fast = False
+    want = a(x).clone()
+    a.fast = True
+    assert torch.equal(a(x), want) and not torch.equal(want, ya)
+    a.ter_minmax.copy_(saved)
+    assert torch.equal(a(x), ya)
+    # replacement after the old storage was dropped: freshly allocated tensors
+    # of the same sizes, which the caching allocator would place where the old
+    # ones were if nothing held them
+    nb = {n: getattr(b, n).clone() for n in ('w_comp', 'row_off', 'ter_minmax')}
+    for n in nb:
+        getattr(a, n).data = torch.empty(0, dtype=nb[n].dtype, device='cuda')
+    for n in nb:
+        fresh = torch.empty_like(nb[n])
+        fresh.copy_(nb[n])
+        getattr(a, n).data = fresh
+    assert torch.equal(a(x), yb)
