@@ -18,10 +18,13 @@
 // (activations under row-min weights, under row-max weights) with
 // v_dot2c_f32_bf16 on (x,0)/(0,x) bf16 pairs; no cross-lane traffic at all.
 // They compute what reference sub1_cuda_kernel.cu:163-201 computes per row.
-// moe_prepared_kernel is the streaming form (persistent grid, a wavefront per
-// slice, the next slice's loads in flight); moe_prepared_small_kernel is the
-// latency form for a handful of tokens (one tile per workgroup, wavefronts
-// share a slice from column checkpoints).  Both give the same bits.
+// Three kernels share that loop and give the same bits:
+// moe_prepared_fused_kernel streams whole tokens (wi, ReLU, wo in one
+// workgroup, h kept in LDS) when there is at least a token per compute unit;
+// moe_prepared_kernel streams tiles of one matrix (persistent grid, a wavefront
+// per slice, the next slice's loads in flight) for smaller batches and for
+// single matrices; moe_prepared_small_kernel is the latency form for a handful
+// of tokens (wavefronts share a slice from column checkpoints).
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -496,8 +499,7 @@ __device__ __forceinline__ void run_chunks(Walk<R> &w, const uint2 *p, int c, ui
 
 // The two sums of this lane's row, in the library's canonical order: groups of
 // 32 codes (kGroupChunks chunks), a partial sum per group from zero, the
-// partial sums added first group first.  Starts at chunk c0 (a multiple of
-// kGroupChunks) with column offset colw and stops before chunk c_end.
+// partial sums added first group first.
 __device__ __forceinline__ void run_slice(SliceWalk &w, const uint16_t *codes, int group_shift,
                                           const uint32_t *tab,
                                           const uint32_t *xa, float &s1, float &s2) {
@@ -1192,8 +1194,6 @@ int prepare_codes(const Source &src, const Prepared &p, hipStream_t s, const cha
   return SUB1_OK;
 }
 
-// Launch of the prepared kernel.  kinds == 2: y = wo(relu(wi x)) per token,
-// workspace required; kinds == 1: y += W x per token, no workspace.
 // Cut of the matrices for a batch that cannot occupy the GPU with a wavefront
 // per slice.  Per projection: a workgroup takes per_wg slices (16 = no sharing)
 // and waves / per_wg wavefronts share each slice, at most one per 32-code group.
@@ -1265,6 +1265,8 @@ size_t plan_small(PreparedArgs &a, int kinds, int tokens, int cus, int waves, si
   return partials;
 }
 
+// Launch of the prepared kernels.  kinds == 2: y = wo(relu(wi x)) per token,
+// workspace required; kinds == 1: y += W x per token, no workspace.
 int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *x, int64_t ldx,
                     void *y, int64_t ldy, int tokens, void *workspace, int64_t workspace_bytes,
                     hipStream_t s, const char *who) {
@@ -1404,7 +1406,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   }
   const size_t lds = lds_base + lds_partials;
   // Batches too small to occupy the GPU with a wavefront per slice go to the
-  // one-tile-per-workgroup kernel, everything else to the persistent one with
+  // latency kernel, everything else to the persistent one; either way at most
   // a workgroup per compute unit (LDS holds the table once).
   const void *fn = small ? reinterpret_cast<const void *>(moe_prepared_small_kernel)
                          : reinterpret_cast<const void *>(moe_prepared_kernel);
