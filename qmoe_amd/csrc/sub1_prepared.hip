@@ -293,6 +293,7 @@ struct KindArgs {
   int split;            // wavefronts that share one slice (1 = a slice per wavefront)
   int groups_max;       // most 32-code groups in a slice of this kind
   int64_t first_slice;  // global index of the kind's first slice (checkpoint addressing)
+  int tail_split;       // fused kernel: wavefronts per slice of a short last pass (0: none)
 };
 
 struct PreparedArgs {
@@ -447,26 +448,35 @@ __device__ __forceinline__ const uint2 *chunk_pointer(const uint16_t *codes, uin
 template <int R>
 struct Walk {
   uint32_t base;     // the slice's first chunk, in chunks; the same in every lane,
-  int nch, nfull;    // like the chunk counts
+  int nch, nfull;    // like the chunk counts (nch: where this wavefront stops)
+  int c0;            // and the chunk this wavefront starts at (0 unless it shares the slice)
+  int colw0;         // this lane's column offset at chunk c0
   int len, ridx;
   uint32_t minmax;
   uint2 ring[R];
 };
 typedef Walk<kRing> SliceWalk;
 
+// g_lo, g_hi: the run of 32-code groups to walk, for a wavefront that shares the
+// slice with others (it then starts from the column checkpoint of group g_lo).
 __device__ __forceinline__ SliceWalk load_slice(const PreparedArgs &a, const KindArgs &k,
-                                                int64_t sl) {
+                                                int64_t sl, int g_lo = 0, int g_hi = 1 << 20) {
   const int lane = threadIdx.x & 63;
   SliceWalk w;
-  w.nch = __builtin_amdgcn_readfirstlane(k.slice_nch[sl]);
-  w.nfull = __builtin_amdgcn_readfirstlane(k.slice_nfull[sl]);
+  const int nch_all = __builtin_amdgcn_readfirstlane(k.slice_nch[sl]);
+  w.nch = min(g_hi * kGroupChunks, nch_all);
+  w.nfull = min(__builtin_amdgcn_readfirstlane(k.slice_nfull[sl]), w.nch);
+  w.c0 = g_lo * kGroupChunks;
   w.len = k.row_len[sl * 64 + lane];
   w.ridx = k.row_idx[sl * 64 + lane];
   w.minmax = k.minmax[sl * 64 + lane];
   w.base = __builtin_amdgcn_readfirstlane(k.slice_base[sl]);
+  w.colw0 = 0;
+  if (g_lo)
+    w.colw0 = a.ckpt[(checkpoint_entry(w.base, k.first_slice + sl) + g_lo) * 64 + lane];
   const uint2 *p = chunk_pointer(a.codes, w.base);
 #pragma unroll
-  for (int i = 0; i < kRing; i++) w.ring[i] = p[min(i, w.nch - 1) * 64];
+  for (int i = 0; i < kRing; i++) w.ring[i] = p[min(w.c0 + i, w.nch - 1) * 64];
   return w;
 }
 
@@ -500,9 +510,11 @@ __device__ __forceinline__ void run_chunks(Walk<R> &w, const uint2 *p, int c, ui
 // The two sums of this lane's row, in the library's canonical order: groups of
 // 32 codes (kGroupChunks chunks), a partial sum per group from zero, the
 // partial sums added first group first.
+// With `part` the wavefront shares its slice: it leaves each group's partial
+// sums at part[group * 64 + lane] for the wavefront that adds them up.
 __device__ __forceinline__ void run_slice(SliceWalk &w, const uint16_t *codes, int group_shift,
-                                          const uint32_t *tab,
-                                          const uint32_t *xa, float &s1, float &s2) {
+                                          const uint32_t *tab, const uint32_t *xa, float &s1,
+                                          float &s2, float2 *part = nullptr) {
   const DotConsts dk = dot_consts();
   const uint32_t shift2 = static_cast<uint32_t>(group_shift) * 0x00010001u;
   // a walk that went through `cur = nxt` may sit in vector registers: put what
@@ -511,32 +523,38 @@ __device__ __forceinline__ void run_slice(SliceWalk &w, const uint16_t *codes, i
   w.nch = __builtin_amdgcn_readfirstlane(w.nch);
   w.nfull = __builtin_amdgcn_readfirstlane(w.nfull);
   const uint2 *p = chunk_pointer(codes, __builtin_amdgcn_readfirstlane(w.base));
+  const int lane = threadIdx.x & 63;
   s1 = 0.f;
   s2 = 0.f;
   float p1 = 0.f, p2 = 0.f;
-  int colw = 0;
-  int c = 0;
+  int colw = w.colw0;
+  int c = __builtin_amdgcn_readfirstlane(w.c0);
+  auto group_done = [&]() {
+    if (part) {
+      part[((c + kRing) / kGroupChunks - 1) * 64 + lane] = make_float2(p1, p2);
+    } else {
+      s1 += p1;
+      s2 += p2;
+    }
+    p1 = 0.f;
+    p2 = 0.f;
+  };
   // chunks every lane of the slice has in full: no per-code checks
   for (; c + kRing <= w.nfull; c += kRing) {
     run_chunks<false>(w, p, c, shift2, tab, xa, colw, p1, p2, dk);
-    if ((c + kRing) % kGroupChunks == 0) {
-      s1 += p1;
-      s2 += p2;
-      p1 = 0.f;
-      p2 = 0.f;
-    }
+    if ((c + kRing) % kGroupChunks == 0) group_done();
   }
   for (; c < w.nch; c += kRing) {
     run_chunks<true>(w, p, c, shift2, tab, xa, colw, p1, p2, dk);
-    if ((c + kRing) % kGroupChunks == 0) {
-      s1 += p1;
-      s2 += p2;
-      p1 = 0.f;
-      p2 = 0.f;
-    }
+    if ((c + kRing) % kGroupChunks == 0) group_done();
   }
-  s1 += p1;   // the last, partial group (+0 if it was just folded)
-  s2 += p2;
+  if (part) {
+    // the slice's last group, unless the loop has just closed it
+    if (c % kGroupChunks) part[(c / kGroupChunks) * 64 + lane] = make_float2(p1, p2);
+  } else {
+    s1 += p1;   // the last, partial group (+0 if it was just folded)
+    s2 += p2;
+  }
 }
 
 // How a row's result leaves the kernel.
@@ -887,19 +905,52 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
     // hide the round trip, late enough that the workgroups that started first
     // do not take the last tokens away from the others
     fetch_next();
-    // wo: h -> y; its first loads go out before the barrier
+    // wo: h -> y; its first loads go out before the barrier.  A short last pass
+    // (tail_split != 0) is shared out: tail_split wavefronts per slice, each a
+    // run of its 32-code groups, partial sums into the LDS that held x.
+    const int whole = ko.tail_split ? ko.slices - ko.slices % waves : ko.slices;
+    const int64_t first = static_cast<int64_t>(e) * ko.slices;
     s = wave;
-    if (s < ko.slices) cur = load_slice(a, ko, static_cast<int64_t>(e) * ko.slices + s);
+    if (s < whole) cur = load_slice(a, ko, first + s);
     __syncthreads();
     uint16_t *dst = a.y + static_cast<int64_t>(t) * a.ldy;
-    for (; s < ko.slices; s += waves) {
-      const bool more = s + waves < ko.slices;
+    for (; s < whole; s += waves) {
+      const bool more = s + waves < whole;
       SliceWalk nxt;
-      if (more) nxt = load_slice(a, ko, static_cast<int64_t>(e) * ko.slices + s + waves);
+      if (more) nxt = load_slice(a, ko, first + s + waves);
       float s1, s2;
       run_slice(cur, a.codes, a.group_shift, tab, ha, s1, s2);
       write_row(dst, cur.ridx, cur.minmax, s1, s2, kStore);
       if (more) cur = nxt;
+    }
+    if (ko.tail_split) {
+      const int lane = threadIdx.x & 63;
+      const int sl = whole + wave / ko.tail_split;
+      const int sub = wave % ko.tail_split;
+      float2 *mine = reinterpret_cast<float2 *>(xa) + (wave / ko.tail_split) * ko.groups_max * 64;
+      int groups = 0;
+      if (sl < ko.slices) {
+        groups = (__builtin_amdgcn_readfirstlane(ko.slice_nch[first + sl]) + kGroupChunks - 1) /
+                 kGroupChunks;
+        const int g_lo = sub * groups / ko.tail_split, g_hi = (sub + 1) * groups / ko.tail_split;
+        if (g_lo < g_hi) {
+          SliceWalk tail = load_slice(a, ko, first + sl, g_lo, g_hi);
+          float s1, s2;
+          run_slice(tail, a.codes, a.group_shift, tab, ha, s1, s2, mine);
+        }
+      }
+      __syncthreads();
+      if (sub == 0 && sl < ko.slices) {
+        // the slice's first wavefront adds the groups in order and writes the rows
+        float s1 = 0.f, s2 = 0.f;
+        for (int g = 0; g < groups; g++) {
+          const float2 v = mine[g * 64 + lane];
+          s1 += v.x;
+          s2 += v.y;
+        }
+        write_row(dst, ko.row_idx[(first + sl) * 64 + lane], ko.minmax[(first + sl) * 64 + lane],
+                  s1, s2, kStore);
+      }
     }
   }
 }
@@ -1363,6 +1414,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     first_slice += static_cast<int64_t>(p.count) * k.slices;
     k.groups_max = (p.max_chunks[i] + kGroupChunks - 1) / kGroupChunks;
     k.split = 1;
+    k.tail_split = 0;
     const int max_parts = (k.slices + waves - 1) / waves;
     if (want > max_parts) idle_units = true;
     // Parts per matrix for the streaming kernel: the count that needs the fewest
@@ -1395,6 +1447,17 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   if (fused) {
     a.xdwords = activation_dwords(a.k[0].width);
     a.hdwords = activation_dwords(a.k[1].width);
+    // wo's last pass: with at most half the wavefronts busy, the idle ones take
+    // groups of those slices (partial sums go where x was)
+    KindArgs &ko = a.k[1];
+    const int rest = ko.slices % waves;
+    if (rest > 0 && rest * 2 <= waves && ko.groups_max > 1) {
+      int split = 1;
+      while (split * 2 * rest <= waves && split * 2 <= ko.groups_max) split *= 2;
+      if (split > 1 &&
+          static_cast<size_t>(rest) * ko.groups_max * 512 <= static_cast<size_t>(a.xdwords) * 4)
+        ko.tail_split = split;
+    }
     const void *fn = reinterpret_cast<const void *>(moe_prepared_fused_kernel);
     HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(lds_fused)));
