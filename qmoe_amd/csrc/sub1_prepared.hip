@@ -507,14 +507,36 @@ __device__ __forceinline__ void run_chunks(Walk<R> &w, const uint2 *p, int c, ui
   }
 }
 
+// The hardware serves the oldest wavefront of a SIMD first; left alone, the
+// wavefronts of a workgroup drift apart and the last ones finish a phase on an
+// idle compute unit.  A wavefront therefore lowers its priority as it gets
+// through its share of the phase, in steps that get finer towards the end
+// (`done` of `total`: below 5/8 priority 3, below 13/16 2, below 15/16 1, then
+// 0), so that the laggards catch up and all finish together.
+__device__ __forceinline__ void progress_priority(int done, int total) {
+  const int p = done * 16 / total;
+  if (p < 10) {
+    __builtin_amdgcn_s_setprio(3);
+  } else if (p < 13) {
+    __builtin_amdgcn_s_setprio(2);
+  } else if (p < 15) {
+    __builtin_amdgcn_s_setprio(1);
+  } else {
+    __builtin_amdgcn_s_setprio(0);
+  }
+}
+
 // The two sums of this lane's row, in the library's canonical order: groups of
 // 32 codes (kGroupChunks chunks), a partial sum per group from zero, the
 // partial sums added first group first.
 // With `part` the wavefront shares its slice: it leaves each group's partial
 // sums at part[group * 64 + lane] for the wavefront that adds them up.
+// pass / passes (passes != 0): this slice is the wavefront's pass-th of `passes`
+// about equal ones in the current phase; sets the priority by progress.
 __device__ __forceinline__ void run_slice(SliceWalk &w, const uint16_t *codes, int group_shift,
                                           const uint32_t *tab, const uint32_t *xa, float &s1,
-                                          float &s2, float2 *part = nullptr) {
+                                          float &s2, float2 *part = nullptr, int pass = 0,
+                                          int passes = 0) {
   const DotConsts dk = dot_consts();
   const uint32_t shift2 = static_cast<uint32_t>(group_shift) * 0x00010001u;
   // a walk that went through `cur = nxt` may sit in vector registers: put what
@@ -529,7 +551,9 @@ __device__ __forceinline__ void run_slice(SliceWalk &w, const uint16_t *codes, i
   float p1 = 0.f, p2 = 0.f;
   int colw = w.colw0;
   int c = __builtin_amdgcn_readfirstlane(w.c0);
+  if (passes) progress_priority(pass, passes);
   auto group_done = [&]() {
+    if (passes) progress_priority(pass * w.nch + c + kRing, passes * w.nch);
     if (part) {
       part[((c + kRing) / kGroupChunks - 1) * 64 + lane] = make_float2(p1, p2);
     } else {
@@ -891,7 +915,8 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
       SliceWalk nxt;
       if (more) nxt = load_slice(a, ki, static_cast<int64_t>(e) * ki.slices + s + waves);
       float s1, s2;
-      run_slice(cur, a.codes, a.group_shift, tab, xa, s1, s2);
+      run_slice(cur, a.codes, a.group_shift, tab, xa, s1, s2, nullptr, s / waves,
+                (ki.slices + waves - 1) / waves);
       if (cur.ridx != 0xffff) {
         uint32_t out = f32_to_bf16(row_result(cur.minmax, s1, s2));
         if (out & 0x8000u) out = 0;   // relu between the projections, on the bf16 value
@@ -919,10 +944,12 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
       SliceWalk nxt;
       if (more) nxt = load_slice(a, ko, first + s + waves);
       float s1, s2;
-      run_slice(cur, a.codes, a.group_shift, tab, ha, s1, s2);
+      run_slice(cur, a.codes, a.group_shift, tab, ha, s1, s2, nullptr, s / waves,
+                (whole + waves - 1) / waves);
       write_row(dst, cur.ridx, cur.minmax, s1, s2, kStore);
       if (more) cur = nxt;
     }
+    __builtin_amdgcn_s_setprio(0);
     if (ko.tail_split) {
       const int lane = threadIdx.x & 63;
       const int sl = whole + wave / ko.tail_split;
