@@ -849,7 +849,8 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
           SliceWalk nxt;
           if (more) nxt = load_slice(a, k, static_cast<int64_t>(e) * k.slices + s + waves);
           float s1, s2;
-          run_slice(cur, a.codes, a.group_shift, tab, xa, s1, s2);
+          run_slice(cur, a.codes, a.group_shift, tab, xa, s1, s2, nullptr, (s - s_lo) / waves,
+                    (s_hi - s_lo + waves - 1) / waves);
           write_row(dst, cur.ridx, cur.minmax, s1, s2, mode);
           if (more) cur = nxt;
         }
