@@ -62,7 +62,9 @@ int sub1_build_tables(int32_t *dec_host, int32_t *trie_host);
  * fits LDS: recode_host[65536] maps a dictionary index to its kernel code;
  * codes below *single_codes index table_host directly, a code c at or above it
  * uses word *single_codes + ((c - *single_codes) >> 3) and its low three bits
- * are the symbol bits of the three slots.  table_host must hold
+ * are the symbol bits of the three slots.  A table word holds the slots'
+ * activation offsets in bytes 0, 1 and 3 and six times the pair count in byte
+ * 2; an empty last slot is 0x82 (sign bit of the word set).  table_host must hold
  * SUB1_KERNEL_TABLE_MAX words; *table_words receives the number used.  Any
  * pointer may be NULL.
  */

@@ -51,7 +51,7 @@ constexpr int kGroupChunks = 8;      // chunks (32 codes) per partial sum, a mul
 constexpr int kSplitRing = 8;        // chunks in flight per lane where wavefronts share a slice
 constexpr int kMaxLen = 4096;        // codes per row: one per column pair at most
 constexpr int kCtrlHeader = 4;       // ctrl[0] ticket, [1] wait-limit hits, [2] bad expert ids
-constexpr uint32_t kIdleWord = 0x00040404u;  // three empty slots, no advance
+constexpr uint32_t kIdleWord = 0x82000404u;  // three empty slots, no advance
 
 // ------------------------------------------------------------- meta layout --
 //
@@ -270,7 +270,7 @@ __global__ __launch_bounds__(256) void checkpoint_kernel(
 #pragma unroll
     for (int q = 0; q < 4; q++) {
       uint32_t idx = min(cs[q], (cs[q] >> 3) + static_cast<uint32_t>(group_shift));
-      colw += table[idx] >> 24;
+      colw += (table[idx] >> 16) & 0xffu;
     }
   }
 }
@@ -320,14 +320,18 @@ struct PreparedArgs {
 // Slot offset 6m + 2q + sym-1 selects the value for the row-min sum (A) or the
 // row-max sum (B); offsets 4 and 5 read zeros.  28 zero columns follow the row
 // (digits of a last codeword that overhang the width, as the reference pads).
+// At least 22 pairs: dword 130 (pair 21) is the zero that empty last slots read.
+__host__ __device__ constexpr int activation_pairs(int width) {
+  return (width + 28 + 1) / 2 + 1 > 22 ? (width + 28 + 1) / 2 + 1 : 22;
+}
 __host__ __device__ constexpr int activation_dwords(int width) {
-  return 6 * ((width + 28 + 1) / 2 + 1);
+  return 6 * activation_pairs(width);
 }
 
 // Every load of a thread is in flight before its first LDS store, so a tile
 // pays one memory round trip for its activations, not one per pass.
 __device__ __forceinline__ void stage_activations(uint32_t *xa, const uint16_t *x, int width) {
-  const int npairs = (width + 28 + 1) / 2 + 1;
+  const int npairs = activation_pairs(width);
   const int step = blockDim.x;
   const bool aligned = (reinterpret_cast<uintptr_t>(x) & 3u) == 0;
   for (int m0 = threadIdx.x; m0 < npairs; m0 += 4 * step) {
@@ -408,10 +412,10 @@ __device__ __forceinline__ void lookup2(const uint32_t *tab, uint32_t pair, uint
   uint32_t w_lo = tab[idx.x];
   uint32_t w_hi = tab[idx.y];
   uint32_t sym = pair & 0x00070007u;
-  uint32_t b_lo = (sym & 0xffffu) * 0x4081u;   // bit j of the code -> bit 8j
-  uint32_t b_hi = (sym >> 16) * 0x4081u;
-  e_lo = (w_lo & ~0x00010101u) | (b_lo & 0x00010101u);
-  e_hi = (w_hi & ~0x00010101u) | (b_hi & 0x00010101u);
+  uint32_t b_lo = (sym & 0xffffu) * 0x400081u;   // bits 0, 1, 2 of the code -> bits 0, 8, 24
+  uint32_t b_hi = (sym >> 16) * 0x400081u;
+  e_lo = (w_lo & ~0x01000101u) | (b_lo & 0x01000101u);
+  e_hi = (w_hi & ~0x01000101u) | (b_hi & 0x01000101u);
   // one v_bfi each; the empty asm keeps the compiler from redoing the merge
   // for every byte it later extracts
   asm("" : "+v"(e_lo));
@@ -426,14 +430,19 @@ __device__ __forceinline__ void lookup4(const uint32_t *tab, uint2 w, uint32_t s
 
 __device__ __forceinline__ void add_codeword(uint32_t e, const uint32_t *xa, int &colw,
                                              float &s1, float &s2, const DotConsts &k) {
+  // slot 2 of a word whose sign bit is set is empty: the column is dropped from
+  // its address, and what is left (130 or 131) is a zero dword all lanes share
+  const int col2 = colw & ~(static_cast<int>(e) >> 31);
+  const int idx[3] = {colw + static_cast<int>(e & 0xffu),
+                      colw + static_cast<int>((e >> 8) & 0xffu),
+                      col2 + static_cast<int>(e >> 24)};
 #pragma unroll
   for (int j = 0; j < 3; j++) {
-    int idx = colw + static_cast<int>((e >> (8 * j)) & 0xffu);
-    bf16x2 v = __builtin_bit_cast(bf16x2, xa[idx]);
+    bf16x2 v = __builtin_bit_cast(bf16x2, xa[idx[j]]);
     s1 = __builtin_amdgcn_fdot2_f32_bf16(v, k.lo, s1, false);
     s2 = __builtin_amdgcn_fdot2_f32_bf16(v, k.hi, s2, false);
   }
-  colw += static_cast<int>(e >> 24);
+  colw += static_cast<int>((e >> 16) & 0xffu);
 }
 
 // This lane's chunk 0 of the slice that starts at chunk `base` of the stream.

@@ -130,13 +130,17 @@ extern "C" int sub1_build_tables(int32_t *dec_host, int32_t *trie_host) {
 //     of its own, and its code is chosen so that its low three bits agree
 //     with its symbols too (bits of empty slots are free).  This is what lets
 //     the kernel insert the code's low bits into the table word unconditionally.
-// Table word: byte j (j = 0..2) = slot j, the dword offset of that non-zero in
-// the activation array relative to the codeword's first column, with the
-// symbol bit cleared; byte 3 = 6 * pair count.  The activation array spends 6
-// dwords per column pair: [A_even, B_even, A_odd, B_odd, 0, 0], A = value
-// routed to the row-min sum, B = to the row-max sum, so a non-zero at in-code
-// position p = 2m + q with symbol s sits at 6m + 2q + (s - 1) and an empty slot
-// points at the zero pair, offset 4.
+// Table word: bytes 0, 1 and 3 = slots 0, 1 and 2, each the dword offset of a
+// non-zero in the activation array relative to the codeword's first column,
+// with the symbol bit cleared; byte 2 = 6 * pair count.  The activation array
+// spends 6 dwords per column pair: [A_even, B_even, A_odd, B_odd, 0, 0], A =
+// value routed to the row-min sum, B = to the row-max sum, so a non-zero at
+// in-code position p = 2m + q with symbol s sits at 6m + 2q + (s - 1).
+// Non-zeros fill the slots from slot 0; an empty slot 0 or 1 points at the zero
+// dwords of its own pair (offset 4).  Half of all codewords in a stream leave
+// slot 2 empty: such a word carries 0x82 there, bit 7 (the word's sign bit)
+// telling the kernel to drop the column from the address, so that all those
+// lanes read ONE dword (130, a zero of pair 21) and take no extra LDS bank.
 //
 // Slots are in column order, except that slots feeding different sums may be
 // swapped (that changes no sum's order of additions): the freedom is needed to
@@ -169,6 +173,7 @@ bool parse_entry(const Str &s, Parsed &p) {
 
 inline uint32_t slot_offset(int pos) { return 6u * (pos / 2) + 2u * (pos & 1); }
 constexpr uint32_t kEmptySlot = 4;
+constexpr uint32_t kEmptyLastSlot = 0x82;   // bit 7: empty; 128 + 2 = zero dword of pair 21
 
 struct Arrangement {
   int cls_mask;   // bits of the code class that are fixed
@@ -184,9 +189,11 @@ void arrangements(const Parsed &p, std::vector<Arrangement> &out) {
   do {
     // perm[i] = slot of non-zero i (only the first p.n matter)
     bool ok = true;
-    for (int a = 0; a < p.n && ok; a++)
+    for (int a = 0; a < p.n && ok; a++) {
+      if (perm[a] >= p.n) ok = false;   // empty slots come last
       for (int b = a + 1; b < p.n && ok; b++)
         if (p.sym[a] == p.sym[b] && perm[a] > perm[b]) ok = false;
+    }
     if (!ok) continue;
     Arrangement ar;
     ar.cls_mask = 0;
@@ -208,9 +215,9 @@ void arrangements(const Parsed &p, std::vector<Arrangement> &out) {
 }
 
 uint32_t table_word(const Parsed &p, const int slot_of[3]) {
-  uint32_t f[3] = {kEmptySlot, kEmptySlot, kEmptySlot};
+  uint32_t f[3] = {kEmptySlot, kEmptySlot, kEmptyLastSlot};
   for (int i = 0; i < p.n; i++) f[slot_of[i]] = slot_offset(p.pos[i]);
-  return f[0] | (f[1] << 8) | (f[2] << 16) | (static_cast<uint32_t>(6 * p.len) << 24);
+  return f[0] | (f[1] << 8) | (static_cast<uint32_t>(6 * p.len) << 16) | (f[2] << 24);
 }
 
 }  // namespace
@@ -275,46 +282,91 @@ extern "C" int sub1_build_kernel_tables(uint16_t *recode_host, uint32_t *table_h
   std::vector<uint16_t> recode(kCount);
   std::vector<uint32_t> table(words);
 
-  // singles: most constrained first, each to the admissible class with most room
+  // Singles: every code class (the code's low three bits) takes exactly nb / 8
+  // of them, and an entry fits a class if one of its arrangements agrees with
+  // the class's bits.  Entries with the same set of admissible classes are
+  // interchangeable, so the assignment is a small transportation problem
+  // (sets of classes x 8 classes), solved by augmenting paths; within a set the
+  // entries go to their classes in dictionary order, which makes the numbering
+  // canonical.
   std::vector<std::vector<Arrangement>> opts(nb);
-  std::vector<int> order(nb);
+  std::vector<int> admissible(nb, 0);
   for (int k = 0; k < nb; k++) {
     arrangements(ps[singles[k]], opts[k]);
-    order[k] = k;
-  }
-  auto classes_of = [&](int k) {
-    int m = 0;
     for (const Arrangement &a : opts[k])
       for (int c = 0; c < 8; c++)
-        if ((c & a.cls_mask) == a.cls_val) m |= 1 << c;
-    return __builtin_popcount(m);
-  };
-  std::vector<int> nclasses(nb);
-  for (int k = 0; k < nb; k++) nclasses[k] = classes_of(k);
-  std::stable_sort(order.begin(), order.end(),
-                   [&](int a, int b) { return nclasses[a] < nclasses[b]; });
-  // Classes 000 and 111 admit only entries whose non-zeros all feed one sum, so
-  // they are filled first; the one-bit and two-bit classes come after.
-  const int rank_of[8] = {0, 1, 1, 2, 1, 2, 2, 0};
-  int used[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if ((c & a.cls_mask) == a.cls_val) admissible[k] |= 1 << c;
+  }
   const int cap = nb / 8;
-  for (int k : order) {
-    int best_c = -1;
-    const Arrangement *best_a = nullptr;
-    for (const Arrangement &a : opts[k])
-      for (int c = 0; c < 8; c++) {
-        if ((c & a.cls_mask) != a.cls_val || used[c] >= cap) continue;
-        bool better = best_c < 0 || rank_of[c] < rank_of[best_c] ||
-                      (rank_of[c] == rank_of[best_c] && used[c] < used[best_c]);
-        if (better) {
-          best_c = c;
-          best_a = &a;
+  int supply[256] = {0};
+  for (int k = 0; k < nb; k++) supply[admissible[k]]++;
+  static int flow[256][8];
+  int load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int m = 0; m < 256; m++)
+    for (int c = 0; c < 8; c++) flow[m][c] = 0;
+  for (int m = 1; m < 256; m++) {
+    while (supply[m] > 0) {
+      // breadth-first search from set m for a class with room, moving units
+      // between classes through the sets that hold them
+      int from_set[8], via_class[8];
+      bool seen[8] = {false, false, false, false, false, false, false, false};
+      int queue[8], head = 0, tail = 0, found = -1;
+      for (int c = 0; c < 8; c++)
+        if (m >> c & 1) {
+          seen[c] = true;
+          from_set[c] = m;
+          via_class[c] = -1;
+          queue[tail++] = c;
+        }
+      while (head < tail && found < 0) {
+        const int c = queue[head++];
+        if (load[c] < cap) {
+          found = c;
+          break;
+        }
+        // class c is full: one of its units, from set t, may move to class d
+        for (int t = 1; t < 256; t++) {
+          if (!flow[t][c]) continue;
+          for (int d = 0; d < 8; d++)
+            if ((t >> d & 1) && !seen[d]) {
+              seen[d] = true;
+              from_set[d] = t;
+              via_class[d] = c;
+              queue[tail++] = d;
+            }
         }
       }
-    if (best_c < 0) return SUB1_ERR_INTERNAL;  // classes cannot be balanced
-    int code = best_c + 8 * used[best_c]++;
+      if (found < 0) return SUB1_ERR_INTERNAL;  // classes cannot be balanced
+      // push one unit along the path
+      int d = found;
+      load[d]++;
+      while (via_class[d] >= 0) {
+        const int t = from_set[d], c = via_class[d];
+        flow[t][d]++;
+        flow[t][c]--;
+        d = c;
+      }
+      flow[m][d]++;
+      supply[m]--;
+    }
+  }
+  int used[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int k = 0; k < nb; k++) {
+    const int m = admissible[k];
+    int c = 0;
+    while (c < 8 && !flow[m][c]) c++;
+    if (c == 8) return SUB1_ERR_INTERNAL;
+    flow[m][c]--;
+    const Arrangement *chosen = nullptr;
+    for (const Arrangement &a : opts[k])
+      if ((c & a.cls_mask) == a.cls_val) {
+        chosen = &a;
+        break;
+      }
+    if (!chosen) return SUB1_ERR_INTERNAL;
+    const int code = c + 8 * used[c]++;
     recode[singles[k]] = static_cast<uint16_t>(code);
-    table[code] = table_word(ps[singles[k]], best_a->slot_of);
+    table[code] = table_word(ps[singles[k]], chosen->slot_of);
   }
 
   const int identity[3] = {0, 1, 2};

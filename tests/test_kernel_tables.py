@@ -23,15 +23,19 @@ def decode_kernel_code(c, table, nb):
     idx = c if c < nb else nb + ((c - nb) >> 3)
     word = int(table[idx])
     slots = []
-    for j in range(3):
-        f = ((word >> (8 * j)) & 0xfe) | ((c >> j) & 1)       # low bit comes from the code
-        if f in (4, 5):
-            continue                                          # the zero pair: empty slot
+    empty_seen = False
+    for j, shift in enumerate((0, 8, 24)):                    # bytes 0, 1, 3 hold the slots
+        f = ((word >> shift) & 0xfe) | ((c >> j) & 1)         # low bit comes from the code
+        if f in (4, 5) and j < 2 or f in (0x82, 0x83) and j == 2:
+            empty_seen = True
+            continue                                          # a zero dword: empty slot
+        assert not empty_seen                                 # non-zeros fill the slots from slot 0
         m, rem = divmod(f, 6)
-        assert rem < 4
+        assert rem < 4 and f < 128
         slots.append((2 * m + rem // 2, 1 + (rem & 1)))
-    assert (word >> 24) % 6 == 0
-    return (word >> 24) // 6, slots
+    advance = (word >> 16) & 0xff
+    assert advance % 6 == 0
+    return advance // 6, slots
 
 
 def test_sizes_and_bijection():
