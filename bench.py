@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 counter runs of this same
 # command (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a 1 GiB device copy reads on
 # those counters); the summaries are under profiles/.  None where no run was made.
-MEASURED_TRAFFIC = {'c2048-sweep': 4.758e9 + 0.041e9}
+MEASURED_TRAFFIC = {'c2048-sweep': 4.758e9 + 0.040e9}
 
 WORKLOADS = {
     # name: (shape key, experts, p_zero, description)
