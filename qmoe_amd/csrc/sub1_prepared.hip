@@ -1016,14 +1016,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_small_kernel(Prepare
     int ticket;
     if (dynamic) {
       __syncthreads();   // the previous tile is done with s_ticket, x and the partial sums
-      if (threadIdx.x == 0) {
-        s_ticket = next_ticket;
-        if (next_ticket < n_all && n_all > static_cast<int>(gridDim.x))
-          next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
-                                               __HIP_MEMORY_SCOPE_AGENT);
-        else
-          next_ticket = n_all;
-      }
+      if (threadIdx.x == 0) s_ticket = next_ticket;
       __syncthreads();
       ticket = __builtin_amdgcn_readfirstlane(s_ticket);
     } else {
@@ -1035,8 +1028,18 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_small_kernel(Prepare
     const Tile tile = decode_tile(a, ticket, dynamic);
     const int kind = tile.kind, t = tile.t, e = tile.e;
     const KindArgs &k = a.k[kind];
+    // the next ticket is asked for late (see the streaming kernel), and not at
+    // all when every workgroup has exactly one tile
+    auto fetch_next = [&]() {
+      if (dynamic && threadIdx.x == 0)
+        next_ticket = n_all > static_cast<int>(gridDim.x)
+                          ? __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT)
+                          : n_all;
+    };
     if (a.kinds == 2 && kind == 1 && e < 0) {
       pass_through(a, k, t, tile.s_lo, tile.s_hi);
+      fetch_next();
       continue;
     }
     if (e >= 0) {
@@ -1047,6 +1050,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_small_kernel(Prepare
       await_activations(a, k, kind, t, xa);
       split_run(a, k, walk, tab, xa, dst, mode);
     }
+    fetch_next();
     if (a.kinds == 2 && kind == 0) publish_h(a, t);
   }
 }
