@@ -282,22 +282,37 @@ class PreparedStack:
 
 
 class PreparedMatrix:
-    """One compressed matrix (the three buffers of a Sub1Linear) copied into
-    the fast layout; `matvec_tokens(x, y)` does y[t] += W x[t] like
-    sub1matvec_tokens, in one launch with the decode table in LDS."""
+    """Compressed matrices of one shape copied into the fast layout;
+    `matvec_tokens(x, y)` does y[t] += W x[t] like sub1matvec_tokens, in one
+    launch with the decode table in LDS.
 
-    def __init__(self, dec, w_comp, row_off, ter_minmax, width):
+    One matrix: the three buffers of a Sub1Linear.  Several: pass lists of
+    equally shaped buffers (or stacked tensors plus `code_base`, int64 [count],
+    the first codeword of each matrix in `w_comp`); `matvec_tokens` then takes
+    `token_matrix`, int32 [T], the matrix each token uses."""
+
+    def __init__(self, dec, w_comp, row_off, ter_minmax, width, code_base=None):
         lib = _lib.load()
         dev = dec.device
-        height = row_off.numel() - 1
-        self.device, self.height, self.width = dev, height, width
+        if isinstance(w_comp, (list, tuple)):
+            sizes = torch.tensor([0] + [t.numel() for t in w_comp], dtype=torch.int64)
+            code_base = sizes.cumsum(0)[:-1].to(dev)
+            w_comp, row_off, ter_minmax = (torch.cat(list(v)) for v in (w_comp, row_off, ter_minmax))
+        count = 1 if code_base is None else code_base.numel()
+        if row_off.numel() % count:
+            raise ValueError('row_off does not hold %d equal parts' % count)
+        height = row_off.numel() // count - 1
+        self.device, self.count, self.height, self.width = dev, count, height, width
         src = _lib.MatrixSet(
             _need(dec, torch.int32, 'dec', numel=_lib.DEC_WORDS),
-            _need(w_comp, torch.int16, 'w_comp', dev), None,
-            _need(row_off, torch.int32, 'row_off', dev),
-            _need(ter_minmax, torch.bfloat16, 'ter_minmax', dev, numel=2 * height),
-            1, height, width)
-        meta_bytes = lib.sub1_matrix_prepared_meta_bytes(1, height, width)
+            _need(w_comp, torch.int16, 'w_comp', dev),
+            None if code_base is None else _need(code_base, torch.int64, 'code_base', dev),
+            _need(row_off, torch.int32, 'row_off', dev, numel=count * (height + 1)),
+            _need(ter_minmax, torch.bfloat16, 'ter_minmax', dev, numel=count * 2 * height),
+            count, height, width)
+        meta_bytes = lib.sub1_matrix_prepared_meta_bytes(count, height, width)
+        if meta_bytes <= 0:
+            raise ValueError('bad matrix dimensions')
         self.meta = torch.empty(meta_bytes, dtype=torch.uint8, device=dev)
         self._c = _lib.MatrixPrepared()
         with torch.cuda.device(dev):
@@ -308,15 +323,19 @@ class PreparedMatrix:
             _lib.check(lib.sub1_matrix_prepare_codes(ctypes.byref(src), ctypes.byref(self._c),
                                                      _stream()))
 
-    def matvec_tokens(self, x, y):
+    def matvec_tokens(self, x, y, token_matrix=None):
         dev = self.device
         p_x = _need(x, torch.bfloat16, 'x', dev, dim=2)
         p_y = _need(y, torch.bfloat16, 'y', dev, dim=2)
         tokens = x.shape[0]
         if x.shape[1] != self.width or y.shape != (tokens, self.height):
             raise ValueError('x must be [T, %d] and y [T, %d]' % (self.width, self.height))
+        if token_matrix is None and self.count > 1:
+            raise ValueError('token_matrix is required with %d matrices' % self.count)
+        p_tm = None if token_matrix is None else _need(token_matrix, torch.int32, 'token_matrix',
+                                                       dev, numel=tokens)
         if tokens == 0:
             return
         with torch.cuda.device(dev):
             _lib.check(_lib.load().sub1_matvec_prepared(
-                ctypes.byref(self._c), None, p_x, self.width, p_y, self.height, tokens, _stream()))
+                ctypes.byref(self._c), p_tm, p_x, self.width, p_y, self.height, tokens, _stream()))

@@ -520,3 +520,28 @@ def test_sub1linear_prepared_copy_follows_the_buffers(gpu, oracle):
         fresh.copy_(nb[n])
         getattr(a, n).data = fresh
     assert torch.equal(a(x), yb)
+
+
+def test_prepared_matrix_set_with_token_matrix(gpu, oracle):
+    """Several matrices of one shape behind one launch: token t uses matrix
+    token_matrix[t]; a token whose index names no matrix adds nothing."""
+    sub1, op = gpu
+    height, width, count = 130, 200, 3
+    cases = [dev_case(oracle, height, width, 0.8, seed=950 + i) for i in range(count)]
+    pm = op.PreparedMatrix(sub1.DEC[0], [c['w_comp'] for c in cases],
+                           [c['row_off_d'] for c in cases], [c['mm_d'] for c in cases], width)
+    which = [0, 2, 1, 1, -1, 0, 7, 2, 2, 0, 1]
+    xs = np.stack([so.synthetic_activation(width, 970 + i) for i in range(len(which))])
+    y0 = np.stack([so.synthetic_activation(height, 990 + i) for i in range(len(which))])
+    y = bf16_dev(y0).clone()
+    pm.matvec_tokens(bf16_dev(xs), y, torch.tensor(which, dtype=torch.int32, device='cuda'))
+    got = bits_host(y)
+    for t, m in enumerate(which):
+        if m < 0 or m >= count:
+            assert np.array_equal(got[t], y0[t])
+        else:
+            c = cases[m]
+            want = oracle.matvec_seq(c['codes'], c['row_off'], c['mm'], xs[t], y=y0[t])
+            assert np.array_equal(got[t], want), (t, m)
+    with pytest.raises(ValueError):
+        pm.matvec_tokens(bf16_dev(xs), y)            # several matrices need token_matrix
