@@ -1483,8 +1483,23 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   // h in LDS, if table + x + h fit.
   const size_t lds_fused = (static_cast<size_t>(a.table_words) + activation_dwords(a.k[0].width) +
                             activation_dwords(a.k[1].width)) * 4;
-  const bool fused = p.kinds == 2 && !small && a.k[0].parts == 1 && a.k[1].parts == 1 &&
-                     lds_fused <= lds_limit;
+  bool fused = p.kinds == 2 && !small && a.k[0].parts == 1 && a.k[1].parts == 1 &&
+               lds_fused <= lds_limit;
+  if (!fused && p.kinds == 2 && lds_fused <= lds_limit && tokens >= 16 && tokens < cus) {
+    // Fewer tokens than compute units: whole tokens per workgroup leave units
+    // idle but pay nothing for cutting the matrices (per-tile staging, h through
+    // memory, waiting).  Measured on the Switch shapes, the cut versions take
+    // about 33 us + tokens / units x (time of one token on one unit), the fused
+    // kernel the time of one token, itself about 8 us + codewords / 5500 per us.
+    const double token_us = 8.0 + static_cast<double>(p.total_chunks) * 256.0 / p.count / 5500.0;
+    if (tokens >= cus * (1.0 - 33.0 / token_us)) {
+      fused = true;
+      for (int i = 0; i < 2; i++) {
+        a.k[i].parts = 1;
+        a.k[i].split = 1;
+      }
+    }
+  }
   if (fused) {
     a.xdwords = activation_dwords(a.k[0].width);
     a.hdwords = activation_dwords(a.k[1].width);
