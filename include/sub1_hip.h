@@ -56,23 +56,6 @@ int sub1_abi_version(void);
 int sub1_build_tables(int32_t *dec_host, int32_t *trie_host);
 
 /*
- * The tables the prepared-stack kernels decode with, built on the HOST (no
- * counterpart in the reference, which decodes from `dec` in global memory,
- * sub1_cuda_kernel.cu:188).  Codes are renumbered so that the decode table
- * fits LDS: recode_host[65536] maps a dictionary index to its kernel code;
- * codes below *single_codes index table_host directly, a code c at or above it
- * uses word *single_codes + ((c - *single_codes) >> 3) and its low three bits
- * are the symbol bits of the three slots.  A table word holds the slots'
- * activation offsets in bytes 0, 1 and 3 and six times the pair count in byte
- * 2; an empty last slot is 0x82 (sign bit of the word set).  table_host must hold
- * SUB1_KERNEL_TABLE_MAX words; *table_words receives the number used.  Any
- * pointer may be NULL.
- */
-#define SUB1_KERNEL_TABLE_MAX 16384
-int sub1_build_kernel_tables(uint16_t *recode_host, uint32_t *table_host,
-                             int32_t *single_codes, int32_t *table_words);
-
-/*
  * y[r] += bf16( sum_k deq(w[r,k]) * x[k] ),  fp32 accumulation, for any
  * height >= 1 and 1 <= width <= SUB1_MAX_WIDTH.  Replaces `sub1matvec`
  * (reference sub1_cuda.cpp:35-45, sub1_cuda_kernel.cu:70-88,129-202), which
@@ -168,12 +151,26 @@ int sub1_moe_grouped(const sub1_moe_stack *stack, const int32_t *token_expert,
 
 /*
  * Prepared stack: the fast form of sub1_moe_grouped (no counterpart in the
- * reference).  Preparing copies the stack once into a layout the GPU streams
- * at full width - rows ordered by code count and cut into 64-row slices, each
- * slice's codes interleaved 8 bytes per lane, codes renumbered as
- * sub1_build_kernel_tables describes - after which the decode table (61.5 KB)
- * and the activations both live in LDS.  Only for the fixed dictionary (dec is
- * compared with it, once) and 1 <= d_model, d_ff <= SUB1_PREPARED_MAX_WIDTH.
+ * reference).  Preparing decodes the stack once and stores every row's
+ * non-zero weights as a gap-coded stream the GPU walks at full width:
+ *
+ *   - a position j counts dwords of the activation array the kernels keep in
+ *     LDS: dword 0 is zero, column c has (x[c], 0) at 3c+1 (read for a row-min
+ *     weight), (0, x[c]) at 3c+2 (row-max weight) and a zero at 3c+3;
+ *   - a row is a sequence of 7-bit entries, each the step from the row's
+ *     position to the next: to the next non-zero weight's dword, or, where
+ *     that is more than 127 away, to the farthest zero dword within reach;
+ *     after its last non-zero a row steps to the next zero dword (if it is
+ *     not on one) and pads with steps of 0;
+ *   - nine entries make a chunk (8 bytes, entry q in bits 7q..7q+6, bit 63
+ *     zero); rows are ordered by chunk count and cut into 64-row slices, each
+ *     as long as its longest row and at least one chunk; chunk c of lane l of
+ *     a slice sits at byte (slice_base * 64 + c * 64 + l) * 8 of `codes`.
+ *
+ * With 10% non-zero weights this takes 0.72 bit per weight (the dictionary
+ * codes: 0.69), and a weight costs the kernel one LDS read and one
+ * multiply-add.  Only for the fixed dictionary (dec is compared with it, once)
+ * and 1 <= d_model, d_ff <= SUB1_PREPARED_MAX_WIDTH.
  *
  *   meta_bytes = sub1_moe_prepared_meta_bytes(experts, d_model, d_ff);
  *   sub1_moe_prepared p;
@@ -185,9 +182,17 @@ int sub1_moe_grouped(const sub1_moe_stack *stack, const int32_t *token_expert,
  * meta and codes are device buffers the caller owns, 256-byte aligned; the
  * original stack is not referenced after sub1_moe_prepare_codes has run.
  * sub1_moe_grouped_prepared has the semantics of sub1_moe_grouped and the same
- * workspace; every row's sums are taken in the same order, so outputs are
- * identical.  With few tokens several wavefronts share a row slice (the code
- * buffer carries column checkpoints for that); the results do not change.
+ * workspace.  A row's result is the fp32 sum of x[c] * w[r, c] over its
+ * non-zero weights, taken in groups of 72 entries (8 chunks): a partial sum
+ * per group from zero, the partial sums added first group first; the same bits
+ * for every batch size.  With few tokens several wavefronts share a row slice
+ * (the buffer carries position checkpoints for that); the results do not
+ * change.
+ *
+ * sub1_moe_prepared_decode writes the symbols (0, 1 = row min, 2 = row max) of
+ * one matrix, read back from the stream, to tern_out (uint8 [rows, width] on
+ * the device; projection 0 = wi, 1 = wo): the check that preparing kept every
+ * weight.
  */
 #define SUB1_PREPARED_MAX_WIDTH 8192
 
@@ -196,7 +201,7 @@ typedef struct sub1_moe_prepared {
   const void *codes;
   int64_t meta_bytes;
   int64_t code_bytes;
-  int64_t total_chunks;    /* 512-byte chunk rows of the code stream; checkpoints follow */
+  int64_t total_chunks;    /* 512-byte chunk rows of the entry stream; checkpoints follow */
   int32_t experts;
   int32_t d_model;
   int32_t d_ff;
@@ -214,6 +219,9 @@ int sub1_moe_prepare_codes(const sub1_moe_stack *stack, const sub1_moe_prepared 
 int sub1_moe_grouped_prepared(const sub1_moe_prepared *prepared, const int32_t *token_expert,
                               const void *x, void *y, int tokens, void *workspace,
                               int64_t workspace_bytes, void *stream);
+
+int sub1_moe_prepared_decode(const sub1_moe_prepared *prepared, int expert, int projection,
+                             void *tern_out, void *stream);
 
 /*
  * The same preparation for plain products: `count` matrices of one shape
@@ -264,6 +272,9 @@ int sub1_matvec_prepared(const sub1_matrix_prepared *prepared, const int32_t *to
                          const void *x, int64_t ldx, void *y, int64_t ldy, int tokens,
                          void *stream);
 
+int sub1_matrix_prepared_decode(const sub1_matrix_prepared *prepared, int matrix,
+                                void *tern_out, void *stream);
+
 /*
  * Average duration in microseconds of the most recent launches, measured with
  * HIP events on the launch stream: call sub1_timing_begin(stream) before and
@@ -279,7 +290,7 @@ int sub1_timing_end(void *stream, double *elapsed_us);
  * random dword per lane from a table of `words` dwords (a power of two), held
  * in LDS (from_lds != 0, words <= 32768) or in global memory, with 16
  * wavefronts per compute unit and four gathers in flight per lane, as in the
- * decode loop.  Allocates and frees its own buffers; synchronises.
+ * kernels' inner loop.  Allocates and frees its own buffers; synchronises.
  */
 int sub1_probe_gather(int from_lds, int words, int steps, double *ns_per_gather, void *stream);
 

@@ -15,6 +15,12 @@
  *   sub1o_dequant        test.py:110, sub1_cuda_kernel.cu:156-157,170-171
  *   sub1o_matvec_lanes   sub1_cuda_kernel.cu:143-201 (lane order, tree, y +=)
  *   sub1o_matvec_seq     same sums, taken per symbol, in groups of 32 codes
+ *   sub1o_gap_entries    a row's non-zero weights as the 7-bit gap entries of
+ *                        the library's prepared stream (no reference lines:
+ *                        the format is the library's own; pinned by decoding
+ *                        the entries back to the row)
+ *   sub1o_matvec_gap     same sums, one fused multiply-add per entry, in
+ *                        groups of 72 entries
  *   sub1o_matvec_f64     textbook GEMV in double on the decoded matrix
  *   sub1o_expert_ffn     sub1.py:132-143 twice with ReLU between (the
  *                        DenseActDense call made at sub1.py:317)
@@ -365,6 +371,85 @@ void sub1o_matvec_seq(const int32_t *dec, const uint16_t *codes,
   }
 }
 
+/* The prepared stream's view of a row.  A position j counts dwords of an
+ * activation array with a zero at 0 and, per column c, x[c] for a row-min
+ * weight at 3c+1, x[c] for a row-max weight at 3c+2, a zero at 3c+3.  The row
+ * is the sequence of steps (0..127) that visits its non-zero weights in column
+ * order: a step to a non-zero more than 127 away first goes to the farthest
+ * zero within reach (the largest multiple of 3 not beyond j+127), repeatedly;
+ * after the last non-zero one step goes to the next zero unless the row stands
+ * on one.  Writes the steps to out (if not NULL; at most cap) and returns their
+ * number, or -1 if the codes do not cover ceil(width/2) pairs. */
+#define SUB1O_GAP_MAX 127
+
+int sub1o_gap_entries(const int32_t *dec, const uint16_t *codes, int ncodes,
+                      int width, uint8_t *out, int cap) {
+  int n = 0, j = 0, idx = 0;
+  for (int c = 0; c < ncodes; c++) {
+    int e = codes[c];
+    int npairs = dec[2 * e] & 0xf;
+    for (int d = 0; d < 2 * npairs && idx + d < width; d++) {
+      int t = entry_digit(dec, e, d);
+      if (!t) continue;
+      int target = 3 * (idx + d) + t;
+      while (target - j > SUB1O_GAP_MAX) {
+        int z = (j + SUB1O_GAP_MAX) / 3 * 3;
+        if (out && n < cap) out[n] = (uint8_t)(z - j);
+        n++;
+        j = z;
+      }
+      if (out && n < cap) out[n] = (uint8_t)(target - j);
+      n++;
+      j = target;
+    }
+    idx += 2 * npairs;
+  }
+  if (idx != ((width + 1) & ~1)) return -1;
+  if (j % 3) {
+    if (out && n < cap) out[n] = (uint8_t)(3 - j % 3);
+    n++;
+  }
+  return n;
+}
+
+/* The product in the order the prepared-stream kernels add: the row's entries
+ * in groups of SUB1O_GAP_GROUP; within a group each entry that stands on an
+ * activation adds x * w (w = row min or max) with one fused multiply-add onto a
+ * partial sum that starts at zero (entries on a zero dword add nothing); the
+ * partial sums are added, first group first, onto the row's sum; bf16; +=. */
+#define SUB1O_GAP_GROUP 72
+
+int sub1o_matvec_gap(const int32_t *dec, const uint16_t *codes,
+                     const int32_t *row_off, const uint16_t *ter_minmax,
+                     const uint16_t *x, uint16_t *y, int height, int width) {
+  int cap = width + width / 40 + 8;
+  uint8_t *steps = (uint8_t *)malloc((size_t)cap);
+  for (int r = 0; r < height; r++) {
+    int n = sub1o_gap_entries(dec, codes + row_off[r], row_off[r + 1] - row_off[r],
+                              width, steps, cap);
+    if (n < 0 || n > cap) {
+      free(steps);
+      return 1 + r;
+    }
+    float w[3] = {0.f, bf16_to_f32(ter_minmax[2 * r]), bf16_to_f32(ter_minmax[2 * r + 1])};
+    float sum = 0.f;
+    int j = 0;
+    for (int i0 = 0; i0 < n; i0 += SUB1O_GAP_GROUP) {
+      float p = 0.f;
+      int i1 = i0 + SUB1O_GAP_GROUP < n ? i0 + SUB1O_GAP_GROUP : n;
+      for (int i = i0; i < i1; i++) {
+        j += steps[i];
+        if (j % 3) p = fmaf(bf16_to_f32(x[j / 3]), w[j % 3], p);
+      }
+      sum += p;
+    }
+    float acc = bf16_to_f32(y[r]) + bf16_to_f32(f32_to_bf16(sum));
+    y[r] = f32_to_bf16(acc);
+  }
+  free(steps);
+  return 0;
+}
+
 /* Dense double-precision product of the decoded matrix with x, and the sum of
  * |w*x| per row that bounds any fp32 summation order's error. */
 void sub1o_matvec_f64(const uint8_t *tern, const uint16_t *ter_minmax,
@@ -387,7 +472,7 @@ void sub1o_matvec_f64(const uint8_t *tern, const uint16_t *ter_minmax,
 /* One expert FFN on one token as the model runs it (sub1.py:317 calls
  * wo(relu(wi(x))), each projection through sub1.py:132-143: zeroed bf16
  * output, one matvec).  h is bf16 between the stages.  order: 0 = lane order,
- * 1 = per-symbol stream order.  h_out may be NULL. */
+ * 1 = per-symbol stream order, 2 = prepared-stream order.  h_out may be NULL. */
 void sub1o_expert_ffn(const int32_t *dec,
                       const uint16_t *wi_codes, const int32_t *wi_row_off,
                       const uint16_t *wi_minmax,
@@ -398,15 +483,19 @@ void sub1o_expert_ffn(const int32_t *dec,
   uint16_t *h = (uint16_t *)calloc((size_t)d_ff, sizeof(uint16_t));
   if (order == 0)
     sub1o_matvec_lanes(dec, wi_codes, wi_row_off, wi_minmax, x, h, d_ff, d_model);
-  else
+  else if (order == 1)
     sub1o_matvec_seq(dec, wi_codes, wi_row_off, wi_minmax, x, h, d_ff, d_model);
+  else
+    sub1o_matvec_gap(dec, wi_codes, wi_row_off, wi_minmax, x, h, d_ff, d_model);
   for (int i = 0; i < d_ff; i++)
     if (h[i] & 0x8000u) h[i] = 0; /* relu; -0 -> +0 as max(x,0) gives */
   if (h_out) memcpy(h_out, h, (size_t)d_ff * sizeof(uint16_t));
   memset(y, 0, (size_t)d_model * sizeof(uint16_t));
   if (order == 0)
     sub1o_matvec_lanes(dec, wo_codes, wo_row_off, wo_minmax, h, y, d_model, d_ff);
-  else
+  else if (order == 1)
     sub1o_matvec_seq(dec, wo_codes, wo_row_off, wo_minmax, h, y, d_model, d_ff);
+  else
+    sub1o_matvec_gap(dec, wo_codes, wo_row_off, wo_minmax, h, y, d_model, d_ff);
   free(h);
 }

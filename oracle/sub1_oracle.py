@@ -201,6 +201,10 @@ class COracle:
             f = getattr(L, name)
             f.argtypes = [vp] * 6 + [ctypes.c_int, ctypes.c_int]
             f.restype = None
+        L.sub1o_matvec_gap.argtypes = [vp] * 6 + [ctypes.c_int, ctypes.c_int]
+        L.sub1o_matvec_gap.restype = ctypes.c_int
+        L.sub1o_gap_entries.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int, vp, ctypes.c_int]
+        L.sub1o_gap_entries.restype = ctypes.c_int
         L.sub1o_matvec_f64.argtypes = [vp] * 5 + [ctypes.c_int, ctypes.c_int]
         L.sub1o_matvec_f64.restype = None
         L.sub1o_expert_ffn.argtypes = [vp] * 10 + [ctypes.c_int] * 3
@@ -288,6 +292,24 @@ class COracle:
         """Per-symbol stream-order arithmetic; returns y."""
         return self._matvec(self.lib.sub1o_matvec_seq, codes, row_off,
                             ter_minmax, x, y, dec)
+
+    def matvec_gap(self, codes, row_off, ter_minmax, x, y=None, dec=None):
+        """Prepared-stream order (groups of 72 gap entries, one fused
+        multiply-add per entry); returns y."""
+        return self._matvec(self.lib.sub1o_matvec_gap, codes, row_off,
+                            ter_minmax, x, y, dec)
+
+    def gap_entries(self, row_codes, width, dec=None):
+        """uint8 steps of one row's prepared stream."""
+        dec = self.tables()[0] if dec is None else dec
+        row_codes = np.ascontiguousarray(row_codes, dtype=np.uint16)
+        cap = width + width // 40 + 8
+        out = np.zeros(cap, dtype=np.uint8)
+        n = self.lib.sub1o_gap_entries(self._p(dec), self._p(row_codes), row_codes.shape[0],
+                                       width, self._p(out), cap)
+        if n < 0 or n > cap:
+            raise ValueError('the codes do not cover the width')
+        return out[:n].copy()
 
     def matvec_f64(self, tern, ter_minmax, x):
         """-> (y float64 [H], sum |w*x| float64 [H]) on the decoded matrix."""

@@ -52,7 +52,6 @@ PROTOTYPES = {
     'sub1_last_error': (ctypes.c_char_p, []),
     'sub1_abi_version': (_int, []),
     'sub1_build_tables': (_int, [_vp, _vp]),
-    'sub1_build_kernel_tables': (_int, [_vp, _vp, _vp, _vp]),
     'sub1_matvec': (_int, [_vp] * 6 + [_int, _int, _vp]),
     'sub1_matvec_tokens': (_int, [_vp] * 6 + [_int, _int, _int, _i64, _i64, _vp]),
     'sub1_pack_count': (_int, [_vp, _vp, _vp, _int, _int, _vp]),
@@ -68,6 +67,7 @@ PROTOTYPES = {
                                       _vp]),
     'sub1_moe_grouped_prepared': (_int, [ctypes.POINTER(MoePrepared), _vp, _vp, _vp, _int,
                                          _vp, _i64, _vp]),
+    'sub1_moe_prepared_decode': (_int, [ctypes.POINTER(MoePrepared), _int, _int, _vp, _vp]),
     'sub1_matrix_prepared_meta_bytes': (_i64, [_int, _int, _int]),
     'sub1_matrix_prepare_layout': (_int, [ctypes.POINTER(MatrixSet), _vp, _i64,
                                           ctypes.POINTER(MatrixPrepared), _vp]),
@@ -75,6 +75,7 @@ PROTOTYPES = {
                                          ctypes.POINTER(MatrixPrepared), _vp]),
     'sub1_matvec_prepared': (_int, [ctypes.POINTER(MatrixPrepared), _vp, _vp, _i64, _vp, _i64,
                                     _int, _vp]),
+    'sub1_matrix_prepared_decode': (_int, [ctypes.POINTER(MatrixPrepared), _int, _vp, _vp]),
     'sub1_timing_begin': (_int, [_vp]),
     'sub1_timing_end': (_int, [_vp, ctypes.POINTER(ctypes.c_double)]),
     'sub1_probe_gather': (_int, [_int, _int, _int, ctypes.POINTER(ctypes.c_double), _vp]),

@@ -4,27 +4,33 @@
 // (reference sub1.py:114-130: one row-major code stream per matrix plus
 // row_off) into a form the GPU can stream at full width:
 //
-//   * rows of every matrix are ordered by code count and cut into slices of
+//   * every row's dictionary codes are decoded once and its non-zero weights
+//     written as a gap-coded stream: 7-bit entries, each the distance to the
+//     next non-zero in units of the LDS activation array (3 dwords per column:
+//     the activation for a row-min weight, for a row-max weight, a zero), so an
+//     entry names the column and the symbol at once; gaps beyond 127 units step
+//     over zero dwords.  At 10% non-zeros this is 0.72 bit per weight against
+//     0.69 for the dictionary codes, and the kernel needs no decode table;
+//   * rows of every matrix are ordered by entry count and cut into slices of
 //     64 rows (one wavefront lane each);
-//   * a slice's codes are interleaved in chunks of 4 codes (8 bytes) per lane:
+//   * a slice's entries are interleaved in chunks of 9 (8 bytes) per lane:
 //     chunk c of lane l sits at slice_base*512 + (c*64 + l)*8 bytes, so one
 //     wavefront load fetches 512 contiguous bytes and every byte of a cache
-//     line is used; lanes are padded to the slice's longest row (about 2%);
-//   * codes are renumbered (sub1_build_kernel_tables) so that the decode table
-//     is 61.5 KB and lives in LDS next to the activations.
+//     line is used; lanes are padded to the slice's longest row with entries
+//     that stay on a zero dword.
 //
-// The kernels then walk 64 rows per wavefront: per codeword one LDS table read
-// and three LDS activation reads, each folded into two running sums
-// (activations under row-min weights, under row-max weights) with
-// v_dot2c_f32_bf16 on (x,0)/(0,x) bf16 pairs; no cross-lane traffic at all.
-// They compute what reference sub1_cuda_kernel.cu:163-201 computes per row.
+// The kernels then walk 64 rows per wavefront: per entry one address add, one
+// LDS read of a bf16 pair (x, 0) or (0, x), and one v_dot2c_f32_bf16 with the
+// row's (min, max) pair, which adds x * min or x * max onto the row's fp32 sum;
+// no cross-lane traffic at all.  They compute what reference
+// sub1_cuda_kernel.cu:163-201 computes per row.
 // Three kernels share that loop and give the same bits:
 // moe_prepared_fused_kernel streams whole tokens (wi, ReLU, wo in one
 // workgroup, h kept in LDS) when there is at least a token per compute unit;
 // moe_prepared_kernel streams tiles of one matrix (persistent grid, a wavefront
 // per slice, the next slice's loads in flight) for smaller batches and for
 // single matrices; moe_prepared_small_kernel is the latency form for a handful
-// of tokens (wavefronts share a slice from column checkpoints).
+// of tokens (wavefronts share a slice from position checkpoints).
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -40,18 +46,18 @@ using sub1::bf16_to_f32;
 using sub1::f32_to_bf16;
 using sub1::fail;
 using sub1::misaligned;
-using sub1::row_result;
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kMaxThreads = 1024;    // 16 wavefronts per workgroup
-constexpr int kChunk = 4;            // codes per lane per chunk
+constexpr int kFields = 9;           // entries per lane per chunk (7 bits each in 8 bytes)
+constexpr int kFieldBits = 7;
+constexpr int kMaxStep = 127;        // the largest entry
 constexpr int kRing = 4;             // chunks in flight per lane (2 KB per wavefront)
-constexpr int kGroupChunks = 8;      // chunks (32 codes) per partial sum, a multiple of kRing
+constexpr int kGroupChunks = 8;      // chunks (72 entries) per partial sum, a multiple of kRing
 constexpr int kSplitRing = 8;        // chunks in flight per lane where wavefronts share a slice
-constexpr int kMaxLen = 4096;        // codes per row: one per column pair at most
+constexpr int kMaxRowChunks = 4096;  // chunks per row the row ordering can count
 constexpr int kCtrlHeader = 4;       // ctrl[0] ticket, [1] wait-limit hits, [2] bad expert ids
-constexpr uint32_t kIdleWord = 0x82000404u;  // three empty slots, no advance
 
 // ------------------------------------------------------------- meta layout --
 //
@@ -60,8 +66,7 @@ constexpr uint32_t kIdleWord = 0x82000404u;  // three empty slots, no advance
 struct KindMeta {
   int64_t slice_base;   // u32 [E*S] (+1): this kind's part of the scanned counts
   int64_t slice_nch;    // u16 [E*S]
-  int64_t slice_nfull;  // u16 [E*S]
-  int64_t row_len;      // u16 [E*S*64]
+  int64_t row_chunks;   // u16 [E*H]: chunks of every row, in the matrix's own row order
   int64_t row_idx;      // u16 [E*S*64]
   int64_t minmax;       // u32 [E*S*64]
   int slices;           // S
@@ -72,8 +77,8 @@ struct MetaLayout {
   KindMeta k[2];
   int kinds;
   int64_t counts;       // i32 [all slices + 1] chunk counts, scanned in place
-  int64_t status;       // i32 [4]: [0] rows with a bad code count, [1], [2] longest slice
-                        // of kind 0 / 1 in chunks
+  int64_t status;       // i32 [4]: [0] rows whose codes do not cover the width, [1], [2]
+                        // longest slice of kind 0 / 1 in chunks
   int64_t bytes;
 };
 
@@ -101,8 +106,7 @@ MetaLayout meta_layout(int experts, int kinds, const int height[2], const int wi
     first[i] = nslices;
     nslices += es;
     k.slice_nch = take(es * 2);
-    k.slice_nfull = take(es * 2);
-    k.row_len = take(es * 64 * 2);
+    k.row_chunks = take(static_cast<int64_t>(experts) * height[i] * 2);
     k.row_idx = take(es * 64 * 2);
     k.minmax = take(es * 64 * 4);
   }
@@ -125,62 +129,136 @@ MetaLayout matrix_layout(int count, int height, int width) {
 
 // ---------------------------------------------------------- prepare kernels --
 
-// One workgroup per matrix: order the rows by code count, longest first, and
+// Calls nz(column, symbol) for every non-zero weight of a row, in column order,
+// and returns the columns the row's codes cover.  Digit d of dictionary entry e
+// is (dec[2e + d/14] >> (4 + 2 (d % 14))) & 3, the low nibble of dec[2e] the
+// entry's pair count (reference sub1.py:60-72, sub1_cuda_kernel.cu:186-192).
+template <class F>
+__device__ __forceinline__ int for_each_nonzero(const uint16_t *codes, int n,
+                                                const int32_t *__restrict__ dec, int width,
+                                                F &&nz) {
+  int col = 0;
+  for (int i = 0; i < n; i++) {
+    const int e = codes[i];
+    const uint32_t w0 = static_cast<uint32_t>(dec[2 * e]);
+    const uint32_t w1 = static_cast<uint32_t>(dec[2 * e + 1]);
+    unsigned long long digits = static_cast<unsigned long long>(w0 >> 4) |
+                                (static_cast<unsigned long long>(w1 >> 4) << 28);
+    while (digits) {
+      const int d = (__ffsll(digits) - 1) >> 1;
+      const int sym = static_cast<int>(digits >> (2 * d)) & 3;
+      digits &= ~(3ull << (2 * d));
+      if (col + d < width) nz(col + d, sym);   // digits past the width are dropped
+    }
+    col += 2 * static_cast<int>(w0 & 15u);
+  }
+  return col;
+}
+
+// Non-zeros to entries.  The position j counts dwords of the LDS activation
+// array: 0 is a zero, column c has x for a row-min weight at 1 + 3c, for a
+// row-max weight at 2 + 3c, and a zero at 3 + 3c.  An entry is the step to the
+// next position, 0..127.  A longer gap goes over zeros (every third dword), as
+// far as each step reaches; after the last non-zero the row parks on the next
+// zero, where steps of 0 pad it to the length of its slice.
+struct EntryWriter {
+  int j = 0;
+  template <class E>
+  __device__ __forceinline__ void nonzero(int col, int sym, E &&emit) {
+    const int target = 3 * col + sym;
+    while (target - j > kMaxStep) {
+      const int z = (j + kMaxStep) / 3 * 3;
+      emit(z - j, j);
+      j = z;
+    }
+    emit(target - j, j);
+    j = target;
+  }
+  template <class E>
+  __device__ __forceinline__ void park(E &&emit) {
+    const int z = (j + 2) / 3 * 3;
+    if (z != j) emit(z - j, j);
+    j = z;
+  }
+};
+
+__device__ __forceinline__ const uint16_t *row_codes(const uint16_t *src, const int64_t *code_base,
+                                                     const int32_t *row_off_all, int e, int r,
+                                                     int height, int width, int &n) {
+  const int32_t *ro = row_off_all + static_cast<int64_t>(e) * (height + 1);
+  n = ro[r + 1] - ro[r];
+  if (n < 1 || n > (width + 1) / 2) n = 0;   // counted as a bad row by count_entries_kernel
+  return src + (code_base ? code_base[e] : 0) + ro[r];   // one matrix: no base array
+}
+
+// One thread per row: how many chunks its entries fill.
+__global__ __launch_bounds__(256) void count_entries_kernel(
+    const uint16_t *__restrict__ src, const int64_t *__restrict__ code_base,
+    const int32_t *__restrict__ row_off_all, const int32_t *__restrict__ dec,
+    uint16_t *__restrict__ row_chunks, int32_t *__restrict__ status, int height, int width,
+    int64_t rows_total) {
+  const int64_t g = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (g >= rows_total) return;
+  const int e = static_cast<int>(g / height);
+  const int r = static_cast<int>(g % height);
+  int n;
+  const uint16_t *codes = row_codes(src, code_base, row_off_all, e, r, height, width, n);
+  int entries = 0;
+  auto emit = [&](int, int) { entries++; };
+  EntryWriter wr;
+  const int covered =
+      for_each_nonzero(codes, n, dec, width, [&](int col, int sym) { wr.nonzero(col, sym, emit); });
+  wr.park(emit);
+  // a row's codes cover its width rounded up to a whole pair, exactly
+  if (covered != ((width + 1) & ~1)) atomicAdd(&status[0], 1);
+  row_chunks[g] = static_cast<uint16_t>((entries + kFields - 1) / kFields);
+}
+
+// One workgroup per matrix: order the rows by chunk count, longest first, and
 // describe the 64-row slices.  The order is a counting sort carried out by one
 // thread, so it is the same on every run.
 __global__ __launch_bounds__(256) void order_rows_kernel(
-    const int32_t *__restrict__ row_off_all, const uint32_t *__restrict__ minmax_all,
-    uint16_t *__restrict__ row_len, uint16_t *__restrict__ row_idx,
-    uint32_t *__restrict__ minmax_sorted, uint16_t *__restrict__ slice_nch,
-    uint16_t *__restrict__ slice_nfull, int32_t *__restrict__ counts,
-    int32_t *__restrict__ status, int height, int width, int slices, int kind) {
-  __shared__ int hist[kMaxLen + 2];
+    const uint16_t *__restrict__ row_chunks_all, const uint32_t *__restrict__ minmax_all,
+    uint16_t *__restrict__ row_idx, uint32_t *__restrict__ minmax_sorted,
+    uint16_t *__restrict__ slice_nch, int32_t *__restrict__ counts,
+    int32_t *__restrict__ status, int height, int slices, int kind) {
+  __shared__ int hist[kMaxRowChunks + 2];
+  __shared__ int first_len[1024];   // chunk count of the first row of up to 1024 slices
   const int e = blockIdx.x;
-  const int32_t *ro = row_off_all + static_cast<int64_t>(e) * (height + 1);
+  const uint16_t *rc = row_chunks_all + static_cast<int64_t>(e) * height;
   const uint32_t *mm = minmax_all + static_cast<int64_t>(e) * height;
   const int64_t lane0 = static_cast<int64_t>(e) * slices * 64;
-  const int max_len = (width + 1) / 2;
-  for (int i = threadIdx.x; i < kMaxLen + 2; i += blockDim.x) hist[i] = 0;
+  for (int i = threadIdx.x; i < kMaxRowChunks + 2; i += blockDim.x) hist[i] = 0;
   __syncthreads();
-  for (int r = threadIdx.x; r < height; r += blockDim.x) {
-    int len = ro[r + 1] - ro[r];
-    if (len < 1 || len > max_len) {
-      atomicAdd(&status[0], 1);
-      len = len < 1 ? 0 : max_len;
-    }
-    atomicAdd(&hist[len], 1);
-  }
+  for (int r = threadIdx.x; r < height; r += blockDim.x)
+    atomicAdd(&hist[min(static_cast<int>(rc[r]), kMaxRowChunks)], 1);
   __syncthreads();
   if (threadIdx.x == 0) {
     int run = 0;  // rows with a larger count come first
-    for (int len = max_len; len >= 0; len--) {
+    for (int len = kMaxRowChunks; len >= 0; len--) {
       int n = hist[len];
       hist[len] = run;
       run += n;
     }
     for (int r = 0; r < height; r++) {
-      int len = ro[r + 1] - ro[r];
-      len = len < 1 ? 0 : (len > max_len ? max_len : len);
+      const int len = min(static_cast<int>(rc[r]), kMaxRowChunks);
       int p = hist[len]++;
-      row_len[lane0 + p] = static_cast<uint16_t>(len);
       row_idx[lane0 + p] = static_cast<uint16_t>(r);
       minmax_sorted[lane0 + p] = mm[r];
+      if ((p & 63) == 0 && (p >> 6) < 1024) first_len[p >> 6] = len;
     }
   }
   for (int p = height + threadIdx.x; p < slices * 64; p += blockDim.x) {
-    row_len[lane0 + p] = 0;
     row_idx[lane0 + p] = 0xffffu;
     minmax_sorted[lane0 + p] = 0u;
   }
   __syncthreads();
   for (int s = threadIdx.x; s < slices; s += blockDim.x) {
-    int first = 64 * s;
-    int last = min(64 * s + 63, height - 1);
-    int nch = (row_len[lane0 + first] + kChunk - 1) / kChunk;
-    int nfull = row_len[lane0 + last] / kChunk;
+    // a slice is as long as its first row, and at least one chunk
+    int nch = s < 1024 ? first_len[s] : static_cast<int>(rc[row_idx[lane0 + 64 * s]]);
+    nch = max(nch, 1);
     int64_t g = static_cast<int64_t>(e) * slices + s;
     slice_nch[g] = static_cast<uint16_t>(nch);
-    slice_nfull[g] = static_cast<uint16_t>(nfull);
     counts[g + 1] = nch;
     atomicMax(&status[1 + kind], nch);
   }
@@ -211,68 +289,85 @@ __global__ __launch_bounds__(1024) void scan_counts_kernel(int32_t *__restrict__
   }
 }
 
-// One wavefront per ordered row: renumber its codes and write them, and the
-// zero padding up to the slice's chunk count, into the interleaved stream.
-__global__ __launch_bounds__(256) void interleave_codes_kernel(
-    const uint16_t *__restrict__ src, const int64_t *__restrict__ code_base,
-    const int32_t *__restrict__ row_off_all, const uint16_t *__restrict__ recode,
-    const uint32_t *__restrict__ slice_base, const uint16_t *__restrict__ slice_nch,
-    const uint16_t *__restrict__ row_idx, uint16_t *__restrict__ dst, int height,
-    int slices, int64_t lanes_total) {
-  const int64_t gl = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / 64;
-  if (gl >= lanes_total) return;
-  const int lane = threadIdx.x & 63;
-  const int64_t slice = gl / 64;
-  const int ln = static_cast<int>(gl % 64);
-  const int e = static_cast<int>(slice / slices);
-  const int ridx = row_idx[gl];
-  uint16_t *d = dst + static_cast<int64_t>(slice_base[slice]) * 256;
-  const int padded = slice_nch[slice] * kChunk;
-  int len = 0;
-  const uint16_t *s = src;
-  if (ridx != 0xffff) {
-    const int32_t *ro = row_off_all + static_cast<int64_t>(e) * (height + 1);
-    s = src + (code_base ? code_base[e] : 0) + ro[ridx];   // one matrix: no base array
-    len = min(max(ro[ridx + 1] - ro[ridx], 0), padded);
-  }
-  for (int j = lane; j < padded; j += 64) {
-    // padding decodes as one zero pair, the shortest entry (dictionary index 0)
-    uint16_t c = recode[j < len ? s[j] : 0];
-    d[(j / kChunk) * 256 + ln * kChunk + (j % kChunk)] = c;
-  }
-}
-
-// Column checkpoints.  For every slice and every group of kGroupChunks chunks,
-// the column offset (in dwords of the LDS activation array, 6 per column pair)
-// at which each lane's row stands when the group begins: 64 x u16 per group,
-// groups of slice g stored from entry slice_base[g]/kGroupChunks + g on.  With
-// them a wavefront can start in the middle of a slice, which is how a small
-// batch is spread over the GPU.  One wavefront per slice walks its codes.
+// Position checkpoints.  For every slice and every group of kGroupChunks chunks,
+// the position at which each lane's row stands when the group begins: 64 x u16
+// per group, groups of slice g stored from entry slice_base[g]/kGroupChunks + g
+// on.  With them a wavefront can start in the middle of a slice, which is how a
+// small batch is spread over the GPU.
 __device__ __forceinline__ int64_t checkpoint_entry(uint32_t slice_base, int64_t slice) {
   return static_cast<int64_t>(slice_base / kGroupChunks) + slice;
 }
 
-__global__ __launch_bounds__(256) void checkpoint_kernel(
-    const uint16_t *__restrict__ codes, const uint32_t *__restrict__ table,
+// One thread per lane of every slice: the row's entries into the interleaved
+// stream, nine to a chunk, zero entries up to the slice's chunk count, and the
+// row's position at the start of every group of chunks into the checkpoints.
+__global__ __launch_bounds__(256) void emit_entries_kernel(
+    const uint16_t *__restrict__ src, const int64_t *__restrict__ code_base,
+    const int32_t *__restrict__ row_off_all, const int32_t *__restrict__ dec,
     const uint32_t *__restrict__ slice_base, const uint16_t *__restrict__ slice_nch,
-    uint16_t *__restrict__ ckpt, int64_t first_slice, int64_t nslices, int group_shift) {
-  const int64_t sl = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / 64;
-  if (sl >= nslices) return;
-  const int lane = threadIdx.x & 63;
+    const uint16_t *__restrict__ row_idx, uint2 *__restrict__ dst, uint16_t *__restrict__ ckpt,
+    int height, int width, int slices, int64_t first_slice, int64_t lanes_total) {
+  const int64_t gl = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (gl >= lanes_total) return;
+  const int64_t slice = gl >> 6;
+  const int ln = static_cast<int>(gl & 63);
+  const int e = static_cast<int>(slice / slices);
+  const int ridx = row_idx[gl];
+  const uint32_t base = slice_base[slice];
+  const int nch = slice_nch[slice];
+  uint2 *d = dst + static_cast<int64_t>(base) * 64 + ln;
+  uint16_t *ck = ckpt + checkpoint_entry(base, first_slice + slice) * 64 + ln;
+  int c = 0, q = 0;
+  unsigned long long w = 0;
+  auto emit = [&](int step, int from) {
+    if (c >= nch) return;   // the slice is as long as its longest row: not reached
+    if (q == 0 && c % kGroupChunks == 0) ck[(c / kGroupChunks) * 64] = static_cast<uint16_t>(from);
+    w |= static_cast<unsigned long long>(step) << (kFieldBits * q);
+    if (++q == kFields) {
+      d[c * 64] = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
+      c++;
+      q = 0;
+      w = 0;
+    }
+  };
+  EntryWriter wr;
+  if (ridx != 0xffff) {
+    int n;
+    const uint16_t *codes = row_codes(src, code_base, row_off_all, e, ridx, height, width, n);
+    for_each_nonzero(codes, n, dec, width, [&](int col, int sym) { wr.nonzero(col, sym, emit); });
+    wr.park(emit);
+  }
+  while (c < nch) emit(0, wr.j);
+}
+
+// The symbols of one prepared matrix back out of the stream: out[row, column]
+// = 1 or 2 at every entry that stands on an activation; out is zero before.
+__global__ __launch_bounds__(256) void decode_entries_kernel(
+    const uint2 *__restrict__ stream, const uint32_t *__restrict__ slice_base,
+    const uint16_t *__restrict__ slice_nch, const uint16_t *__restrict__ row_idx,
+    uint8_t *__restrict__ out, int64_t first, int slices, int width) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= slices * 64) return;
+  const int64_t sl = first + (t >> 6);
+  const int ridx = row_idx[sl * 64 + (t & 63)];
+  if (ridx == 0xffff) return;
+  const uint2 *p = stream + static_cast<int64_t>(slice_base[sl]) * 64 + (t & 63);
   const int nch = slice_nch[sl];
-  const uint2 *p = reinterpret_cast<const uint2 *>(codes + static_cast<int64_t>(slice_base[sl]) * 256) + lane;
-  uint16_t *out = ckpt + checkpoint_entry(slice_base[sl], first_slice + sl) * 64 + lane;
-  uint32_t colw = 0;
+  int j = 0;
   for (int c = 0; c < nch; c++) {
-    if (c % kGroupChunks == 0) out[(c / kGroupChunks) * 64] = static_cast<uint16_t>(colw);
-    const uint2 w = p[c * 64];
-    const uint32_t cs[4] = {w.x & 0xffffu, w.x >> 16, w.y & 0xffffu, w.y >> 16};
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-      uint32_t idx = min(cs[q], (cs[q] >> 3) + static_cast<uint32_t>(group_shift));
-      colw += (table[idx] >> 16) & 0xffu;
+    const uint2 cw = p[c * 64];
+    const unsigned long long w = (static_cast<unsigned long long>(cw.y) << 32) | cw.x;
+    for (int q = 0; q < kFields; q++) {
+      j += static_cast<int>(w >> (kFieldBits * q)) & kMaxStep;
+      if (j % 3 != 0 && j / 3 < width)
+        out[static_cast<int64_t>(ridx) * width + j / 3] = static_cast<uint8_t>(j % 3);
     }
   }
+}
+
+__global__ void fill_bytes_kernel(uint8_t *p, int64_t n, uint8_t v) {
+  int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
 }
 
 __global__ void zero_words_kernel(int32_t *p, int n) {
@@ -285,21 +380,18 @@ __global__ void zero_words_kernel(int32_t *p, int n) {
 struct KindArgs {
   const uint32_t *slice_base;
   const uint16_t *slice_nch;
-  const uint16_t *slice_nfull;
-  const uint16_t *row_len;
   const uint16_t *row_idx;
   const uint32_t *minmax;
   int slices, height, width, parts;
   int split;            // wavefronts that share one slice (1 = a slice per wavefront)
-  int groups_max;       // most 32-code groups in a slice of this kind
+  int groups_max;       // most groups of chunks in a slice of this kind
   int64_t first_slice;  // global index of the kind's first slice (checkpoint addressing)
   int tail_split;       // fused kernel: wavefronts per slice of a short last pass (0: none)
 };
 
 struct PreparedArgs {
-  const uint32_t *table;      // kernel decode table (global copy, staged into LDS)
-  const uint16_t *codes;
-  const uint16_t *ckpt;       // column checkpoints, behind the code stream
+  const uint2 *stream;        // the interleaved entries
+  const uint16_t *ckpt;       // position checkpoints, behind the stream
   KindArgs k[2];
   const int32_t *token_expert;   // NULL: every token uses matrix 0
   const uint16_t *x;
@@ -309,31 +401,27 @@ struct PreparedArgs {
   int64_t ldx, ldy;              // element strides between tokens of x and y
   int kinds;                     // 2: y = wo(relu(wi x));  1: y += W x
   int tokens, experts;
-  int table_words, single_codes, group_shift;  // group_shift = single_codes - single_codes/8
-  int xdwords;                                 // LDS dwords reserved for the activations
-  int hdwords;                                 // fused kernel: LDS dwords of h (wo's activations)
+  int xdwords;                   // LDS dwords reserved for the activations
+  int hdwords;                   // fused kernel: LDS dwords of h (wo's activations)
   int spin_limit;
 };
 
-// Activations in LDS, 6 dwords per column pair:
-//   [A_even, B_even, A_odd, B_odd, 0, 0],  A = (x, 0), B = (0, x) as bf16 pairs.
-// Slot offset 6m + 2q + sym-1 selects the value for the row-min sum (A) or the
-// row-max sum (B); offsets 4 and 5 read zeros.  28 zero columns follow the row
-// (digits of a last codeword that overhang the width, as the reference pads).
-// At least 22 pairs: dword 130 (pair 21) is the zero that empty last slots read.
-__host__ __device__ constexpr int activation_pairs(int width) {
-  return (width + 28 + 1) / 2 + 1 > 22 ? (width + 28 + 1) / 2 + 1 : 22;
-}
+// Activations in LDS: dword 0 is zero, then 3 dwords per column,
+//   [A, B, 0],  A = (x, 0), B = (0, x) as bf16 pairs;
+// position 3c + 1 is column c's value for a row-min weight, 3c + 2 for a row-max
+// weight, every third dword a zero for long gaps and padding.  Rounded up to
+// whole 16 bytes (what follows in LDS stays aligned).
 __host__ __device__ constexpr int activation_dwords(int width) {
-  return 6 * activation_pairs(width);
+  return (3 * width + 1 + 3) / 4 * 4;
 }
 
 // Every load of a thread is in flight before its first LDS store, so a tile
 // pays one memory round trip for its activations, not one per pass.
 __device__ __forceinline__ void stage_activations(uint32_t *xa, const uint16_t *x, int width) {
-  const int npairs = activation_pairs(width);
+  const int npairs = (width + 1) / 2;
   const int step = blockDim.x;
   const bool aligned = (reinterpret_cast<uintptr_t>(x) & 3u) == 0;
+  if (threadIdx.x == 0) xa[0] = 0u;
   for (int m0 = threadIdx.x; m0 < npairs; m0 += 4 * step) {
     uint32_t v[4];
 #pragma unroll
@@ -351,104 +439,51 @@ __device__ __forceinline__ void stage_activations(uint32_t *xa, const uint16_t *
     for (int u = 0; u < 4; u++) {
       const int m = m0 + u * step;
       if (m < npairs) {
-        uint32_t *p = xa + 6 * m;
+        uint32_t *p = xa + 1 + 6 * m;
         p[0] = v[u] & 0xffffu;
         p[1] = v[u] << 16;
-        p[2] = v[u] >> 16;
-        p[3] = v[u] & 0xffff0000u;
-        p[4] = 0u;
-        p[5] = 0u;
+        p[2] = 0u;
+        if (2 * m + 1 < width) {
+          p[3] = v[u] >> 16;
+          p[4] = v[u] & 0xffff0000u;
+          p[5] = 0u;
+        }
       }
     }
   }
 }
 
-// The decode table into LDS with 16-byte loads, all of a thread's loads in
-// flight before its first store.  `words` is a multiple of 4 and the global
-// copy is padded to it.
-__device__ __forceinline__ void stage_table(uint32_t *tab, const uint32_t *src, int words) {
-  const uint4 *s4 = reinterpret_cast<const uint4 *>(src);
-  uint4 *d4 = reinterpret_cast<uint4 *>(tab);
-  const int n4 = words >> 2;
-  const int step = blockDim.x;
-  for (int i0 = threadIdx.x; i0 < n4; i0 += 4 * step) {
-    const int i1 = i0 + step, i2 = i1 + step, i3 = i2 + step;
-    const uint4 v0 = s4[i0];   // indices clamped: every load is valid and unconditional
-    const uint4 v1 = s4[min(i1, n4 - 1)];
-    const uint4 v2 = s4[min(i2, n4 - 1)];
-    const uint4 v3 = s4[min(i3, n4 - 1)];
-    d4[i0] = v0;
-    if (i1 < n4) d4[i1] = v1;
-    if (i2 < n4) d4[i2] = v2;
-    if (i3 < n4) d4[i3] = v3;
-  }
+typedef __attribute__((address_space(3))) const uint32_t lds_word;
+
+// The LDS byte address of a dword of the activation array.
+__device__ __forceinline__ uint32_t lds_address(const uint32_t *xa) {
+  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_word *)xa));
 }
 
-struct DotConsts {
-  bf16x2 lo, hi;   // (1, 0) and (0, 1)
-};
-
-__device__ __forceinline__ DotConsts dot_consts() {
-  // Kept in scalar registers through asm so that the compiler cannot turn
-  // (1.0, 0) into an inline constant of the packed-bf16 operand.
-  uint32_t k1, k2;
-  asm volatile("s_mov_b32 %0, 0x3f80" : "=s"(k1));
-  asm volatile("s_mov_b32 %0, 0x3f800000" : "=s"(k2));
-  DotConsts c;
-  c.lo = __builtin_bit_cast(bf16x2, k1);
-  c.hi = __builtin_bit_cast(bf16x2, k2);
-  return c;
-}
-
-typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-
-// Table words of the two kernel codes packed in `pair`, with each code's symbol
-// bits put in place.  idx = min(c, (c >> 3) + group_shift) per 16-bit half.
-__device__ __forceinline__ void lookup2(const uint32_t *tab, uint32_t pair, uint32_t shift2,
-                                        uint32_t &e_lo, uint32_t &e_hi) {
-  u16x2 c = __builtin_bit_cast(u16x2, pair);
-  u16x2 g = (c >> static_cast<unsigned short>(3)) + __builtin_bit_cast(u16x2, shift2);
-  u16x2 idx = __builtin_elementwise_min(c, g);
-  uint32_t w_lo = tab[idx.x];
-  uint32_t w_hi = tab[idx.y];
-  uint32_t sym = pair & 0x00070007u;
-  uint32_t b_lo = (sym & 0xffffu) * 0x400081u;   // bits 0, 1, 2 of the code -> bits 0, 8, 24
-  uint32_t b_hi = (sym >> 16) * 0x400081u;
-  e_lo = (w_lo & ~0x01000101u) | (b_lo & 0x01000101u);
-  e_hi = (w_hi & ~0x01000101u) | (b_hi & 0x01000101u);
-  // one v_bfi each; the empty asm keeps the compiler from redoing the merge
-  // for every byte it later extracts
-  asm("" : "+v"(e_lo));
-  asm("" : "+v"(e_hi));
-}
-
-__device__ __forceinline__ void lookup4(const uint32_t *tab, uint2 w, uint32_t shift2,
-                                        uint32_t (&e)[4]) {
-  lookup2(tab, w.x, shift2, e[0], e[1]);
-  lookup2(tab, w.y, shift2, e[2], e[3]);
-}
-
-__device__ __forceinline__ void add_codeword(uint32_t e, const uint32_t *xa, int &colw,
-                                             float &s1, float &s2, const DotConsts &k) {
-  // slot 2 of a word whose sign bit is set is empty: the column is dropped from
-  // its address, and what is left (130 or 131) is a zero dword all lanes share
-  const int col2 = colw & ~(static_cast<int>(e) >> 31);
-  const int idx[3] = {colw + static_cast<int>(e & 0xffu),
-                      colw + static_cast<int>((e >> 8) & 0xffu),
-                      col2 + static_cast<int>(e >> 24)};
+// The nine entries of a chunk: each moves the row's LDS address `at` (bytes)
+// and adds the bf16 pair found there, times the row's (min, max), onto acc.
+// v_bfe_u32 and v_lshl_add_u32 are written out because the compiler expands the
+// same arithmetic into three instructions per entry instead of two.
+__device__ __forceinline__ void add_chunk(uint2 cw, uint32_t &at, float &acc, bf16x2 minmax) {
+  const uint32_t mid = __builtin_amdgcn_alignbit(cw.y, cw.x, 28);   // bits 28..59: entries 4..7
+  uint32_t f[kFields];
 #pragma unroll
-  for (int j = 0; j < 3; j++) {
-    bf16x2 v = __builtin_bit_cast(bf16x2, xa[idx[j]]);
-    s1 = __builtin_amdgcn_fdot2_f32_bf16(v, k.lo, s1, false);
-    s2 = __builtin_amdgcn_fdot2_f32_bf16(v, k.hi, s2, false);
+  for (int q = 0; q < 4; q++) {
+    asm("v_bfe_u32 %0, %1, %2, 7" : "=v"(f[q]) : "v"(cw.x), "n"(kFieldBits * q));
+    asm("v_bfe_u32 %0, %1, %2, 7" : "=v"(f[4 + q]) : "v"(mid), "n"(kFieldBits * q));
   }
-  colw += static_cast<int>((e >> 16) & 0xffu);
+  asm("v_bfe_u32 %0, %1, 24, 7" : "=v"(f[8]) : "v"(cw.y));           // bits 56..62
+#pragma unroll
+  for (int q = 0; q < kFields; q++) {
+    asm("v_lshl_add_u32 %0, %1, 2, %0" : "+v"(at) : "v"(f[q]));
+    const bf16x2 v = __builtin_bit_cast(bf16x2, *(lds_word *)static_cast<uintptr_t>(at));
+    acc = __builtin_amdgcn_fdot2_f32_bf16(v, minmax, acc, false);
+  }
 }
 
 // This lane's chunk 0 of the slice that starts at chunk `base` of the stream.
-__device__ __forceinline__ const uint2 *chunk_pointer(const uint16_t *codes, uint32_t base) {
-  return reinterpret_cast<const uint2 *>(codes + static_cast<int64_t>(base) * 256) +
-         (threadIdx.x & 63);
+__device__ __forceinline__ const uint2 *chunk_pointer(const uint2 *stream, uint32_t base) {
+  return stream + static_cast<int64_t>(base) * 64 + (threadIdx.x & 63);
 }
 
 // What a lane needs to walk its row of one slice; load_slice issues the loads
@@ -457,44 +492,41 @@ __device__ __forceinline__ const uint2 *chunk_pointer(const uint16_t *codes, uin
 template <int R>
 struct Walk {
   uint32_t base;     // the slice's first chunk, in chunks; the same in every lane,
-  int nch, nfull;    // like the chunk counts (nch: where this wavefront stops)
+  int nch;           // like the chunk count (where this wavefront stops)
   int c0;            // and the chunk this wavefront starts at (0 unless it shares the slice)
-  int colw0;         // this lane's column offset at chunk c0
-  int len, ridx;
+  int j0;            // this lane's position at chunk c0
+  int ridx;
   uint32_t minmax;
   uint2 ring[R];
 };
 typedef Walk<kRing> SliceWalk;
 
-// g_lo, g_hi: the run of 32-code groups to walk, for a wavefront that shares the
-// slice with others (it then starts from the column checkpoint of group g_lo).
+// g_lo, g_hi: the run of chunk groups to walk, for a wavefront that shares the
+// slice with others (it then starts from the position checkpoint of group g_lo).
 __device__ __forceinline__ SliceWalk load_slice(const PreparedArgs &a, const KindArgs &k,
                                                 int64_t sl, int g_lo = 0, int g_hi = 1 << 20) {
   const int lane = threadIdx.x & 63;
   SliceWalk w;
   const int nch_all = __builtin_amdgcn_readfirstlane(k.slice_nch[sl]);
   w.nch = min(g_hi * kGroupChunks, nch_all);
-  w.nfull = min(__builtin_amdgcn_readfirstlane(k.slice_nfull[sl]), w.nch);
   w.c0 = g_lo * kGroupChunks;
-  w.len = k.row_len[sl * 64 + lane];
   w.ridx = k.row_idx[sl * 64 + lane];
   w.minmax = k.minmax[sl * 64 + lane];
   w.base = __builtin_amdgcn_readfirstlane(k.slice_base[sl]);
-  w.colw0 = 0;
+  w.j0 = 0;
   if (g_lo)
-    w.colw0 = a.ckpt[(checkpoint_entry(w.base, k.first_slice + sl) + g_lo) * 64 + lane];
-  const uint2 *p = chunk_pointer(a.codes, w.base);
+    w.j0 = a.ckpt[(checkpoint_entry(w.base, k.first_slice + sl) + g_lo) * 64 + lane];
+  const uint2 *p = chunk_pointer(a.stream, w.base);
 #pragma unroll
   for (int i = 0; i < kRing; i++) w.ring[i] = p[min(w.c0 + i, w.nch - 1) * 64];
   return w;
 }
 
 // R chunks (the depth of the walk's ring) starting at chunk c added onto the
-// partial sums p1, p2.  kChecked: compare every code with the lane's own count.
+// partial sum.  kChecked: the wavefront's last chunks, fewer than R.
 template <bool kChecked, int R>
-__device__ __forceinline__ void run_chunks(Walk<R> &w, const uint2 *p, int c, uint32_t shift2,
-                                           const uint32_t *tab, const uint32_t *xa, int &colw,
-                                           float &p1, float &p2, const DotConsts &dk) {
+__device__ __forceinline__ void run_chunks(Walk<R> &w, const uint2 *p, int c, uint32_t &at,
+                                           float &part, bf16x2 minmax) {
   const int nch = w.nch;
 #pragma unroll
   for (int i = 0; i < R; i++) {
@@ -503,16 +535,8 @@ __device__ __forceinline__ void run_chunks(Walk<R> &w, const uint2 *p, int c, ui
       // unconditional, clamped to the last chunk: the load can target the ring
       // register itself and the loop needs no wait for it
       w.ring[i] = p[min(c + i + R, nch - 1) * 64];
-      uint32_t e[4];
-      lookup4(tab, cw, shift2, e);
-      const int j = kChunk * (c + i);
-#pragma unroll
-      for (int q = 0; q < 4; q++)
-        add_codeword(!kChecked || j + q < w.len ? e[q] : kIdleWord, xa, colw, p1, p2, dk);
+      add_chunk(cw, at, part, minmax);
     }
-    // a deep ring is for latency: keep the scheduler from also hoisting every
-    // chunk's table words, which would not fit the registers
-    if (R > kRing) __builtin_amdgcn_sched_barrier(0);
   }
 }
 
@@ -535,68 +559,58 @@ __device__ __forceinline__ void progress_priority(int done, int total) {
   }
 }
 
-// The two sums of this lane's row, in the library's canonical order: groups of
-// 32 codes (kGroupChunks chunks), a partial sum per group from zero, the
-// partial sums added first group first.
+// The sum of this lane's row, in the library's canonical order: groups of 72
+// entries (kGroupChunks chunks), a partial sum per group from zero, the partial
+// sums added first group first.
 // With `part` the wavefront shares its slice: it leaves each group's partial
-// sums at part[group * 64 + lane] for the wavefront that adds them up.
+// sum at part[group * 64 + lane] for the wavefront that adds them up.
 // pass / passes (passes != 0): this slice is the wavefront's pass-th of `passes`
 // about equal ones in the current phase; sets the priority by progress.
-__device__ __forceinline__ void run_slice(SliceWalk &w, const uint16_t *codes, int group_shift,
-                                          const uint32_t *tab, const uint32_t *xa, float &s1,
-                                          float &s2, float2 *part = nullptr, int pass = 0,
-                                          int passes = 0) {
-  const DotConsts dk = dot_consts();
-  const uint32_t shift2 = static_cast<uint32_t>(group_shift) * 0x00010001u;
+__device__ __forceinline__ float run_slice(SliceWalk &w, const uint2 *stream, const uint32_t *xa,
+                                           float *part = nullptr, int pass = 0, int passes = 0) {
   // a walk that went through `cur = nxt` may sit in vector registers: put what
   // is the same in all lanes back into scalar ones, for scalar loop control
   // and scalar address arithmetic
   w.nch = __builtin_amdgcn_readfirstlane(w.nch);
-  w.nfull = __builtin_amdgcn_readfirstlane(w.nfull);
-  const uint2 *p = chunk_pointer(codes, __builtin_amdgcn_readfirstlane(w.base));
+  const uint2 *p = chunk_pointer(stream, __builtin_amdgcn_readfirstlane(w.base));
   const int lane = threadIdx.x & 63;
-  s1 = 0.f;
-  s2 = 0.f;
-  float p1 = 0.f, p2 = 0.f;
-  int colw = w.colw0;
+  const bf16x2 minmax = __builtin_bit_cast(bf16x2, w.minmax);
+  float sum = 0.f, partial = 0.f;
+  uint32_t at = lds_address(xa) + 4u * static_cast<uint32_t>(w.j0);
   int c = __builtin_amdgcn_readfirstlane(w.c0);
   if (passes) progress_priority(pass, passes);
   auto group_done = [&]() {
     if (passes) progress_priority(pass * w.nch + c + kRing, passes * w.nch);
     if (part) {
-      part[((c + kRing) / kGroupChunks - 1) * 64 + lane] = make_float2(p1, p2);
+      part[((c + kRing) / kGroupChunks - 1) * 64 + lane] = partial;
     } else {
-      s1 += p1;
-      s2 += p2;
+      sum += partial;
     }
-    p1 = 0.f;
-    p2 = 0.f;
+    partial = 0.f;
   };
-  // chunks every lane of the slice has in full: no per-code checks
-  for (; c + kRing <= w.nfull; c += kRing) {
-    run_chunks<false>(w, p, c, shift2, tab, xa, colw, p1, p2, dk);
+  for (; c + kRing <= w.nch; c += kRing) {
+    run_chunks<false>(w, p, c, at, partial, minmax);
     if ((c + kRing) % kGroupChunks == 0) group_done();
   }
-  for (; c < w.nch; c += kRing) {
-    run_chunks<true>(w, p, c, shift2, tab, xa, colw, p1, p2, dk);
+  if (c < w.nch) {
+    run_chunks<true>(w, p, c, at, partial, minmax);
     if ((c + kRing) % kGroupChunks == 0) group_done();
+    c += kRing;
   }
   if (part) {
     // the slice's last group, unless the loop has just closed it
-    if (c % kGroupChunks) part[(c / kGroupChunks) * 64 + lane] = make_float2(p1, p2);
+    if (c % kGroupChunks) part[(c / kGroupChunks) * 64 + lane] = partial;
   } else {
-    s1 += p1;   // the last, partial group (+0 if it was just folded)
-    s2 += p2;
+    sum += partial;   // the last, partial group (+0 if it was just folded)
   }
+  return sum;
 }
 
 // How a row's result leaves the kernel.
 enum OutMode { kStoreRelu = 0, kStore = 1, kAccumulate = 2 };
 
-__device__ __forceinline__ void write_row(uint16_t *dst, int ridx, uint32_t minmax, float s1,
-                                          float s2, int mode) {
+__device__ __forceinline__ void write_row(uint16_t *dst, int ridx, float res, int mode) {
   if (ridx == 0xffff) return;   // padding lane
-  float res = row_result(minmax, s1, s2);
   uint16_t out = f32_to_bf16(res);
   if (mode == kStoreRelu) {
     if (out & 0x8000u) out = 0;   // relu between the projections, on the bf16 value
@@ -608,21 +622,21 @@ __device__ __forceinline__ void write_row(uint16_t *dst, int ridx, uint32_t minm
 }
 
 // Small-batch form of a tile: `split` wavefronts share each slice, every one
-// taking a run of the slice's 32-code groups (it starts from the column
-// checkpoint of its first group) and leaving one partial-sum pair per group in
-// LDS; after a barrier the slice's first wavefront adds the groups in order,
-// which is the canonical order, so the result is the same to the bit as with a
+// taking a run of the slice's chunk groups (it starts from the position
+// checkpoint of its first group) and leaving one partial sum per group in LDS;
+// after a barrier the slice's first wavefront adds the groups in order, which
+// is the canonical order, so the result is the same to the bit as with a
 // wavefront per slice.  Built for latency: split_begin puts the loads of a
 // whole group in flight, and the kernel calls it before it waits for and
 // stages the activations.
 struct SplitWalk {
   Walk<kSplitRing> w;   // w.nch: this wavefront's last chunk + 1
-  int g_lo, g_hi, ngroups, colw;
+  int g_lo, g_hi, ngroups;
   int64_t sl;
   bool mine;
 };
 
-// Everything but len, colw and the ring is the same in all lanes and is kept
+// Everything but the position and the ring is the same in all lanes and is kept
 // in scalar registers (the wavefront index goes through readfirstlane).  The
 // ring loads are unconditional, with the chunk index clamped to the wavefront's
 // last chunk, so that they all leave at once.
@@ -637,28 +651,27 @@ __device__ __forceinline__ SplitWalk split_begin(const PreparedArgs &a, const Ki
   r.ngroups = 0;
   r.g_lo = 0;
   r.g_hi = 0;
-  r.colw = 0;
   r.sl = static_cast<int64_t>(e) * k.slices + s;
   r.w.base = 0;
+  r.w.j0 = 0;
+  r.w.nch = 0;
+  r.w.minmax = 0u;
+  r.w.ridx = 0xffff;
   if (r.mine) {
     const int nch_all = __builtin_amdgcn_readfirstlane(k.slice_nch[r.sl]);
     r.ngroups = (nch_all + kGroupChunks - 1) / kGroupChunks;
     r.g_lo = sub * r.ngroups / k.split;
     r.g_hi = (sub + 1) * r.ngroups / k.split;
-    if (sub == 0) {   // the wavefront that will write the slice's rows
-      r.w.ridx = k.row_idx[r.sl * 64 + lane];
-      r.w.minmax = k.minmax[r.sl * 64 + lane];
-    }
+    r.w.minmax = k.minmax[r.sl * 64 + lane];
+    if (sub == 0) r.w.ridx = k.row_idx[r.sl * 64 + lane];   // it will write the slice's rows
     if (r.g_lo < r.g_hi) {
       const uint32_t base = __builtin_amdgcn_readfirstlane(k.slice_base[r.sl]);
-      r.w.nfull = __builtin_amdgcn_readfirstlane(k.slice_nfull[r.sl]);
-      r.w.len = k.row_len[r.sl * 64 + lane];
       r.w.base = base;
-      const uint2 *p = chunk_pointer(a.codes, base);
+      const uint2 *p = chunk_pointer(a.stream, base);
       const int c_lo = r.g_lo * kGroupChunks;
       r.w.nch = min(r.g_hi * kGroupChunks, nch_all);
       if (r.g_lo)
-        r.colw = a.ckpt[(checkpoint_entry(base, k.first_slice + r.sl) + r.g_lo) * 64 + lane];
+        r.w.j0 = a.ckpt[(checkpoint_entry(base, k.first_slice + r.sl) + r.g_lo) * 64 + lane];
 #pragma unroll
       for (int i = 0; i < kSplitRing; i++)
         r.w.ring[i] = p[min(c_lo + i, r.w.nch - 1) * 64];
@@ -671,43 +684,36 @@ __device__ __forceinline__ SplitWalk split_begin(const PreparedArgs &a, const Ki
 // has its slice to itself (split 1) adds the groups in registers, in the same
 // order, and leaves the partial-sum area alone.
 __device__ __forceinline__ void split_run(const PreparedArgs &a, const KindArgs &k, SplitWalk &r,
-                                          const uint32_t *tab, const uint32_t *xa, uint16_t *dst,
-                                          int mode) {
-  float2 *part = reinterpret_cast<float2 *>(const_cast<uint32_t *>(xa) + a.xdwords);
+                                          const uint32_t *xa, uint16_t *dst, int mode) {
+  float *part = reinterpret_cast<float *>(const_cast<uint32_t *>(xa) + a.xdwords);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int local = wave / k.split;
   const bool alone = k.split == 1;
-  const DotConsts dk = dot_consts();
-  const uint32_t shift2 = static_cast<uint32_t>(a.group_shift) * 0x00010001u;
-  int colw = r.colw;
-  float s1 = 0.f, s2 = 0.f;
-  const uint2 *p = chunk_pointer(a.codes, r.w.base);
+  const bf16x2 minmax = __builtin_bit_cast(bf16x2, r.w.minmax);
+  uint32_t at = lds_address(xa) + 4u * static_cast<uint32_t>(r.w.j0);
+  float sum = 0.f;
+  const uint2 *p = chunk_pointer(a.stream, r.w.base);
   for (int g = r.g_lo; g < r.g_hi; g++) {
-    float p1 = 0.f, p2 = 0.f;
+    float partial = 0.f;
     const int c_end = min((g + 1) * kGroupChunks, r.w.nch);
     for (int c = g * kGroupChunks; c < c_end; c += kSplitRing) {
-      if (c + kSplitRing <= r.w.nfull)
-        run_chunks<false>(r.w, p, c, shift2, tab, xa, colw, p1, p2, dk);
+      if (c + kSplitRing <= c_end)
+        run_chunks<false>(r.w, p, c, at, partial, minmax);
       else
-        run_chunks<true>(r.w, p, c, shift2, tab, xa, colw, p1, p2, dk);
+        run_chunks<true>(r.w, p, c, at, partial, minmax);
     }
     if (alone) {
-      s1 += p1;
-      s2 += p2;
+      sum += partial;
     } else {
-      part[(local * k.groups_max + g) * 64 + lane] = make_float2(p1, p2);
+      part[(local * k.groups_max + g) * 64 + lane] = partial;
     }
   }
   __syncthreads();
   if (r.mine && wave % k.split == 0) {
     if (!alone)
-      for (int g = 0; g < r.ngroups; g++) {
-        float2 v = part[(local * k.groups_max + g) * 64 + lane];
-        s1 += v.x;
-        s2 += v.y;
-      }
-    write_row(dst, r.w.ridx, r.w.minmax, s1, s2, mode);
+      for (int g = 0; g < r.ngroups; g++) sum += part[(local * k.groups_max + g) * 64 + lane];
+    write_row(dst, r.w.ridx, sum, mode);
   }
 }
 
@@ -803,11 +809,9 @@ __device__ __forceinline__ void publish_h(const PreparedArgs &a, int t) {
 __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs a) {
   extern __shared__ __align__(16) uint32_t lds[];
   __shared__ int s_ticket;
-  uint32_t *tab = lds;
-  uint32_t *xa = lds + a.table_words;
+  uint32_t *xa = lds;
   const int threads = blockDim.x;
   const int waves = threads >> 6;
-  stage_table(tab, a.table, a.table_words);
   const int n_wi = a.tokens * a.k[0].parts;
   const int n_all = n_wi + (a.kinds == 2 ? a.tokens * a.k[1].parts : 0);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -847,7 +851,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
     if (e >= 0) {
       int mode;
       uint16_t *dst = tile_output(a, k, kind, t, mode);
-      // the first loads of the codes go out before the wait and the staging
+      // the first loads of the stream go out before the wait and the staging
       {
         int s = s_lo + wave;
         SliceWalk cur;
@@ -857,10 +861,9 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
           const bool more = s + waves < s_hi;
           SliceWalk nxt;
           if (more) nxt = load_slice(a, k, static_cast<int64_t>(e) * k.slices + s + waves);
-          float s1, s2;
-          run_slice(cur, a.codes, a.group_shift, tab, xa, s1, s2, nullptr, (s - s_lo) / waves,
-                    (s_hi - s_lo + waves - 1) / waves);
-          write_row(dst, cur.ridx, cur.minmax, s1, s2, mode);
+          const float res = run_slice(cur, a.stream, xa, nullptr, (s - s_lo) / waves,
+                                      (s_hi - s_lo + waves - 1) / waves);
+          write_row(dst, cur.ridx, res, mode);
           if (more) cur = nxt;
         }
       }
@@ -874,21 +877,19 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
 // a token, and the workgroup runs wi, ReLU and wo back to back with h kept in
 // LDS, already in the layout wo reads its activations from.  No workspace
 // traffic for h, no waiting between workgroups; tickets only balance the load.
-// LDS: table | x (wi's activations) | h (wo's activations).
+// LDS: x (wi's activations) | h (wo's activations).
 __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(PreparedArgs a) {
   extern __shared__ __align__(16) uint32_t lds[];
   __shared__ int s_ticket;
-  uint32_t *tab = lds;
-  uint32_t *xa = lds + a.table_words;
+  uint32_t *xa = lds;
   uint32_t *ha = xa + a.xdwords;
   const int threads = blockDim.x;
   const int waves = threads >> 6;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const KindArgs &ki = a.k[0];
   const KindArgs &ko = a.k[1];
-  stage_table(tab, a.table, a.table_words);
-  // h: the lanes overwrite the two value dwords of their rows; the empty slots
-  // and the columns past d_ff stay zero for the whole launch
+  // h: the lanes overwrite the two value dwords of their rows; the zeros between
+  // them stay for the whole launch
   for (int i = threadIdx.x; i < a.hdwords; i += threads) ha[i] = 0u;
   int next_ticket = 0;
   auto fetch_next = [&]() {
@@ -924,13 +925,12 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
       const bool more = s + waves < ki.slices;
       SliceWalk nxt;
       if (more) nxt = load_slice(a, ki, static_cast<int64_t>(e) * ki.slices + s + waves);
-      float s1, s2;
-      run_slice(cur, a.codes, a.group_shift, tab, xa, s1, s2, nullptr, s / waves,
-                (ki.slices + waves - 1) / waves);
+      const float res = run_slice(cur, a.stream, xa, nullptr, s / waves,
+                                  (ki.slices + waves - 1) / waves);
       if (cur.ridx != 0xffff) {
-        uint32_t out = f32_to_bf16(row_result(cur.minmax, s1, s2));
+        uint32_t out = f32_to_bf16(res);
         if (out & 0x8000u) out = 0;   // relu between the projections, on the bf16 value
-        uint32_t *p = ha + 6 * (cur.ridx >> 1) + 2 * (cur.ridx & 1);
+        uint32_t *p = ha + 1 + 3 * cur.ridx;
         p[0] = out;
         p[1] = out << 16;
       }
@@ -942,7 +942,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
     fetch_next();
     // wo: h -> y; its first loads go out before the barrier.  A short last pass
     // (tail_split != 0) is shared out: tail_split wavefronts per slice, each a
-    // run of its 32-code groups, partial sums into the LDS that held x.
+    // run of its chunk groups, partial sums into the LDS that held x.
     const int whole = ko.tail_split ? ko.slices - ko.slices % waves : ko.slices;
     const int64_t first = static_cast<int64_t>(e) * ko.slices;
     s = wave;
@@ -953,10 +953,9 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
       const bool more = s + waves < whole;
       SliceWalk nxt;
       if (more) nxt = load_slice(a, ko, first + s + waves);
-      float s1, s2;
-      run_slice(cur, a.codes, a.group_shift, tab, ha, s1, s2, nullptr, s / waves,
-                (whole + waves - 1) / waves);
-      write_row(dst, cur.ridx, cur.minmax, s1, s2, kStore);
+      const float res = run_slice(cur, a.stream, ha, nullptr, s / waves,
+                                  (whole + waves - 1) / waves);
+      write_row(dst, cur.ridx, res, kStore);
       if (more) cur = nxt;
     }
     __builtin_amdgcn_s_setprio(0);
@@ -964,7 +963,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
       const int lane = threadIdx.x & 63;
       const int sl = whole + wave / ko.tail_split;
       const int sub = wave % ko.tail_split;
-      float2 *mine = reinterpret_cast<float2 *>(xa) + (wave / ko.tail_split) * ko.groups_max * 64;
+      float *mine = reinterpret_cast<float *>(xa) + (wave / ko.tail_split) * ko.groups_max * 64;
       int groups = 0;
       if (sl < ko.slices) {
         groups = (__builtin_amdgcn_readfirstlane(ko.slice_nch[first + sl]) + kGroupChunks - 1) /
@@ -972,21 +971,15 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
         const int g_lo = sub * groups / ko.tail_split, g_hi = (sub + 1) * groups / ko.tail_split;
         if (g_lo < g_hi) {
           SliceWalk tail = load_slice(a, ko, first + sl, g_lo, g_hi);
-          float s1, s2;
-          run_slice(tail, a.codes, a.group_shift, tab, ha, s1, s2, mine);
+          run_slice(tail, a.stream, ha, mine);
         }
       }
       __syncthreads();
       if (sub == 0 && sl < ko.slices) {
         // the slice's first wavefront adds the groups in order and writes the rows
-        float s1 = 0.f, s2 = 0.f;
-        for (int g = 0; g < groups; g++) {
-          const float2 v = mine[g * 64 + lane];
-          s1 += v.x;
-          s2 += v.y;
-        }
-        write_row(dst, ko.row_idx[(first + sl) * 64 + lane], ko.minmax[(first + sl) * 64 + lane],
-                  s1, s2, kStore);
+        float sum = 0.f;
+        for (int g = 0; g < groups; g++) sum += mine[g * 64 + lane];
+        write_row(dst, ko.row_idx[(first + sl) * 64 + lane], sum, kStore);
       }
     }
   }
@@ -996,14 +989,12 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
 // for latency.  `split` wavefronts share a slice (split_begin / split_run) and
 // all of a wavefront's loads leave before anything waits.  With no more tiles
 // than compute units every workgroup runs one tile; beyond that the grid is
-// persistent and keeps its table.  Tiles are taken by ticket like in the
-// streaming kernel, so a wo tile's wait for its token's wi tiles ends for the
-// same reason.
+// persistent.  Tiles are taken by ticket like in the streaming kernel, so a wo
+// tile's wait for its token's wi tiles ends for the same reason.
 __global__ __launch_bounds__(kMaxThreads) void moe_prepared_small_kernel(PreparedArgs a) {
   extern __shared__ __align__(16) uint32_t lds[];
   __shared__ int s_ticket;
-  uint32_t *tab = lds;
-  uint32_t *xa = lds + a.table_words;
+  uint32_t *xa = lds;
   const bool dynamic = a.ctrl != nullptr;
   const int n_all = a.tokens * (a.k[0].parts + (a.kinds == 2 ? a.k[1].parts : 0));
   int static_ticket = blockIdx.x;
@@ -1011,7 +1002,6 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_small_kernel(Prepare
   if (dynamic && threadIdx.x == 0)
     next_ticket = __hip_atomic_fetch_add(&a.ctrl[0], 1, __ATOMIC_RELAXED,
                                          __HIP_MEMORY_SCOPE_AGENT);
-  stage_table(tab, a.table, a.table_words);
   for (;;) {
     int ticket;
     if (dynamic) {
@@ -1048,54 +1038,20 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_small_kernel(Prepare
       // the launch cuts the matrices so that a tile has at most waves / split slices
       SplitWalk walk = split_begin(a, k, e, tile.s_lo, tile.s_hi);
       await_activations(a, k, kind, t, xa);
-      split_run(a, k, walk, tab, xa, dst, mode);
+      split_run(a, k, walk, xa, dst, mode);
     }
     fetch_next();
     if (a.kinds == 2 && kind == 0) publish_h(a, t);
   }
 }
 
-// ------------------------------------------------------ per-device tables --
-
-struct DeviceTables {
-  int device;
-  uint16_t *recode;
-  uint32_t *table;
-  int single_codes, words;
-};
+// ------------------------------------------------------------ host side --
 
 std::mutex g_mutex;
-std::vector<DeviceTables> g_tables;
 std::vector<std::pair<int, const int32_t *>> g_checked_dec;   // (device, dec) known to be the fixed table
 
-int device_tables(hipStream_t stream, const DeviceTables **out) {
-  int device = 0;
-  HIP_TRY(hipGetDevice(&device));
-  std::lock_guard<std::mutex> lock(g_mutex);
-  for (const DeviceTables &t : g_tables)
-    if (t.device == device) {
-      *out = &t;
-      return SUB1_OK;
-    }
-  std::vector<uint16_t> recode(SUB1_DICT_ENTRIES);
-  std::vector<uint32_t> table(SUB1_KERNEL_TABLE_MAX, 0u);
-  DeviceTables t;
-  t.device = device;
-  int rc = sub1_build_kernel_tables(recode.data(), table.data(), &t.single_codes, &t.words);
-  if (rc) return fail(rc, "sub1_build_kernel_tables failed");
-  HIP_TRY(hipMalloc(&t.recode, recode.size() * sizeof(uint16_t)));
-  HIP_TRY(hipMalloc(&t.table, table.size() * sizeof(uint32_t)));
-  HIP_TRY(hipMemcpyAsync(t.recode, recode.data(), recode.size() * sizeof(uint16_t),
-                         hipMemcpyHostToDevice, stream));
-  HIP_TRY(hipMemcpyAsync(t.table, table.data(), table.size() * sizeof(uint32_t),
-                         hipMemcpyHostToDevice, stream));
-  HIP_TRY(hipStreamSynchronize(stream));  // the host vectors go away
-  g_tables.push_back(t);
-  *out = &g_tables.back();
-  return SUB1_OK;
-}
-
-// The renumbering belongs to the fixed dictionary: refuse any other dec.
+// The prepare kernels read dec as the fixed dictionary's table (symbols 0..2,
+// unused digits zero): refuse any other.
 int check_dec(const int32_t *dec, hipStream_t stream) {
   int device = 0;
   HIP_TRY(hipGetDevice(&device));
@@ -1220,13 +1176,16 @@ int prepare_layout(const Source &src, void *meta, int64_t meta_bytes, LayoutResu
   int64_t slice0 = 0;
   for (int i = 0; i < src.kinds; i++) {
     const KindMeta &k = m.k[i];
+    uint16_t *row_chunks = reinterpret_cast<uint16_t *>(base + k.row_chunks);
+    const int64_t rows = static_cast<int64_t>(src.count) * k.height;
+    count_entries_kernel<<<static_cast<unsigned>((rows + 255) / 256), 256, 0, s>>>(
+        src.w_comp, src.code_base[i], src.row_off[i], src.dec, row_chunks, status, k.height,
+        k.width, rows);
     order_rows_kernel<<<src.count, 256, 0, s>>>(
-        src.row_off[i], src.minmax[i], reinterpret_cast<uint16_t *>(base + k.row_len),
-        reinterpret_cast<uint16_t *>(base + k.row_idx),
+        row_chunks, src.minmax[i], reinterpret_cast<uint16_t *>(base + k.row_idx),
         reinterpret_cast<uint32_t *>(base + k.minmax),
-        reinterpret_cast<uint16_t *>(base + k.slice_nch),
-        reinterpret_cast<uint16_t *>(base + k.slice_nfull), counts + slice0, status, k.height,
-        k.width, k.slices, i);
+        reinterpret_cast<uint16_t *>(base + k.slice_nch), counts + slice0, status, k.height,
+        k.slices, i);
     slice0 += static_cast<int64_t>(src.count) * k.slices;
   }
   scan_counts_kernel<<<1, 1024, 0, s>>>(counts, static_cast<int>(slice0));
@@ -1237,11 +1196,11 @@ int prepare_layout(const Source &src, void *meta, int64_t meta_bytes, LayoutResu
   HIP_TRY(hipMemcpyAsync(&total, counts + slice0, 4, hipMemcpyDeviceToHost, s));
   HIP_TRY(hipStreamSynchronize(s));
   if (host[0])
-    return fail(SUB1_ERR_SHAPE, "%s: %d rows have a code count outside 1..width/2", who, host[0]);
+    return fail(SUB1_ERR_SHAPE, "%s: the codes of %d rows do not cover the width", who, host[0]);
   if (total < 0) return fail(SUB1_ERR_SHAPE, "%s: stream too large", who);
   out->meta_bytes = m.bytes;
   out->total_chunks = total;
-  // the code stream, then one 128-byte checkpoint entry per group of chunks
+  // the entry stream, then one 128-byte checkpoint entry per group of chunks
   out->code_bytes = static_cast<int64_t>(total) * 512 +
                     (static_cast<int64_t>(total) / kGroupChunks + slice0 + 1) * 128;
   out->max_chunks[0] = host[1];
@@ -1253,8 +1212,7 @@ int prepare_codes(const Source &src, const Prepared &p, hipStream_t s, const cha
   if (!p.meta || !p.codes) return fail(SUB1_ERR_NULL, "%s: NULL argument", who);
   if (misaligned(p.meta, 256) || misaligned(p.codes, 256))
     return fail(SUB1_ERR_ALIGN, "%s: buffers must be 256-byte aligned", who);
-  const DeviceTables *t = nullptr;
-  int rc = device_tables(s, &t);
+  int rc = check_dec(src.dec, s);
   if (rc) return rc;
   const MetaLayout m = meta_layout(src.count, src.kinds, src.height, src.width);
   const char *base = static_cast<const char *>(p.meta);
@@ -1263,23 +1221,19 @@ int prepare_codes(const Source &src, const Prepared &p, hipStream_t s, const cha
   if (p.total_chunks < 0 || p.meta_bytes < m.bytes ||
       p.code_bytes < p.total_chunks * 512 + (p.total_chunks / kGroupChunks + nslices + 1) * 128)
     return fail(SUB1_ERR_SHAPE, "%s: buffers smaller than the layout needs", who);
-  uint16_t *codes = static_cast<uint16_t *>(const_cast<void *>(p.codes));
-  uint16_t *ckpt = codes + p.total_chunks * 256;
-  const int group_shift = t->single_codes - t->single_codes / 8;
+  uint2 *stream = static_cast<uint2 *>(const_cast<void *>(p.codes));
+  uint16_t *ckpt = reinterpret_cast<uint16_t *>(stream + p.total_chunks * 64);
   int64_t first_slice = 0;
   for (int i = 0; i < src.kinds; i++) {
     const KindMeta &k = m.k[i];
     const int64_t kslices = static_cast<int64_t>(src.count) * k.slices;
     const int64_t lanes = kslices * 64;
-    interleave_codes_kernel<<<static_cast<unsigned>((lanes + 3) / 4), 256, 0, s>>>(
-        src.w_comp, src.code_base[i], src.row_off[i], t->recode,
+    emit_entries_kernel<<<static_cast<unsigned>((lanes + 255) / 256), 256, 0, s>>>(
+        src.w_comp, src.code_base[i], src.row_off[i], src.dec,
         reinterpret_cast<const uint32_t *>(base + k.slice_base),
         reinterpret_cast<const uint16_t *>(base + k.slice_nch),
-        reinterpret_cast<const uint16_t *>(base + k.row_idx), codes, k.height, k.slices, lanes);
-    checkpoint_kernel<<<static_cast<unsigned>((kslices + 3) / 4), 256, 0, s>>>(
-        codes, t->table, reinterpret_cast<const uint32_t *>(base + k.slice_base),
-        reinterpret_cast<const uint16_t *>(base + k.slice_nch), ckpt, first_slice, kslices,
-        group_shift);
+        reinterpret_cast<const uint16_t *>(base + k.row_idx), stream, ckpt, k.height, k.width,
+        k.slices, first_slice, lanes);
     first_slice += kslices;
   }
   HIP_TRY(hipGetLastError());
@@ -1315,7 +1269,7 @@ size_t plan_small(PreparedArgs &a, int kinds, int tokens, int cus, int waves, si
     for (int per_wg = 1; per_wg <= waves; per_wg *= 2) {
       Option o;
       o.split = waves / per_wg < groups_pow2 ? waves / per_wg : groups_pow2;
-      o.partials = o.split > 1 ? static_cast<size_t>(per_wg) * k.groups_max * 512 : 0;
+      o.partials = o.split > 1 ? static_cast<size_t>(per_wg) * k.groups_max * 256 : 0;
       if (o.partials > lds_room) continue;
       if (o.split == 1 && per_wg != waves) continue;
       o.parts = (k.slices + per_wg - 1) / per_wg;
@@ -1378,17 +1332,13 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
                   static_cast<long long>(sub1_moe_workspace_bytes(tokens, d_ff)));
     if (misaligned(workspace, 256)) return fail(SUB1_ERR_ALIGN, "%s: misaligned workspace", who);
   }
-  const DeviceTables *t = nullptr;
-  int rc = device_tables(s, &t);
-  if (rc) return rc;
   const MetaLayout m = meta_layout(p.count, p.kinds, p.height, p.width);
   if (p.meta_bytes < m.bytes) return fail(SUB1_ERR_SHAPE, "%s: meta smaller than its layout", who);
   const char *base = static_cast<const char *>(p.meta);
 
   PreparedArgs a;
-  a.table = t->table;
-  a.codes = static_cast<const uint16_t *>(p.codes);
-  a.ckpt = a.codes + p.total_chunks * 256;
+  a.stream = static_cast<const uint2 *>(p.codes);
+  a.ckpt = reinterpret_cast<const uint16_t *>(a.stream + p.total_chunks * 64);
   a.kinds = p.kinds;
   int wmax = 0;
   for (int i = 0; i < 2; i++) {
@@ -1401,8 +1351,6 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     const KindMeta &k = m.k[i];
     ka.slice_base = reinterpret_cast<const uint32_t *>(base + k.slice_base);
     ka.slice_nch = reinterpret_cast<const uint16_t *>(base + k.slice_nch);
-    ka.slice_nfull = reinterpret_cast<const uint16_t *>(base + k.slice_nfull);
-    ka.row_len = reinterpret_cast<const uint16_t *>(base + k.row_len);
     ka.row_idx = reinterpret_cast<const uint16_t *>(base + k.row_idx);
     ka.minmax = reinterpret_cast<const uint32_t *>(base + k.minmax);
     ka.slices = k.slices;
@@ -1431,14 +1379,11 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   }
   a.tokens = tokens;
   a.experts = p.count;
-  a.table_words = (t->words + 3) & ~3;   // the device copy is zero-padded to the maximum
-  a.single_codes = t->single_codes;
-  a.group_shift = t->single_codes - t->single_codes / 8;
   a.xdwords = activation_dwords(wmax);
   a.hdwords = 0;
   a.spin_limit = 1 << 24;
   const size_t lds_limit = 160 * 1024 - 64;
-  const size_t lds_base = (static_cast<size_t>(a.table_words) + a.xdwords) * 4;
+  const size_t lds_base = static_cast<size_t>(a.xdwords) * 4;
   if (lds_base > lds_limit) return fail(SUB1_ERR_SHAPE, "%s: width %d does not fit LDS", who, wmax);
   // Tiles.  Whole matrices when the tokens alone keep every compute unit busy;
   // otherwise each matrix is cut into parts, down to one slice per wavefront
@@ -1481,7 +1426,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   if (tiles > INT32_MAX - (1 << 20)) return fail(SUB1_ERR_SHAPE, "%s: too many tiles", who);
   // At least a token per compute unit: a workgroup takes whole tokens and keeps
   // h in LDS, if table + x + h fit.
-  const size_t lds_fused = (static_cast<size_t>(a.table_words) + activation_dwords(a.k[0].width) +
+  const size_t lds_fused = (static_cast<size_t>(activation_dwords(a.k[0].width)) +
                             activation_dwords(a.k[1].width)) * 4;
   bool fused = p.kinds == 2 && !small && a.k[0].parts == 1 && a.k[1].parts == 1 &&
                lds_fused <= lds_limit;
@@ -1511,7 +1456,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
       int split = 1;
       while (split * 2 * rest <= waves && split * 2 <= ko.groups_max) split *= 2;
       if (split > 1 &&
-          static_cast<size_t>(rest) * ko.groups_max * 512 <= static_cast<size_t>(a.xdwords) * 4)
+          static_cast<size_t>(rest) * ko.groups_max * 256 <= static_cast<size_t>(a.xdwords) * 4)
         ko.tail_split = split;
     }
     const void *fn = reinterpret_cast<const void *>(moe_prepared_fused_kernel);
@@ -1542,6 +1487,30 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     const int64_t grid = tiles < cus ? tiles : cus;
     moe_prepared_kernel<<<static_cast<unsigned>(grid), 64 * waves, lds, s>>>(a);
   }
+  HIP_TRY(hipGetLastError());
+  return SUB1_OK;
+}
+
+// The symbols of matrix `index` of kind `kind`, read back from the stream.
+int decode_prepared(const Prepared &p, int kind, int index, void *tern_out, hipStream_t s,
+                    const char *who) {
+  if (!p.meta || !p.codes || !tern_out) return fail(SUB1_ERR_NULL, "%s: NULL argument", who);
+  if (kind < 0 || kind >= p.kinds || index < 0 || index >= p.count)
+    return fail(SUB1_ERR_SHAPE, "%s: no matrix %d of kind %d", who, index, kind);
+  if (misaligned(p.meta, 256) || misaligned(p.codes, 256))
+    return fail(SUB1_ERR_ALIGN, "%s: misaligned pointer", who);
+  const MetaLayout m = meta_layout(p.count, p.kinds, p.height, p.width);
+  if (p.meta_bytes < m.bytes) return fail(SUB1_ERR_SHAPE, "%s: meta smaller than its layout", who);
+  const char *base = static_cast<const char *>(p.meta);
+  const KindMeta &k = m.k[kind];
+  const int64_t n = static_cast<int64_t>(k.height) * k.width;
+  uint8_t *out = static_cast<uint8_t *>(tern_out);
+  fill_bytes_kernel<<<static_cast<unsigned>((n + 255) / 256), 256, 0, s>>>(out, n, 0);
+  decode_entries_kernel<<<(k.slices * 64 + 255) / 256, 256, 0, s>>>(
+      static_cast<const uint2 *>(p.codes), reinterpret_cast<const uint32_t *>(base + k.slice_base),
+      reinterpret_cast<const uint16_t *>(base + k.slice_nch),
+      reinterpret_cast<const uint16_t *>(base + k.row_idx), out,
+      static_cast<int64_t>(index) * k.slices, k.slices, k.width);
   HIP_TRY(hipGetLastError());
   return SUB1_OK;
 }
@@ -1656,6 +1625,16 @@ extern "C" int sub1_moe_grouped_prepared(const sub1_moe_prepared *p, const int32
                          "sub1_moe_grouped_prepared");
 }
 
+extern "C" int sub1_moe_prepared_decode(const sub1_moe_prepared *p, int expert, int projection,
+                                        void *tern_out, void *stream) {
+  if (!p) return fail(SUB1_ERR_NULL, "sub1_moe_prepared_decode: NULL argument");
+  if (bad_dims(p->experts, p->d_ff, p->d_model) || bad_dims(p->experts, p->d_model, p->d_ff))
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_prepared_decode: experts %d d_model %d d_ff %d",
+                p->experts, p->d_model, p->d_ff);
+  return decode_prepared(from_moe(p), projection, expert, tern_out,
+                         static_cast<hipStream_t>(stream), "sub1_moe_prepared_decode");
+}
+
 extern "C" int64_t sub1_matrix_prepared_meta_bytes(int count, int height, int width) {
   if (count < 1 || height < 1 || width < 1) return 0;
   return matrix_layout(count, height, width).bytes;
@@ -1704,4 +1683,14 @@ extern "C" int sub1_matvec_prepared(const sub1_matrix_prepared *p, const int32_t
                 p->height, p->width);
   return launch_prepared(from_matrix(p), token_matrix, x, ldx, y, ldy, tokens, nullptr, 0,
                          static_cast<hipStream_t>(stream), "sub1_matvec_prepared");
+}
+
+extern "C" int sub1_matrix_prepared_decode(const sub1_matrix_prepared *p, int matrix,
+                                           void *tern_out, void *stream) {
+  if (!p) return fail(SUB1_ERR_NULL, "sub1_matrix_prepared_decode: NULL argument");
+  if (bad_dims(p->count, p->height, p->width))
+    return fail(SUB1_ERR_SHAPE, "sub1_matrix_prepared_decode: %d matrices of %d x %d", p->count,
+                p->height, p->width);
+  return decode_prepared(from_matrix(p), 0, matrix, tern_out, static_cast<hipStream_t>(stream),
+                         "sub1_matrix_prepared_decode");
 }

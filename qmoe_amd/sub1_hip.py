@@ -225,10 +225,12 @@ class ExpertStack:
 
 
 class PreparedStack:
-    """An ExpertStack copied into the layout the GPU streams at full width
-    (rows ordered by code count, 64-row slices, interleaved and renumbered
-    codes; decode table and activations in LDS).  `forward` has the semantics
-    of ExpertStack.forward and gives identical outputs."""
+    """An ExpertStack decoded once into the form the GPU streams at full width:
+    every row's non-zero weights as 7-bit gap entries, rows ordered by length,
+    64-row slices, entries interleaved 8 bytes per lane; the kernels keep only
+    the activations in LDS.  `forward` has the semantics of
+    ExpertStack.forward; a row's fp32 sum is taken in the stream's own order,
+    so outputs agree with it to rounding, not to the bit."""
 
     def __init__(self, stack):
         lib = _lib.load()
@@ -280,11 +282,21 @@ class PreparedStack:
         ctrl = self.workspace(tokens)[:16].view(torch.int32).tolist()
         return ctrl[1], ctrl[2]
 
+    def decode(self, expert, projection):
+        """uint8 [rows, width]: the symbols of one matrix (projection 0 = wi,
+        1 = wo) read back from the prepared stream."""
+        rows, width = (self.d_ff, self.d_model) if projection == 0 else (self.d_model, self.d_ff)
+        out = torch.empty(rows, width, dtype=torch.uint8, device=self.device)
+        with torch.cuda.device(self.device):
+            _lib.check(_lib.load().sub1_moe_prepared_decode(
+                ctypes.byref(self._c), expert, projection, out.data_ptr(), _stream()))
+        return out
+
 
 class PreparedMatrix:
     """Compressed matrices of one shape copied into the fast layout;
     `matvec_tokens(x, y)` does y[t] += W x[t] like sub1matvec_tokens, in one
-    launch with the decode table in LDS.
+    launch over the prepared stream.
 
     One matrix: the three buffers of a Sub1Linear.  Several: pass lists of
     equally shaped buffers (or stacked tensors plus `code_base`, int64 [count],
@@ -339,3 +351,12 @@ class PreparedMatrix:
         with torch.cuda.device(dev):
             _lib.check(_lib.load().sub1_matvec_prepared(
                 ctypes.byref(self._c), p_tm, p_x, self.width, p_y, self.height, tokens, _stream()))
+
+    def decode(self, matrix=0):
+        """uint8 [height, width]: the symbols of one matrix read back from the
+        prepared stream."""
+        out = torch.empty(self.height, self.width, dtype=torch.uint8, device=self.device)
+        with torch.cuda.device(self.device):
+            _lib.check(_lib.load().sub1_matrix_prepared_decode(
+                ctypes.byref(self._c), matrix, out.data_ptr(), _stream()))
+        return out

@@ -1,6 +1,7 @@
-"""Pins the oracle's three products (sub1o_matvec_lanes: the reference
-kernel's lane order; sub1o_matvec_seq: per-symbol stream order;
-sub1o_matvec_f64: double precision) and the expert FFN:
+"""Pins the oracle's products (sub1o_matvec_lanes: the reference kernel's
+lane order; sub1o_matvec_seq: per-symbol stream order; sub1o_matvec_gap: the
+prepared stream's order; sub1o_matvec_f64: double precision) and the expert
+FFN:
 
   * matvec_f64 against numpy's float64 GEMV on the dequantised matrix;
   * both fp32 orders against it within the a-priori bound
@@ -8,7 +9,10 @@ sub1o_matvec_f64: double precision) and the expert FFN:
     (bf16 rounding of the result plus fp32 accumulation);
   * closed forms: x = e_k returns column k exactly, x = 1 returns
     n_min*min + n_max*max, an all-zero row returns 0;
-  * the in-place accumulate: y preset to a value gets bf16(y + bf16(res)).
+  * the in-place accumulate: y preset to a value gets bf16(y + bf16(res));
+  * the prepared stream's entries (sub1o_gap_entries): hand-worked rows, an
+    independent numpy writer working from the symbols instead of the codes,
+    and a reader that walks the entries back to the row.
 The tolerance the task states for outputs is 1e-2 relative; the bound above
 is tighter and is what the tests assert.
 """
@@ -52,6 +56,7 @@ def test_fp32_orders_within_bound(oracle):
         exact, sum_abs = dense_f64(t, mm, x)
         assert within_bound(oracle.matvec_lanes(codes, row_off, mm, x), exact, sum_abs)
         assert within_bound(oracle.matvec_seq(codes, row_off, mm, x), exact, sum_abs)
+        assert within_bound(oracle.matvec_gap(codes, row_off, mm, x), exact, sum_abs)
 
 
 def test_unit_vector_picks_a_column(oracle):
@@ -61,7 +66,7 @@ def test_unit_vector_picks_a_column(oracle):
     for k in (0, 1, 27, 28, 99, 199):
         x = np.zeros(200, dtype=np.uint16)
         x[k] = one
-        for fn in (oracle.matvec_lanes, oracle.matvec_seq):
+        for fn in (oracle.matvec_lanes, oracle.matvec_seq, oracle.matvec_gap):
             y = fn(codes, row_off, mm, x)
             assert np.array_equal(so.bf16_bits_to_f32(y), so.bf16_bits_to_f32(w[:, k]))
 
@@ -101,10 +106,94 @@ def test_expert_ffn_is_two_products_with_relu(oracle):
     wi = oracle.encode(ti) + (mi,)
     wo = oracle.encode(to) + (mo,)
     x = so.synthetic_activation(d_model, 23)
-    for order, fn in ((0, oracle.matvec_lanes), (1, oracle.matvec_seq)):
+    for order, fn in ((0, oracle.matvec_lanes), (1, oracle.matvec_seq), (2, oracle.matvec_gap)):
         y, h = oracle.expert_ffn(wi, wo, x, order=order)
         h_ref = fn(wi[0], wi[1], mi, x)
         h_ref = np.where(so.bf16_bits_to_f32(h_ref) > 0, h_ref, 0).astype(np.uint16)
         assert np.array_equal(h, h_ref)
         assert np.array_equal(y, fn(wo[0], wo[1], mo, h_ref))
     assert (so.bf16_bits_to_f32(h) > 0).any() and (h == 0).any()
+
+
+# ---------------------------------------------------- prepared-stream entries --
+
+def entries_from_symbols(row):
+    """The steps of a row, written from its symbols: position 3c + s for symbol
+    s at column c, zeros at every multiple of 3, steps of at most 127."""
+    steps, j = [], 0
+    for c in np.flatnonzero(row):
+        target = 3 * int(c) + int(row[c])
+        while target - j > 127:
+            z = max(v for v in range(j + 1, j + 128) if v % 3 == 0)
+            steps.append(z - j)
+            j = z
+        steps.append(target - j)
+        j = target
+    if j % 3:
+        steps.append(3 - j % 3)
+    return np.array(steps, dtype=np.uint8)
+
+
+def symbols_from_entries(steps, width):
+    row = np.zeros(width, dtype=np.int32)
+    j = 0
+    for s in steps:
+        j += int(s)
+        if j % 3:
+            assert row[j // 3] == 0
+            row[j // 3] = j % 3
+    return row, j
+
+
+def test_gap_entries_by_hand(oracle):
+    def entries_of(row):
+        t = np.array([row], dtype=np.int32)
+        codes, row_off = oracle.encode(t)
+        return list(oracle.gap_entries(codes, t.shape[1]))
+    assert entries_of([0] * 64) == []
+    assert entries_of([1] + [0] * 63) == [1, 2]            # position 1, then on to the zero at 3
+    assert entries_of([2] + [0] * 63) == [2, 1]
+    assert entries_of([0, 2, 1] + [0] * 61) == [5, 2, 2]   # 3*1+2 = 5, 3*2+1 = 7, zero at 9
+    # a symbol 2 at column 100 stands at 302: 0 -> 126 -> 252 -> 302 -> 303
+    assert entries_of([0] * 100 + [2] + [0] * 27) == [126, 126, 50, 1]
+    # 127 is the longest single step: column 42, symbol 1
+    assert entries_of([0] * 42 + [1] + [0] * 21) == [127, 2]
+    assert entries_of([0] * 42 + [2] + [0] * 21) == [126, 2, 1]
+
+
+def test_gap_entries_against_symbols(oracle):
+    for height, width, p0, seed in [(24, 768, 0.9, 3), (8, 3072, 0.97, 4), (16, 333, 0.5, 5),
+                                    (6, 2080, 0.995, 6)]:
+        t, _ = so.synthetic_ternary(height, width, p0, seed)
+        t[1, :] = 0
+        t[2, :] = 2                     # a row without zeros: one entry per column
+        codes, row_off = oracle.encode(t)
+        assert np.array_equal(oracle.decode(codes, row_off, width), t)
+        for r in range(height):
+            steps = oracle.gap_entries(codes[row_off[r]:row_off[r + 1]], width)
+            assert np.array_equal(steps, entries_from_symbols(t[r]))
+            assert steps.max(initial=0) <= 127
+            row, end = symbols_from_entries(steps, width)
+            assert np.array_equal(row, t[r]) and end % 3 == 0 and end <= 3 * width
+
+
+def test_gap_product_sums_in_groups_of_72_entries(oracle):
+    """The order written out in numpy float32: one fused multiply-add per entry
+    (the product of two bf16 is exact in fp32, so a plain multiply and add round
+    the same way), partial sums per 72 entries."""
+    t, mm, codes, row_off, x = make_case(oracle, 12, 2080, 0.88, 31)
+    f = so.bf16_bits_to_f32(mm)
+    xv = so.bf16_bits_to_f32(x)
+    want = np.zeros(12, dtype=np.uint16)
+    for r in range(12):
+        steps = entries_from_symbols(t[r])
+        pos = np.cumsum(steps.astype(np.int64))
+        total = np.float32(0)
+        for g in range(0, len(pos), 72):
+            part = np.float32(0)
+            for j in pos[g:g + 72]:
+                if j % 3:
+                    part = np.float32(part + np.float32(xv[j // 3] * f[2 * r + j % 3 - 1]))
+            total = np.float32(total + part)
+        want[r] = so.f32_to_bf16_bits(np.array([total], np.float32))[0]
+    assert np.array_equal(oracle.matvec_gap(codes, row_off, mm, x), want)
