@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 counter runs of this same
 # command (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a 1 GiB device copy reads on
 # those counters); the summaries are under profiles/.  None where no run was made.
-MEASURED_TRAFFIC = {'c2048-sweep': 4.758e9 + 0.040e9}
+MEASURED_TRAFFIC = {'c2048-sweep': 4.948e9 + 0.034e9}
 
 WORKLOADS = {
     # name: (shape key, experts, p_zero, description)
@@ -37,15 +37,23 @@ WORKLOADS = {
 
 
 def algorithmic_bytes(stack, experts_used):
-    """Bytes the products of one launch have to read and write (per product:
-    2*codes + 4*(H+1) row offsets + 4*H min/max + 2*W input + 2*H output), plus
-    the 61.5 KB decode table once per launch."""
-    total = 15388 * 4
+    """Bytes the products of one launch have to read and write, on the
+    reference's compressed layout (per product: 2*codes + 4*(H+1) row offsets +
+    4*H min/max + 2*W input + 2*H output)."""
+    total = 0
     for e in experts_used:
         total += 2 * int(stack.wi_codes[e]) + 2 * int(stack.wo_codes[e])
         for h, w in ((stack.d_ff, stack.d_model), (stack.d_model, stack.d_ff)):
             total += 4 * (h + 1) + 4 * h + 2 * w + 2 * h
     return total
+
+
+def rel_diff(a, b):
+    """Normwise relative difference of two bf16 results (the kernels on the
+    packed layout and on the prepared stream add in different orders)."""
+    import torch
+    a, b = a.float().double(), b.float().double()
+    return float('%.3g' % (torch.linalg.norm(a - b) / torch.linalg.norm(b)).item())
 
 
 def time_launches(fn, steps, warmup, stream_ptr):
@@ -222,7 +230,7 @@ def main():
                     help='instead of the benchmark, run only the one-product-per-shape protocol')
     ap.add_argument('--probe-gathers', action='store_true',
                     help='instead of the benchmark, measure the time per random-gather '
-                         'instruction from LDS and from global tables (the bound of the decode loop)')
+                         'instruction from LDS and from global tables (the bound of the inner loop)')
     ap.add_argument('--seed', type=int, default=20231116)
     ap.add_argument('--calibrate-copy', type=int, default=0, metavar='MIB',
                     help='instead of the benchmark, run a plain device copy of this many MiB '
@@ -281,8 +289,8 @@ def main():
     tick = time.perf_counter()
     prep = stack.prepare()
     torch.cuda.synchronize()
-    print('prepared in %.2f s: %.3f GB of interleaved codes (%.3f x the packed stream) + %.3f GB '
-          'of column checkpoints' %
+    print('prepared in %.2f s: %.3f GB of interleaved gap entries (%.3f x the packed codes) + '
+          '%.3f GB of position checkpoints' %
           (time.perf_counter() - tick, prep.stream_bytes / 1e9,
            prep.stream_bytes / (2.0 * stack.w_comp.numel()),
            (prep.code_bytes - prep.stream_bytes) / 1e9), file=sys.stderr)
@@ -320,11 +328,12 @@ def main():
         'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
         'ms_per_step': round(ms_per_step, 4),
         'higher_is_better': False, 'scaling': 'weak', 'vs_baseline': None,
-        'dtype': 'bf16 in/out, fp32 accumulate, u16 codes',
+        'dtype': 'bf16 in/out, fp32 accumulate, u16 codes transcoded to 7-bit gap entries',
         'data': 'synthetic (seeded iid ternary experts, N(0,1) bf16 tokens)',
         'config': {'workload': desc, 'experts': experts, 'd_model': d_model, 'd_ff': d_ff,
                    'p_zero': p_zero, 'tokens': experts,
                    'compressed_bytes': stack.compressed_bytes(),
+                   'prepared_stream_bytes': int(prep.stream_bytes),
                    'bits_per_weight': round(16.0 * stack.w_comp.numel()
                                             / (2.0 * experts * d_model * d_ff), 4)},
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS,
@@ -348,7 +357,7 @@ def main():
     y2 = torch.empty_like(x)
     _, us_ref = time_launches(lambda: stack.forward(x, route, y2), 3, 1, stream_ptr)
     also['reference_layout_kernel_us'] = round(us_ref, 1)
-    also['prepared_equals_reference_layout'] = bool(torch.equal(y, y2))
+    also['prepared_vs_reference_layout_rel_diff'] = rel_diff(y, y2)
     # batched decode: 64 tokens routed top-1 by a seeded softmax router (skewed counts)
     t5 = 64
     x5 = synthetic.activations(t5, d_model, args.seed + 3)
@@ -358,7 +367,7 @@ def main():
     y5b = stack.forward(x5, r5)
     also['routed_64_tokens'] = {'us_per_layer': round(us5, 2),
                                 'experts_hit': int(torch.unique(r5).numel()),
-                                'equals_reference_layout_kernel': bool(torch.equal(y5, y5b))}
+                                'vs_reference_layout_kernel_rel_diff': rel_diff(y5, y5b)}
     if not args.no_dense:
         n = min(experts, 128)
         d_us = dense_gemv_us(stack, x, n)

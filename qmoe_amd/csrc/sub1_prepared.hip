@@ -606,6 +606,14 @@ __device__ __forceinline__ float run_slice(SliceWalk &w, const uint2 *stream, co
   return sum;
 }
 
+// The slice a wavefront takes in its pass-th turn through `count` slices that
+// are ordered longest first: back and forth, so that every wavefront gets
+// about the same number of chunks.  >= count: no slice left in this pass.
+__device__ __forceinline__ int slice_of_pass(int pass, int wave, int waves, int count) {
+  const int s = pass * waves + ((pass & 1) ? waves - 1 - wave : wave);
+  return s < count ? s : count;
+}
+
 // How a row's result leaves the kernel.
 enum OutMode { kStoreRelu = 0, kStore = 1, kAccumulate = 2 };
 
@@ -853,18 +861,21 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
       uint16_t *dst = tile_output(a, k, kind, t, mode);
       // the first loads of the stream go out before the wait and the staging
       {
-        int s = s_lo + wave;
+        const int count = s_hi - s_lo;
+        const int passes = (count + waves - 1) / waves;
+        const int64_t first = static_cast<int64_t>(e) * k.slices + s_lo;
+        int s = slice_of_pass(0, wave, waves, count);
         SliceWalk cur;
-        if (s < s_hi) cur = load_slice(a, k, static_cast<int64_t>(e) * k.slices + s);
+        if (s < count) cur = load_slice(a, k, first + s);
         await_activations(a, k, kind, t, xa);
-        for (; s < s_hi; s += waves) {
-          const bool more = s + waves < s_hi;
+        for (int pass = 0; s < count; pass++) {
+          const int s_next = slice_of_pass(pass + 1, wave, waves, count);
           SliceWalk nxt;
-          if (more) nxt = load_slice(a, k, static_cast<int64_t>(e) * k.slices + s + waves);
-          const float res = run_slice(cur, a.stream, xa, nullptr, (s - s_lo) / waves,
-                                      (s_hi - s_lo + waves - 1) / waves);
+          if (s_next < count) nxt = load_slice(a, k, first + s_next);
+          const float res = run_slice(cur, a.stream, xa, nullptr, pass, passes);
           write_row(dst, cur.ridx, res, mode);
-          if (more) cur = nxt;
+          if (s_next < count) cur = nxt;
+          s = s_next;
         }
       }
     }
@@ -916,16 +927,17 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
       continue;
     }
     // wi: x -> relu(h) into LDS
-    int s = wave;
+    const int64_t first_i = static_cast<int64_t>(e) * ki.slices;
+    int s = slice_of_pass(0, wave, waves, ki.slices);
     SliceWalk cur;
-    if (s < ki.slices) cur = load_slice(a, ki, static_cast<int64_t>(e) * ki.slices + s);
+    if (s < ki.slices) cur = load_slice(a, ki, first_i + s);
     stage_activations(xa, a.x + static_cast<int64_t>(t) * a.ldx, ki.width);
     __syncthreads();
-    for (; s < ki.slices; s += waves) {
-      const bool more = s + waves < ki.slices;
+    for (int pass = 0; s < ki.slices; pass++) {
+      const int s_next = slice_of_pass(pass + 1, wave, waves, ki.slices);
       SliceWalk nxt;
-      if (more) nxt = load_slice(a, ki, static_cast<int64_t>(e) * ki.slices + s + waves);
-      const float res = run_slice(cur, a.stream, xa, nullptr, s / waves,
+      if (s_next < ki.slices) nxt = load_slice(a, ki, first_i + s_next);
+      const float res = run_slice(cur, a.stream, xa, nullptr, pass,
                                   (ki.slices + waves - 1) / waves);
       if (cur.ridx != 0xffff) {
         uint32_t out = f32_to_bf16(res);
@@ -934,7 +946,8 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
         p[0] = out;
         p[1] = out << 16;
       }
-      if (more) cur = nxt;
+      if (s_next < ki.slices) cur = nxt;
+      s = s_next;
     }
     // the next token is asked for halfway through this one: early enough to
     // hide the round trip, late enough that the workgroups that started first
@@ -945,18 +958,18 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
     // run of its chunk groups, partial sums into the LDS that held x.
     const int whole = ko.tail_split ? ko.slices - ko.slices % waves : ko.slices;
     const int64_t first = static_cast<int64_t>(e) * ko.slices;
-    s = wave;
+    s = slice_of_pass(0, wave, waves, whole);
     if (s < whole) cur = load_slice(a, ko, first + s);
     __syncthreads();
     uint16_t *dst = a.y + static_cast<int64_t>(t) * a.ldy;
-    for (; s < whole; s += waves) {
-      const bool more = s + waves < whole;
+    for (int pass = 0; s < whole; pass++) {
+      const int s_next = slice_of_pass(pass + 1, wave, waves, whole);
       SliceWalk nxt;
-      if (more) nxt = load_slice(a, ko, first + s + waves);
-      const float res = run_slice(cur, a.stream, ha, nullptr, s / waves,
-                                  (whole + waves - 1) / waves);
+      if (s_next < whole) nxt = load_slice(a, ko, first + s_next);
+      const float res = run_slice(cur, a.stream, ha, nullptr, pass, (whole + waves - 1) / waves);
       write_row(dst, cur.ridx, res, kStore);
-      if (more) cur = nxt;
+      if (s_next < whole) cur = nxt;
+      s = s_next;
     }
     __builtin_amdgcn_s_setprio(0);
     if (ko.tail_split) {
@@ -1242,18 +1255,22 @@ int prepare_codes(const Source &src, const Prepared &p, hipStream_t s, const cha
 
 // Cut of the matrices for a batch that cannot occupy the GPU with a wavefront
 // per slice.  Per projection: a workgroup takes per_wg slices (16 = no sharing)
-// and waves / per_wg wavefronts share each slice, at most one per 32-code group.
+// and waves / per_wg wavefronts share each slice, at most one per chunk group.
 // The choice minimises an estimate of the kernel time in microseconds: a round
-// of workgroups costs a fixed part (table, activations, first loads: they do
-// not overlap with the previous round, LDS admits one workgroup per compute
-// unit) plus the groups that the busiest SIMD walks one after the other.
-// Sets split and parts of every projection; returns the LDS bytes for partial
-// sums, 0 if sharing nothing is estimated best (then nothing is changed).
-// The two constants come from timing every cut of the Switch base and c-2048
-// layers at 1 to 64 tokens on an MI355X.
-constexpr double kRoundFixedUs = 8.0;   // a round of workgroups before its first codeword
-constexpr double kGroupUs = 1.5;        // one 32-code group on a SIMD
-size_t plan_small(PreparedArgs &a, int kinds, int tokens, int cus, int waves, size_t lds_room) {
+// of workgroups costs a fixed part (activations, first loads: they do not
+// overlap with the previous round) plus the groups that the busiest SIMD walks
+// one after the other.  Sets split and parts of every projection; returns the
+// LDS bytes for partial sums, 0 if sharing nothing is estimated best (then
+// nothing is changed), and the estimate in *estimate_us.
+// The constants come from timing every cut of the Switch base, large and
+// c-2048 layers at 1 to 64 tokens on an MI355X; the estimate ranks the cuts and
+// is about 13 us below the measured time of a launch.
+constexpr double kRoundFixedUs = 6.0;      // a round of workgroups before its first entry
+constexpr double kGroupUs = 0.75;          // one group of 72 entries on a SIMD
+constexpr double kResidentBonusUs = 8.0;   // wo workgroups already waiting when h arrives
+constexpr double kLaunchUs = 13.0;         // measured launch minus estimate
+size_t plan_small(PreparedArgs &a, int kinds, int tokens, int cus, int waves, size_t lds_room,
+                  double *estimate_us) {
   struct Option {
     int split, parts;
     int64_t tiles;
@@ -1292,7 +1309,7 @@ size_t plan_small(PreparedArgs &a, int kinds, int tokens, int cus, int waves, si
         // fixed part behind them when h arrives
         const bool resident = o0.tiles + o1.tiles <= cus;
         us += std::max(1.0, static_cast<double>(o1.tiles) / cus) * o1.round_us -
-              (resident ? kRoundFixedUs : 0.0);
+              (resident ? kResidentBonusUs : 0.0);
       }
       if (us < best) {
         best = us;
@@ -1303,6 +1320,7 @@ size_t plan_small(PreparedArgs &a, int kinds, int tokens, int cus, int waves, si
   size_t partials = 0;
   for (int i = 0; i < kinds; i++)
     if (opt[i][pick[i]].partials > partials) partials = opt[i][pick[i]].partials;
+  *estimate_us = best;
   if (partials == 0) return 0;
   for (int i = 0; i < kinds; i++) {
     a.k[i].split = opt[i][pick[i]].split;
@@ -1419,25 +1437,30 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     }
   }
   size_t lds_partials = 0;
-  if (idle_units) lds_partials = plan_small(a, p.kinds, tokens, cus, waves, lds_limit - lds_base);
+  double small_us = 0.0;
+  if (idle_units)
+    lds_partials = plan_small(a, p.kinds, tokens, cus, waves, lds_limit - lds_base, &small_us);
   const bool small = lds_partials != 0;
   int64_t tiles = 0;
   for (int i = 0; i < p.kinds; i++) tiles += static_cast<int64_t>(tokens) * a.k[i].parts;
   if (tiles > INT32_MAX - (1 << 20)) return fail(SUB1_ERR_SHAPE, "%s: too many tiles", who);
   // At least a token per compute unit: a workgroup takes whole tokens and keeps
-  // h in LDS, if table + x + h fit.
+  // h in LDS, if x + h fit.
   const size_t lds_fused = (static_cast<size_t>(activation_dwords(a.k[0].width)) +
                             activation_dwords(a.k[1].width)) * 4;
   bool fused = p.kinds == 2 && !small && a.k[0].parts == 1 && a.k[1].parts == 1 &&
                lds_fused <= lds_limit;
-  if (!fused && p.kinds == 2 && lds_fused <= lds_limit && tokens >= 16 && tokens < cus) {
+  if (!fused && p.kinds == 2 && lds_fused <= lds_limit && tokens < cus) {
     // Fewer tokens than compute units: whole tokens per workgroup leave units
     // idle but pay nothing for cutting the matrices (per-tile staging, h through
-    // memory, waiting).  Measured on the Switch shapes, the cut versions take
-    // about 33 us + tokens / units x (time of one token on one unit), the fused
-    // kernel the time of one token, itself about 8 us + codewords / 5500 per us.
-    const double token_us = 8.0 + static_cast<double>(p.total_chunks) * 256.0 / p.count / 5500.0;
-    if (tokens >= cus * (1.0 - 33.0 / token_us)) {
+    // memory, waiting).  The fused kernel then takes the time of one token,
+    // measured on the Switch shapes as about 8 us + entries / 23400 per us; the
+    // cut versions take the estimate above when wavefronts share slices and
+    // about 33 us + tokens / units x (time of one token) otherwise.
+    const double token_us = 8.0 + static_cast<double>(p.total_chunks) * (64.0 * kFields) /
+                                      p.count / 23400.0;
+    const double cut_us = small ? small_us + kLaunchUs : 33.0 + token_us * tokens / cus;
+    if (token_us < cut_us) {
       fused = true;
       for (int i = 0; i < 2; i++) {
         a.k[i].parts = 1;
