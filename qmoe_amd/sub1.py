@@ -8,8 +8,8 @@ Differences from the reference that a caller can observe:
   * importing works without a GPU (the reference indexes GPUS[-1] at import,
     sub1.py:107-111); the device tables are then empty until a GPU exists;
   * `Sub1Linear.forward` runs all tokens in one launch (the reference loops
-    over tokens, sub1.py:137-142), from a copy of the codes in a GPU-friendly
-    layout that it makes on first use (`Sub1Linear.fast`);
+    over tokens, sub1.py:137-142), from a gap-coded stream of the non-zero
+    weights that it decodes from the codes on first use (`Sub1Linear.fast`);
   * any (height, width) works, not only the six Switch shapes.
 """
 import torch
@@ -57,10 +57,11 @@ class Sub1Linear(nn.Module):
         self.register_buffer('ter_minmax', torch.zeros(2 * height, dtype=torch.bfloat16))
         self.register_buffer('weight', torch.zeros(0, dtype=torch.bfloat16))
 
-    # forward() goes through a copy of the codes in the layout the GPU streams
-    # fastest, made on first use (it costs about as much memory again as w_comp
+    # forward() goes through the prepared stream of the non-zero weights, made
+    # from the codes on first use (it costs about as much memory again as w_comp
     # and is remade when a buffer is replaced or written in place).  Set to
-    # False to run straight from the packed buffers instead.
+    # False to run straight from the packed buffers instead (the two add a
+    # row's terms in different orders and agree to rounding, not to the bit).
     fast = True
 
     def _prepared(self, width):

@@ -162,7 +162,7 @@ def test_layer_launch_replays_from_a_graph(gpu):
         x = synthetic.activations(tokens, d_model, seed=62)
         route = (torch.arange(tokens, dtype=torch.int32, device='cuda') * 3) % 8
         y = torch.empty_like(x)
-        prep.forward(x, route, y)            # first call: tables, workspace
+        prep.forward(x, route, y)            # first call: workspace
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
