@@ -473,7 +473,9 @@ def test_extreme_widths_in_every_batch_regime(gpu, oracle, d_model, d_ff):
 
 
 @pytest.mark.parametrize('height,width,p0', SWITCH_SHAPES + [(77, 333, 0.7), (5, 1, 0.5),
-                                                             (130, 15, 0.9), (300, 8192, 0.99)])
+                                                             (130, 15, 0.9), (300, 8192, 0.99),
+                                                             (64, 56, 0.0), (33, 29, 0.3),
+                                                             (1, 4000, 0.95), (200, 8192, 0.9995)])
 def test_prepared_matrix_product(gpu, oracle, height, width, p0):
     """The single-matrix fast path (what Sub1Linear.forward uses): y += W x for
     several tokens, bit-exact against the oracle, accumulating like sub1matvec."""
@@ -569,3 +571,42 @@ def test_prepared_matrix_set_with_token_matrix(gpu, oracle):
             assert np.array_equal(got[t], want), (t, m)
     with pytest.raises(ValueError):
         pm.matvec_tokens(bf16_dev(xs), y)            # several matrices need token_matrix
+
+
+def test_prepared_stream_edge_rows(gpu, oracle):
+    """Rows the gap stream treats specially: no non-zero at all (no entries, the
+    slice still has one chunk), one non-zero in the last column after a gap of
+    many steps over zeros, no zero at all (one entry per column), a row whose
+    min equals its max (the packer codes every weight as symbol 2), and rows of
+    very different lengths in one 64-row slice."""
+    sub1, op = gpu
+    height, width = 70, 1500
+    t, mm = so.synthetic_ternary(height, width, 0.9, seed=4242)
+    t[0, :] = 0
+    t[1, :] = 0
+    t[1, width - 1] = 2
+    t[2, :] = 1
+    t[3, :] = 2
+    t[4, :] = 0
+    t[4, 0] = 1
+    t[5, :] = 0
+    t[5, 42] = 1                     # a step of exactly 127
+    t[6, :] = 0
+    t[6, 42] = 2                     # 128: one step too long
+    t[65:, :] = 0                    # the second slice holds only empty rows
+    mm[2 * 3] = mm[2 * 3 + 1]        # row 3: min == max
+    codes, row_off = oracle.encode(t)
+    x = so.synthetic_activation(width, 77)
+    w_comp = torch.from_numpy(codes.view(np.int16)).cuda()
+    pm = op.PreparedMatrix(sub1.DEC[0], w_comp, torch.from_numpy(row_off).cuda(), bf16_dev(mm), width)
+    assert np.array_equal(pm.decode().cpu().numpy(), t)
+    for tokens in (1, 3):
+        xs = np.stack([x] * tokens)
+        y = torch.zeros((tokens, height), dtype=torch.bfloat16, device='cuda')
+        pm.matvec_tokens(bf16_dev(xs), y)
+        want = oracle.matvec_gap(codes, row_off, mm, x)
+        for i in range(tokens):
+            assert np.array_equal(bits_host(y[i]), want)
+    assert want[0] == 0 and want[70 - 1] == 0
+    c = dict(t=t, mm=mm, codes=codes, row_off=row_off, x=x)
+    check_product(oracle, c, want, prepared=True)
