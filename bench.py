@@ -358,6 +358,8 @@ def main():
     _, us_ref = time_launches(lambda: stack.forward(x, route, y2), 3, 1, stream_ptr)
     also['reference_layout_kernel_us'] = round(us_ref, 1)
     also['prepared_vs_reference_layout_rel_diff'] = rel_diff(y, y2)
+    if not also['prepared_vs_reference_layout_rel_diff'] <= 1e-2:
+        raise SystemExit('the prepared kernel and the packed-layout kernel disagree on the sweep')
     # batched decode: 64 tokens routed top-1 by a seeded softmax router (skewed counts)
     t5 = 64
     x5 = synthetic.activations(t5, d_model, args.seed + 3)

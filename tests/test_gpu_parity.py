@@ -333,6 +333,21 @@ def test_prepare_rejects_foreign_dictionary(gpu, oracle):
         bad.prepare()
 
 
+def test_prepare_rejects_rows_that_do_not_cover_the_width(gpu, oracle):
+    """A row_off that cuts a row's codes short (or a width the codes were not
+    made for) is refused when the stream is prepared, not decoded into garbage."""
+    from qmoe_amd._lib import Sub1Error
+    sub1, op = gpu
+    c = dev_case(oracle, 96, 200, 0.8, seed=710)
+    bad = c['row_off_d'].clone()
+    bad[40] -= 1                                  # row 39 loses a code, row 40 gains it
+    with pytest.raises(Sub1Error):
+        op.PreparedMatrix(sub1.DEC[0], c['w_comp'], bad, c['mm_d'], 200)
+    with pytest.raises(Sub1Error):
+        op.PreparedMatrix(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], 204)
+    op.PreparedMatrix(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], 200)
+
+
 def test_large_stack_paths_agree_and_match_oracle(gpu, oracle):
     """128 Switch-base experts, one token each (the Switch-base-128 layer):
     many tiles on many compute units, so the hand-off of the intermediate
