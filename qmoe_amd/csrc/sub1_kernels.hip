@@ -502,7 +502,7 @@ hipEvent_t g_ev_begin = nullptr, g_ev_end = nullptr;
 
 extern "C" const char *sub1_last_error(void) { return sub1::g_err.c_str(); }
 
-extern "C" int sub1_abi_version(void) { return 1; }
+extern "C" int sub1_abi_version(void) { return 2; }
 
 extern "C" int sub1_matvec_tokens(const int32_t *dec, const int16_t *w_comp,
                                   const int32_t *row_off, const void *ter_minmax,
