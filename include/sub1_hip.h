@@ -154,14 +154,16 @@ int sub1_moe_grouped(const sub1_moe_stack *stack, const int32_t *token_expert,
  * reference).  Preparing decodes the stack once and stores every row's
  * non-zero weights as a gap-coded stream the GPU walks at full width:
  *
- *   - a position j counts dwords of the activation array the kernels keep in
- *     LDS: dword 0 is zero, column c has (x[c], 0) at 3c+1 (read for a row-min
- *     weight), (0, x[c]) at 3c+2 (row-max weight) and a zero at 3c+3;
+ *   - the kernels keep the activations in LDS by physical column: real column
+ *     c is physical column q = c + c/16 + 1, every 17th physical column (0, 17,
+ *     34, ...) holds zeros; a physical column is two dwords, (x[c], 0) read for
+ *     a row-min weight and (0, x[c]) read for a row-max weight.  A position
+ *     p = 2q + symbol - 1 therefore names a weight's column and symbol;
  *   - a row is a sequence of 7-bit entries, each the step from the row's
- *     position to the next: to the next non-zero weight's dword, or, where
- *     that is more than 127 away, to the farthest zero dword within reach;
- *     after its last non-zero a row steps to the next zero dword (if it is
- *     not on one) and pads with steps of 0;
+ *     position (0 at the start) to the next: to the next non-zero weight's
+ *     position, or, where that is more than 127 away, to the farthest zero
+ *     column within reach (a multiple of 34); after its last non-zero a row
+ *     steps to the next multiple of 34 and pads with steps of 0;
  *   - nine entries make a chunk (8 bytes, entry q in bits 7q..7q+6, bit 63
  *     zero); rows are ordered by chunk count and cut into 64-row slices, each
  *     as long as its longest row and at least one chunk; chunk c of lane l of
@@ -194,7 +196,7 @@ int sub1_moe_grouped(const sub1_moe_stack *stack, const int32_t *token_expert,
  * the device; projection 0 = wi, 1 = wo): the check that preparing kept every
  * weight.
  */
-#define SUB1_PREPARED_MAX_WIDTH 8192
+#define SUB1_PREPARED_MAX_WIDTH 12288
 
 typedef struct sub1_moe_prepared {
   const void *meta;

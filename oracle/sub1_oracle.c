@@ -371,19 +371,25 @@ void sub1o_matvec_seq(const int32_t *dec, const uint16_t *codes,
   }
 }
 
-/* The prepared stream's view of a row.  A position j counts dwords of an
- * activation array with a zero at 0 and, per column c, x[c] for a row-min
- * weight at 3c+1, x[c] for a row-max weight at 3c+2, a zero at 3c+3.  The row
- * is the sequence of steps (0..127) that visits its non-zero weights in column
- * order: a step to a non-zero more than 127 away first goes to the farthest
- * zero within reach (the largest multiple of 3 not beyond j+127), repeatedly;
- * after the last non-zero one step goes to the next zero unless the row stands
- * on one.  Writes the steps to out (if not NULL; at most cap) and returns their
- * number, or -1 if the codes do not cover ceil(width/2) pairs. */
+/* The prepared stream's view of a row.  Activations are laid out by physical
+ * column: real column c is physical column q = c + c/16 + 1, every 17th
+ * physical column (0, 17, 34, ...) is a zero column.  A position p = 2q + s - 1
+ * names the column and the symbol (1 = row min, 2 = row max) of a weight; the
+ * positions 34k and 34k+1 are zeros.  The row is the sequence of steps (0..127)
+ * that visits its non-zero weights in column order, starting from 0: a step to
+ * a non-zero more than 127 away first goes to the farthest zero column within
+ * reach (the largest multiple of 34 not beyond p+127), repeatedly; after the
+ * last non-zero one step goes to the next multiple of 34.  Writes the steps to
+ * out (if not NULL; at most cap) and returns their number, or -1 if the codes
+ * do not cover ceil(width/2) pairs. */
 #define SUB1O_GAP_MAX 127
+#define SUB1O_GAP_ZERO 17
+
+static int gap_position(int col, int sym) { return 2 * (col + col / 16 + 1) + sym - 1; }
 
 int sub1o_gap_entries(const int32_t *dec, const uint16_t *codes, int ncodes,
                       int width, uint8_t *out, int cap) {
+  const int period = 2 * SUB1O_GAP_ZERO;
   int n = 0, j = 0, idx = 0;
   for (int c = 0; c < ncodes; c++) {
     int e = codes[c];
@@ -391,9 +397,9 @@ int sub1o_gap_entries(const int32_t *dec, const uint16_t *codes, int ncodes,
     for (int d = 0; d < 2 * npairs && idx + d < width; d++) {
       int t = entry_digit(dec, e, d);
       if (!t) continue;
-      int target = 3 * (idx + d) + t;
+      int target = gap_position(idx + d, t);
       while (target - j > SUB1O_GAP_MAX) {
-        int z = (j + SUB1O_GAP_MAX) / 3 * 3;
+        int z = (j + SUB1O_GAP_MAX) / period * period;
         if (out && n < cap) out[n] = (uint8_t)(z - j);
         n++;
         j = z;
@@ -405,8 +411,9 @@ int sub1o_gap_entries(const int32_t *dec, const uint16_t *codes, int ncodes,
     idx += 2 * npairs;
   }
   if (idx != ((width + 1) & ~1)) return -1;
-  if (j % 3) {
-    if (out && n < cap) out[n] = (uint8_t)(3 - j % 3);
+  if ((j / 2) % SUB1O_GAP_ZERO) {
+    int z = (j + period - 1) / period * period;
+    if (out && n < cap) out[n] = (uint8_t)(z - j);
     n++;
   }
   return n;
@@ -415,7 +422,7 @@ int sub1o_gap_entries(const int32_t *dec, const uint16_t *codes, int ncodes,
 /* The product in the order the prepared-stream kernels add: the row's entries
  * in groups of SUB1O_GAP_GROUP; within a group each entry that stands on an
  * activation adds x * w (w = row min or max) with one fused multiply-add onto a
- * partial sum that starts at zero (entries on a zero dword add nothing); the
+ * partial sum that starts at zero (entries on a zero column add nothing); the
  * partial sums are added, first group first, onto the row's sum; bf16; +=. */
 #define SUB1O_GAP_GROUP 72
 
@@ -431,7 +438,7 @@ int sub1o_matvec_gap(const int32_t *dec, const uint16_t *codes,
       free(steps);
       return 1 + r;
     }
-    float w[3] = {0.f, bf16_to_f32(ter_minmax[2 * r]), bf16_to_f32(ter_minmax[2 * r + 1])};
+    float w[2] = {bf16_to_f32(ter_minmax[2 * r]), bf16_to_f32(ter_minmax[2 * r + 1])};
     float sum = 0.f;
     int j = 0;
     for (int i0 = 0; i0 < n; i0 += SUB1O_GAP_GROUP) {
@@ -439,7 +446,8 @@ int sub1o_matvec_gap(const int32_t *dec, const uint16_t *codes,
       int i1 = i0 + SUB1O_GAP_GROUP < n ? i0 + SUB1O_GAP_GROUP : n;
       for (int i = i0; i < i1; i++) {
         j += steps[i];
-        if (j % 3) p = fmaf(bf16_to_f32(x[j / 3]), w[j % 3], p);
+        int q = j / 2;
+        if (q % SUB1O_GAP_ZERO) p = fmaf(bf16_to_f32(x[q - 1 - q / SUB1O_GAP_ZERO]), w[j & 1], p);
       }
       sum += p;
     }

@@ -10,7 +10,7 @@ DICT_ENTRIES = 65536
 DEC_WORDS = 2 * DICT_ENTRIES
 TRIE_ROWS = DICT_ENTRIES + 1
 MAX_WIDTH = 12288
-PREPARED_MAX_WIDTH = 8192
+PREPARED_MAX_WIDTH = 12288
 
 _vp = ctypes.c_void_p
 _int = ctypes.c_int

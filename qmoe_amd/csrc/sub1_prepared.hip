@@ -6,11 +6,12 @@
 //
 //   * every row's dictionary codes are decoded once and its non-zero weights
 //     written as a gap-coded stream: 7-bit entries, each the distance to the
-//     next non-zero in units of the LDS activation array (3 dwords per column:
-//     the activation for a row-min weight, for a row-max weight, a zero), so an
-//     entry names the column and the symbol at once; gaps beyond 127 units step
-//     over zero dwords.  At 10% non-zeros this is 0.72 bit per weight against
-//     0.69 for the dictionary codes, and the kernel needs no decode table;
+//     next non-zero in units of the LDS activation array (2 dwords per column:
+//     the activation for a row-min weight and for a row-max weight; every 17th
+//     column is a zero column), so an entry names the column and the symbol at
+//     once; gaps beyond 127 units step over zero columns.  At 10% non-zeros
+//     this is 0.72 bit per weight against 0.69 for the dictionary codes, and
+//     the kernel needs no decode table;
 //   * rows of every matrix are ordered by entry count and cut into slices of
 //     64 rows (one wavefront lane each);
 //   * a slice's entries are interleaved in chunks of 9 (8 bytes) per lane:
@@ -155,19 +156,34 @@ __device__ __forceinline__ int for_each_nonzero(const uint16_t *codes, int n,
   return col;
 }
 
-// Non-zeros to entries.  The position j counts dwords of the LDS activation
-// array: 0 is a zero, column c has x for a row-min weight at 1 + 3c, for a
-// row-max weight at 2 + 3c, and a zero at 3 + 3c.  An entry is the step to the
-// next position, 0..127.  A longer gap goes over zeros (every third dword), as
-// far as each step reaches; after the last non-zero the row parks on the next
-// zero, where steps of 0 pad it to the length of its slice.
+// Positions.  The kernels keep the activations in LDS by physical column: real
+// column c is physical column q = c + c/16 + 1, so that every 17th physical
+// column (0, 17, 34, ...) is a zero column; a physical column is two dwords,
+// and position p = 2q + (symbol - 1) is the dword a weight with that symbol
+// reads: (x, 0) for a row-min weight, (0, x) for a row-max weight, zero in a
+// zero column.  The low bit of a position is the symbol, the rest the column.
+constexpr int kZeroPeriod = 17;                  // physical columns from one zero column to the next
+__host__ __device__ constexpr int physical_column(int c) { return c + (c >> 4) + 1; }
+__host__ __device__ constexpr int position_of(int c, int sym) {
+  return 2 * physical_column(c) + (sym - 1);
+}
+// Physical columns an array for `width` real columns needs: up to and including
+// the zero column that follows the last real one.
+__host__ __device__ constexpr int physical_columns(int width) {
+  return (physical_column(width - 1) / kZeroPeriod + 1) * kZeroPeriod + 1;
+}
+
+// Non-zeros to entries.  An entry is the step from the row's position (0 at
+// the start) to the next, 0..127.  A longer gap goes over zero columns, as far
+// as each step reaches; after the last non-zero the row parks on the next zero
+// column, where steps of 0 pad it to the length of its slice.
 struct EntryWriter {
   int j = 0;
   template <class E>
   __device__ __forceinline__ void nonzero(int col, int sym, E &&emit) {
-    const int target = 3 * col + sym;
+    const int target = position_of(col, sym);
     while (target - j > kMaxStep) {
-      const int z = (j + kMaxStep) / 3 * 3;
+      const int z = (j + kMaxStep) / (2 * kZeroPeriod) * (2 * kZeroPeriod);
       emit(z - j, j);
       j = z;
     }
@@ -176,8 +192,9 @@ struct EntryWriter {
   }
   template <class E>
   __device__ __forceinline__ void park(E &&emit) {
-    const int z = (j + 2) / 3 * 3;
-    if (z != j) emit(z - j, j);
+    if ((j >> 1) % kZeroPeriod == 0) return;
+    const int z = (j + 2 * kZeroPeriod - 1) / (2 * kZeroPeriod) * (2 * kZeroPeriod);
+    emit(z - j, j);
     j = z;
   }
 };
@@ -359,8 +376,10 @@ __global__ __launch_bounds__(256) void decode_entries_kernel(
     const unsigned long long w = (static_cast<unsigned long long>(cw.y) << 32) | cw.x;
     for (int q = 0; q < kFields; q++) {
       j += static_cast<int>(w >> (kFieldBits * q)) & kMaxStep;
-      if (j % 3 != 0 && j / 3 < width)
-        out[static_cast<int64_t>(ridx) * width + j / 3] = static_cast<uint8_t>(j % 3);
+      const int pc = j >> 1;   // physical column
+      const int col = pc - 1 - pc / kZeroPeriod;
+      if (pc % kZeroPeriod != 0 && col < width)
+        out[static_cast<int64_t>(ridx) * width + col] = static_cast<uint8_t>((j & 1) + 1);
     }
   }
 }
@@ -406,13 +425,11 @@ struct PreparedArgs {
   int spin_limit;
 };
 
-// Activations in LDS: dword 0 is zero, then 3 dwords per column,
-//   [A, B, 0],  A = (x, 0), B = (0, x) as bf16 pairs;
-// position 3c + 1 is column c's value for a row-min weight, 3c + 2 for a row-max
-// weight, every third dword a zero for long gaps and padding.  Rounded up to
-// whole 16 bytes (what follows in LDS stays aligned).
+// Activations in LDS: two dwords per physical column, A = (x, 0) and B = (0, x)
+// as bf16 pairs, zeros in the zero columns (see "Positions" above).  Rounded up
+// to whole 16 bytes (what follows in LDS stays aligned).
 __host__ __device__ constexpr int activation_dwords(int width) {
-  return (3 * width + 1 + 3) / 4 * 4;
+  return (2 * physical_columns(width) + 3) / 4 * 4;
 }
 
 // Every load of a thread is in flight before its first LDS store, so a tile
@@ -421,7 +438,10 @@ __device__ __forceinline__ void stage_activations(uint32_t *xa, const uint16_t *
   const int npairs = (width + 1) / 2;
   const int step = blockDim.x;
   const bool aligned = (reinterpret_cast<uintptr_t>(x) & 3u) == 0;
-  if (threadIdx.x == 0) xa[0] = 0u;
+  for (int z = threadIdx.x * kZeroPeriod; z < physical_columns(width); z += step * kZeroPeriod) {
+    xa[2 * z] = 0u;
+    xa[2 * z + 1] = 0u;
+  }
   for (int m0 = threadIdx.x; m0 < npairs; m0 += 4 * step) {
     uint32_t v[4];
 #pragma unroll
@@ -439,14 +459,13 @@ __device__ __forceinline__ void stage_activations(uint32_t *xa, const uint16_t *
     for (int u = 0; u < 4; u++) {
       const int m = m0 + u * step;
       if (m < npairs) {
-        uint32_t *p = xa + 1 + 6 * m;
+        // columns 2m and 2m+1 are neighbours among the physical columns too
+        uint32_t *p = xa + 2 * physical_column(2 * m);
         p[0] = v[u] & 0xffffu;
         p[1] = v[u] << 16;
-        p[2] = 0u;
         if (2 * m + 1 < width) {
-          p[3] = v[u] >> 16;
-          p[4] = v[u] & 0xffff0000u;
-          p[5] = 0u;
+          p[2] = v[u] >> 16;
+          p[3] = v[u] & 0xffff0000u;
         }
       }
     }
@@ -942,7 +961,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
       if (cur.ridx != 0xffff) {
         uint32_t out = f32_to_bf16(res);
         if (out & 0x8000u) out = 0;   // relu between the projections, on the bf16 value
-        uint32_t *p = ha + 1 + 3 * cur.ridx;
+        uint32_t *p = ha + 2 * physical_column(cur.ridx);
         p[0] = out;
         p[1] = out << 16;
       }

@@ -466,7 +466,7 @@ def test_token_per_workgroup_tiles_with_dropped_tokens(gpu, oracle):
     assert close(y, stack.forward(x, route))
 
 
-@pytest.mark.parametrize('d_model,d_ff', [(64, 8192), (8192, 64), (2, 2)])
+@pytest.mark.parametrize('d_model,d_ff', [(64, 12288), (12288, 64), (2, 2)])
 def test_extreme_widths_in_every_batch_regime(gpu, oracle, d_model, d_ff):
     """The widest activations the fast layout takes and the narrowest, from one
     token to more tokens than compute units: every regime must give the same
@@ -490,7 +490,8 @@ def test_extreme_widths_in_every_batch_regime(gpu, oracle, d_model, d_ff):
 @pytest.mark.parametrize('height,width,p0', SWITCH_SHAPES + [(77, 333, 0.7), (5, 1, 0.5),
                                                              (130, 15, 0.9), (300, 8192, 0.99),
                                                              (64, 56, 0.0), (33, 29, 0.3),
-                                                             (1, 4000, 0.95), (200, 8192, 0.9995)])
+                                                             (1, 4000, 0.95), (200, 8192, 0.9995),
+                                                             (40, 12288, 0.97)])
 def test_prepared_matrix_product(gpu, oracle, height, width, p0):
     """The single-matrix fast path (what Sub1Linear.forward uses): y += W x for
     several tokens, bit-exact against the oracle, accumulating like sub1matvec."""
@@ -605,9 +606,9 @@ def test_prepared_stream_edge_rows(gpu, oracle):
     t[4, :] = 0
     t[4, 0] = 1
     t[5, :] = 0
-    t[5, 42] = 1                     # a step of exactly 127
+    t[5, 59] = 2                     # a step of exactly 127
     t[6, :] = 0
-    t[6, 42] = 2                     # 128: one step too long
+    t[6, 60] = 1                     # 128: one step too long
     t[65:, :] = 0                    # the second slice holds only empty rows
     mm[2 * 3] = mm[2 * 3 + 1]        # row 3: min == max
     codes, row_off = oracle.encode(t)

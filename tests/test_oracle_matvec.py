@@ -117,20 +117,33 @@ def test_expert_ffn_is_two_products_with_relu(oracle):
 
 # ---------------------------------------------------- prepared-stream entries --
 
+def position(c, sym):
+    """Dword of the activation array a weight reads: two dwords per physical
+    column, real column c being physical column c + c // 16 + 1 (every 17th
+    physical column holds zeros), the low bit the symbol."""
+    return 2 * (c + c // 16 + 1) + sym - 1
+
+
+def is_zero_position(p):
+    return (p // 2) % 17 == 0
+
+
 def entries_from_symbols(row):
-    """The steps of a row, written from its symbols: position 3c + s for symbol
-    s at column c, zeros at every multiple of 3, steps of at most 127."""
+    """The steps of a row, written from its symbols: steps of at most 127, long
+    gaps over the farthest zero column within reach, a last step onto the next
+    zero column."""
     steps, j = [], 0
     for c in np.flatnonzero(row):
-        target = 3 * int(c) + int(row[c])
+        target = position(int(c), int(row[c]))
         while target - j > 127:
-            z = max(v for v in range(j + 1, j + 128) if v % 3 == 0)
+            z = max(v for v in range(j + 1, j + 128) if v % 34 == 0)
             steps.append(z - j)
             j = z
         steps.append(target - j)
         j = target
-    if j % 3:
-        steps.append(3 - j % 3)
+    if not is_zero_position(j):
+        z = min(v for v in range(j, j + 40) if v % 34 == 0)
+        steps.append(z - j)
     return np.array(steps, dtype=np.uint8)
 
 
@@ -139,9 +152,11 @@ def symbols_from_entries(steps, width):
     j = 0
     for s in steps:
         j += int(s)
-        if j % 3:
-            assert row[j // 3] == 0
-            row[j // 3] = j % 3
+        if not is_zero_position(j):
+            q = j // 2
+            c = q - 1 - q // 17
+            assert row[c] == 0
+            row[c] = (j & 1) + 1
     return row, j
 
 
@@ -151,14 +166,21 @@ def test_gap_entries_by_hand(oracle):
         codes, row_off = oracle.encode(t)
         return list(oracle.gap_entries(codes, t.shape[1]))
     assert entries_of([0] * 64) == []
-    assert entries_of([1] + [0] * 63) == [1, 2]            # position 1, then on to the zero at 3
-    assert entries_of([2] + [0] * 63) == [2, 1]
-    assert entries_of([0, 2, 1] + [0] * 61) == [5, 2, 2]   # 3*1+2 = 5, 3*2+1 = 7, zero at 9
-    # a symbol 2 at column 100 stands at 302: 0 -> 126 -> 252 -> 302 -> 303
-    assert entries_of([0] * 100 + [2] + [0] * 27) == [126, 126, 50, 1]
-    # 127 is the longest single step: column 42, symbol 1
-    assert entries_of([0] * 42 + [1] + [0] * 21) == [127, 2]
-    assert entries_of([0] * 42 + [2] + [0] * 21) == [126, 2, 1]
+    # column 0 is physical column 1: positions 2 (min) and 3 (max); the next zero column is 17
+    assert entries_of([1] + [0] * 63) == [2, 32]
+    assert entries_of([2] + [0] * 63) == [3, 31]
+    # column 1 max -> 5, column 2 min -> 6, then on to 34
+    assert entries_of([0, 2, 1] + [0] * 61) == [5, 1, 28]
+    # column 15 is physical 16, column 16 physical 18 (17 holds zeros)
+    assert entries_of([0] * 15 + [1, 2] + [0] * 47) == [32, 5, 31]
+    # column 100 is physical 107: a max weight stands at 215 = 102 + 113 (102 = 3 * 34 is the
+    # farthest zero column within 127 of the start); 238 = 7 * 34 follows
+    assert entries_of([0] * 100 + [2] + [0] * 27) == [102, 113, 23]
+    # column 200 is physical 213, a min weight at 426 = 102 + 102 + 102 + 120
+    assert entries_of([0] * 200 + [1] + [0] * 55) == [102, 102, 102, 120, 16]
+    # 127 is the longest single step: column 59 is physical 63, its max weight at 127
+    assert entries_of([0] * 59 + [2] + [0] * 4) == [127, 9]
+    assert entries_of([0] * 60 + [1] + [0] * 3) == [102, 26, 8]
 
 
 def test_gap_entries_against_symbols(oracle):
@@ -174,7 +196,7 @@ def test_gap_entries_against_symbols(oracle):
             assert np.array_equal(steps, entries_from_symbols(t[r]))
             assert steps.max(initial=0) <= 127
             row, end = symbols_from_entries(steps, width)
-            assert np.array_equal(row, t[r]) and end % 3 == 0 and end <= 3 * width
+            assert np.array_equal(row, t[r]) and is_zero_position(end)
 
 
 def test_gap_product_sums_in_groups_of_72_entries(oracle):
@@ -192,8 +214,9 @@ def test_gap_product_sums_in_groups_of_72_entries(oracle):
         for g in range(0, len(pos), 72):
             part = np.float32(0)
             for j in pos[g:g + 72]:
-                if j % 3:
-                    part = np.float32(part + np.float32(xv[j // 3] * f[2 * r + j % 3 - 1]))
+                if not is_zero_position(j):
+                    q = j // 2
+                    part = np.float32(part + np.float32(xv[q - 1 - q // 17] * f[2 * r + (j & 1)]))
             total = np.float32(total + part)
         want[r] = so.f32_to_bf16_bits(np.array([total], np.float32))[0]
     assert np.array_equal(oracle.matvec_gap(codes, row_off, mm, x), want)
