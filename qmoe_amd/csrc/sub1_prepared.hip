@@ -35,6 +35,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -648,6 +649,118 @@ __device__ __forceinline__ void write_row(uint16_t *dst, int ridx, float res, in
   dst[ridx] = out;
 }
 
+// ----------------------------------------------------- four tokens per walk --
+//
+// Where several tokens go through the same matrix, the stream is walked once
+// for four of them.  The activation array then holds, per physical column, the
+// two dwords (x0, x1) and (x2, x3) of tokens 0..3 as bf16 pairs (zeros in the
+// zero columns), and an entry costs one address, one 8-byte LDS read and four
+// v_dot2c_f32_bf16: the weight, picked by the position's low bit, sits in one
+// half of the second operand so that each instruction adds one token's term.
+// (Two 4-byte reads from separate arrays measured 10% slower in this kernel.)
+// Every token's sum is taken in the same order as when it is walked alone, so
+// the results are the same to the bit (for finite activations: a token's
+// infinity or NaN also spoils the sum of the token it shares a dword with).
+constexpr int kGroupTokens = 4;
+
+struct GroupSums {
+  float v[kGroupTokens];
+};
+
+__device__ __forceinline__ void stage_group(uint32_t *xa, const uint16_t *x, int64_t ldx,
+                                            int tokens_left, int width) {
+  const int npairs = (width + 1) / 2;
+  const int step = blockDim.x;
+  for (int z = threadIdx.x * kZeroPeriod; z < physical_columns(width); z += step * kZeroPeriod) {
+    xa[2 * z] = 0u;
+    xa[2 * z + 1] = 0u;
+  }
+  for (int m = threadIdx.x; m < npairs; m += step) {
+    uint32_t v[kGroupTokens];
+#pragma unroll
+    for (int t = 0; t < kGroupTokens; t++) {
+      v[t] = 0u;
+      if (t < tokens_left) {
+        const uint16_t *row = x + t * ldx;
+        if ((reinterpret_cast<uintptr_t>(row) & 3u) == 0 && 2 * m + 1 < width) {
+          v[t] = *reinterpret_cast<const uint32_t *>(row + 2 * m);
+        } else {
+          v[t] = row[2 * m];
+          if (2 * m + 1 < width) v[t] |= static_cast<uint32_t>(row[2 * m + 1]) << 16;
+        }
+      }
+    }
+    uint32_t *p = xa + 2 * physical_column(2 * m);
+    p[0] = (v[0] & 0xffffu) | (v[1] << 16);
+    p[1] = (v[2] & 0xffffu) | (v[3] << 16);
+    if (2 * m + 1 < width) {
+      p[2] = (v[0] >> 16) | (v[1] & 0xffff0000u);
+      p[3] = (v[2] >> 16) | (v[3] & 0xffff0000u);
+    }
+  }
+}
+
+// The nine entries of a chunk for four tokens.  `at` is the position's LDS byte
+// address as in add_chunk (the array starts on an 8-byte boundary): bit 2 is
+// the symbol, the rest the physical column's two dwords.
+__device__ __forceinline__ void add_chunk_group(uint2 cw, uint32_t &at, GroupSums &acc,
+                                                uint32_t w_min, uint32_t w_max) {
+  const uint32_t mid = __builtin_amdgcn_alignbit(cw.y, cw.x, 28);
+  uint32_t f[kFields];
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    asm("v_bfe_u32 %0, %1, %2, 7" : "=v"(f[q]) : "v"(cw.x), "n"(kFieldBits * q));
+    asm("v_bfe_u32 %0, %1, %2, 7" : "=v"(f[4 + q]) : "v"(mid), "n"(kFieldBits * q));
+  }
+  asm("v_bfe_u32 %0, %1, 24, 7" : "=v"(f[8]) : "v"(cw.y));
+#pragma unroll
+  for (int q = 0; q < kFields; q++) {
+    asm("v_lshl_add_u32 %0, %1, 2, %0" : "+v"(at) : "v"(f[q]));
+    const uint32_t is_max = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int>(at), 2, 1));
+    const uint32_t k_lo = (w_max & is_max) | (w_min & ~is_max);   // (w, 0): one v_bfi_b32
+    const uint32_t k_hi = k_lo << 16;                             // (0, w)
+    lds_word *col = (lds_word *)static_cast<uintptr_t>(at & ~7u);
+    const bf16x2 v01 = __builtin_bit_cast(bf16x2, col[0]);
+    const bf16x2 v23 = __builtin_bit_cast(bf16x2, col[1]);
+    acc.v[0] = __builtin_amdgcn_fdot2_f32_bf16(v01, __builtin_bit_cast(bf16x2, k_lo), acc.v[0], false);
+    acc.v[1] = __builtin_amdgcn_fdot2_f32_bf16(v01, __builtin_bit_cast(bf16x2, k_hi), acc.v[1], false);
+    acc.v[2] = __builtin_amdgcn_fdot2_f32_bf16(v23, __builtin_bit_cast(bf16x2, k_lo), acc.v[2], false);
+    acc.v[3] = __builtin_amdgcn_fdot2_f32_bf16(v23, __builtin_bit_cast(bf16x2, k_hi), acc.v[3], false);
+  }
+}
+
+// run_slice for four tokens: the same groups of 72 entries per token.
+__device__ __forceinline__ GroupSums run_slice_group(SliceWalk &w, const uint2 *stream,
+                                                     const uint32_t *xa, int pass, int passes) {
+  w.nch = __builtin_amdgcn_readfirstlane(w.nch);
+  const uint2 *p = chunk_pointer(stream, __builtin_amdgcn_readfirstlane(w.base));
+  const uint32_t w_min = w.minmax & 0xffffu, w_max = w.minmax >> 16;
+  GroupSums sum = {{0.f, 0.f, 0.f, 0.f}}, partial = {{0.f, 0.f, 0.f, 0.f}};
+  uint32_t at = lds_address(xa);
+  progress_priority(pass, passes);
+  for (int c = 0; c < w.nch; c += kRing) {
+#pragma unroll
+    for (int i = 0; i < kRing; i++) {
+      if (c + i < w.nch) {
+        const uint2 cw = w.ring[i];
+        w.ring[i] = p[min(c + i + kRing, w.nch - 1) * 64];
+        add_chunk_group(cw, at, partial, w_min, w_max);
+      }
+    }
+    if ((c + kRing) % kGroupChunks == 0) {
+      progress_priority(pass * w.nch + c + kRing, passes * w.nch);
+#pragma unroll
+      for (int t = 0; t < kGroupTokens; t++) {
+        sum.v[t] += partial.v[t];
+        partial.v[t] = 0.f;
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < kGroupTokens; t++) sum.v[t] += partial.v[t];   // the last, partial group
+  return sum;
+}
+
 // Small-batch form of a tile: `split` wavefronts share each slice, every one
 // taking a run of the slice's chunk groups (it starts from the position
 // checkpoint of its first group) and leaving one partial sum per group in LDS;
@@ -1077,6 +1190,47 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_small_kernel(Prepare
   }
 }
 
+// y[t] += W x[t] for many tokens through ONE matrix (matrix 0 of the prepared
+// set): a tile is (four tokens, part of the matrix), static order, persistent
+// grid; the stream of a tile's slices is walked once for its four tokens.
+__global__ __launch_bounds__(kMaxThreads) void matvec_group_kernel(PreparedArgs a) {
+  extern __shared__ __align__(16) uint32_t lds[];
+  uint32_t *xa = lds;
+  const KindArgs &k = a.k[0];
+  const int waves = blockDim.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int groups = (a.tokens + kGroupTokens - 1) / kGroupTokens;
+  const int n_all = groups * k.parts;
+  for (int tile = blockIdx.x; tile < n_all; tile += gridDim.x) {
+    const int g = tile / k.parts;
+    const int part = tile - g * k.parts;
+    const int s_lo = static_cast<int>(static_cast<int64_t>(k.slices) * part / k.parts);
+    const int s_hi = static_cast<int>(static_cast<int64_t>(k.slices) * (part + 1) / k.parts);
+    const int count = s_hi - s_lo;
+    const int passes = (count + waves - 1) / waves;
+    const int t0 = g * kGroupTokens;
+    const int left = min(a.tokens - t0, kGroupTokens);
+    int s = slice_of_pass(0, wave, waves, count);
+    SliceWalk cur;
+    if (s < count) cur = load_slice(a, k, s_lo + s);
+    __syncthreads();   // the previous tile has read its activations
+    stage_group(xa, a.x + static_cast<int64_t>(t0) * a.ldx, a.ldx, left, k.width);
+    __syncthreads();
+    for (int pass = 0; s < count; pass++) {
+      const int s_next = slice_of_pass(pass + 1, wave, waves, count);
+      SliceWalk nxt;
+      if (s_next < count) nxt = load_slice(a, k, s_lo + s_next);
+      const GroupSums res = run_slice_group(cur, a.stream, xa, pass, passes);
+#pragma unroll
+      for (int t = 0; t < kGroupTokens; t++)
+        if (t < left)
+          write_row(a.y + static_cast<int64_t>(t0 + t) * a.ldy, cur.ridx, res.v[t], kAccumulate);
+      if (s_next < count) cur = nxt;
+      s = s_next;
+    }
+  }
+}
+
 // ------------------------------------------------------------ host side --
 
 std::mutex g_mutex;
@@ -1455,6 +1609,41 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
       }
     }
   }
+  // Many tokens through one matrix: four tokens per walk of the stream, once
+  // such tiles (four tokens x 16 slices at least) can occupy half the compute
+  // units; below that the per-token kernels, which can cut a matrix finer, are
+  // faster (measured on the Switch shapes: 1.9x faster at 568 tokens, 2.3x at
+  // 2048, break-even between 50 and 400 tokens depending on the shape).
+  const int groups = (tokens + kGroupTokens - 1) / kGroupTokens;
+  const int group_parts = (a.k[0].slices + waves - 1) / waves;
+  bool by_groups = p.kinds == 1 && !token_matrix &&
+                   static_cast<int64_t>(groups) * group_parts * 2 >= cus;
+#ifdef SUB1_TUNE
+  if (const char *env = getenv("SUB1_GROUP_MIN"))
+    by_groups = p.kinds == 1 && !token_matrix && tokens >= atoi(env);
+#endif
+  if (by_groups) {
+    KindArgs &k = a.k[0];
+    const int max_parts = group_parts;
+    double best = 1e30;
+    for (int parts = 1; parts <= max_parts; parts++) {
+      const int per_tile = (k.slices + parts - 1) / parts;
+      const int64_t rounds = (static_cast<int64_t>(groups) * parts + cus - 1) / cus;
+      const double cost = rounds * ((per_tile + waves - 1) / waves + 0.25);
+      if (cost < best - 1e-9) {
+        best = cost;
+        k.parts = parts;
+      }
+    }
+    const int64_t tiles = static_cast<int64_t>(groups) * k.parts;
+    const void *fn = reinterpret_cast<const void *>(matvec_group_kernel);
+    HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(lds_base)));
+    matvec_group_kernel<<<static_cast<unsigned>(tiles < cus ? tiles : cus), 64 * waves, lds_base,
+                          s>>>(a);
+    HIP_TRY(hipGetLastError());
+    return SUB1_OK;
+  }
   size_t lds_partials = 0;
   double small_us = 0.0;
   if (idle_units)
@@ -1493,10 +1682,15 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     // wo's last pass: with at most half the wavefronts busy, the idle ones take
     // groups of those slices (partial sums go where x was)
     KindArgs &ko = a.k[1];
-    const int rest = ko.slices % waves;
-    if (rest > 0 && rest * 2 <= waves && ko.groups_max > 1) {
+    // Two workgroups of 8 wavefronts per compute unit, where two fit LDS and
+    // there are tokens for both: one's barriers between the phases of a token
+    // fall into the other's work (measured 3% faster than one of 16).
+    const int per_cu = 2 * lds_fused <= lds_limit && tokens >= 2 * cus ? 2 : 1;
+    const int fw = waves / per_cu;   // wavefronts per workgroup
+    const int rest = ko.slices % fw;
+    if (rest > 0 && rest * 2 <= fw && ko.groups_max > 1) {
       int split = 1;
-      while (split * 2 * rest <= waves && split * 2 <= ko.groups_max) split *= 2;
+      while (split * 2 * rest <= fw && split * 2 <= ko.groups_max) split *= 2;
       if (split > 1 &&
           static_cast<size_t>(rest) * ko.groups_max * 256 <= static_cast<size_t>(a.xdwords) * 4)
         ko.tail_split = split;
@@ -1505,8 +1699,8 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(lds_fused)));
     zero_words_kernel<<<1, 256, 0, s>>>(a.ctrl, kCtrlHeader);
-    const int grid = tokens < cus ? tokens : cus;
-    moe_prepared_fused_kernel<<<grid, 64 * waves, lds_fused, s>>>(a);
+    const int grid = tokens < cus * per_cu ? tokens : cus * per_cu;
+    moe_prepared_fused_kernel<<<grid, 64 * fw, lds_fused, s>>>(a);
     HIP_TRY(hipGetLastError());
     return SUB1_OK;
   }

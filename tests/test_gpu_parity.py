@@ -626,3 +626,34 @@ def test_prepared_stream_edge_rows(gpu, oracle):
     assert want[0] == 0 and want[70 - 1] == 0
     c = dict(t=t, mm=mm, codes=codes, row_off=row_off, x=x)
     check_product(oracle, c, want, prepared=True)
+
+
+@pytest.mark.parametrize('height,width,p0,tokens', [(3072, 768, 0.9, 171), (768, 3072, 0.9, 513),
+                                                    (77, 333, 0.7, 510), (130, 15, 0.9, 509),
+                                                    (6144, 2080, 0.9, 86), (5, 1, 0.5, 515),
+                                                    (200, 12288, 0.97, 511)])
+def test_prepared_matrix_many_tokens(gpu, oracle, height, width, p0, tokens):
+    """Enough tokens through one matrix that the launch walks the stream once
+    per four tokens (ragged last group; rows of x that start on odd 2-byte
+    boundaries when the width is odd): every token must come out as if it were
+    walked alone, i.e. equal to the oracle to the bit, accumulated onto what y
+    held."""
+    sub1, op = gpu
+    c = dev_case(oracle, height, width, p0, seed=7 * height + width + tokens)
+    pm = op.PreparedMatrix(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], width)
+    rng = np.random.default_rng(tokens)
+    xs = so.f32_to_bf16_bits(rng.standard_normal((tokens, width)).astype(np.float32))
+    pre = so.f32_to_bf16_bits(rng.standard_normal((tokens, height)).astype(np.float32))
+    y = bf16_dev(pre).clone()
+    pm.matvec_tokens(bf16_dev(xs), y)
+    got = bits_host(y)
+    for i in list(range(0, tokens, 23)) + list(range(tokens - 5, tokens)):
+        want = oracle.matvec_gap(c['codes'], c['row_off'], c['mm'], xs[i], y=pre[i])
+        assert np.array_equal(got[i], want), i
+    # all tokens, one launch each for a few and in small batches for the rest
+    # (the per-token kernels)
+    y1 = bf16_dev(pre).clone()
+    xd = bf16_dev(xs)
+    for lo in range(0, tokens, 16):
+        pm.matvec_tokens(xd[lo:lo + 16], y1[lo:lo + 16])
+    assert torch.equal(y1, y)
