@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 counter runs of this same
 # command (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a 1 GiB device copy reads on
 # those counters); the summaries are under profiles/.  None where no run was made.
-MEASURED_TRAFFIC = {'c2048-sweep': 4.948e9 + 0.034e9}
+MEASURED_TRAFFIC = {'c2048-sweep': 4.905e9 + 0.057e9}
 
 WORKLOADS = {
     # name: (shape key, experts, p_zero, description)
@@ -166,7 +166,8 @@ def single_matrix_protocol(seed, stream_ptr):
     from HIP events over back-to-back calls for the prepared layout, the
     packed layout (`sub1matvec`, the drop-in call) and the dense product, and
     the reference's wall-clock protocol (synchronise after every call) for the
-    drop-in call and the dense product."""
+    drop-in call and the dense product.  Plus 568 tokens through the same
+    matrix in one launch, against the dense GEMM."""
     import torch
     from qmoe_amd import sub1, sub1_hip, synthetic
 
@@ -208,6 +209,16 @@ def single_matrix_protocol(seed, stream_ptr):
             'sync_each_packed_us': round(sync_each_us(packed), 2),
             'sync_each_dense_us': round(sync_each_us(matmul), 2),
             'compressed_bytes': 2 * w_comp.numel(), 'dense_bytes': 2 * h * w}
+        # a sequence through the same layer (the encoder side): 568 tokens in one
+        # launch, the stream walked once per four tokens, against a dense bf16 GEMM
+        xt = torch.randn((568, w), generator=g, device='cuda').bfloat16()
+        yt = torch.zeros((568, h), dtype=torch.bfloat16, device='cuda')
+        ydt = torch.zeros((h, 568), dtype=torch.bfloat16, device='cuda')
+        xdt = xt.t().contiguous()
+        rows[name]['tokens568_prepared_us'] = round(
+            time_launches(lambda: pm.matvec_tokens(xt, yt), 100, 10, stream_ptr)[1], 2)
+        rows[name]['tokens568_dense_bf16_us'] = round(
+            time_launches(lambda: torch.matmul(dense, xdt, out=ydt), 100, 10, stream_ptr)[1], 2)
     return rows
 
 
