@@ -657,3 +657,45 @@ def test_prepared_matrix_many_tokens(gpu, oracle, height, width, p0, tokens):
     for lo in range(0, tokens, 16):
         pm.matvec_tokens(xd[lo:lo + 16], y1[lo:lo + 16])
     assert torch.equal(y1, y)
+
+
+def test_prepared_paths_on_random_shapes(gpu, oracle):
+    """Seeded random shapes, densities and token counts through the prepared
+    single-matrix path (which picks among the latency kernel, the streaming
+    kernel and four tokens per walk by shape and batch) and through a two-expert
+    layer: sampled tokens must equal the oracle to the bit, and the stream must
+    decode back to the symbols."""
+    sub1, op = gpu
+    from qmoe_amd import sub1_hip
+    rng = np.random.default_rng(20240611)
+    for trial in range(24):
+        height = int(rng.integers(1, 400))
+        width = int(rng.integers(1, 3000)) if trial % 3 else int(rng.integers(1, 40))
+        p0 = float(rng.choice([0.0, 0.3, 0.8, 0.9, 0.97, 0.999]))
+        tokens = int(rng.choice([1, 2, 3, 5, 17, 130, 600]))
+        c = dev_case(oracle, height, width, p0, seed=5000 + trial)
+        pm = op.PreparedMatrix(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], width)
+        assert np.array_equal(pm.decode().cpu().numpy(), c['t']), (trial, height, width)
+        xs = so.f32_to_bf16_bits(rng.standard_normal((tokens, width)).astype(np.float32))
+        pre = so.f32_to_bf16_bits(rng.standard_normal((tokens, height)).astype(np.float32))
+        y = bf16_dev(pre).clone()
+        pm.matvec_tokens(bf16_dev(xs), y)
+        got = bits_host(y)
+        for i in sorted(set([0, tokens // 2, tokens - 1])):
+            want = oracle.matvec_gap(c['codes'], c['row_off'], c['mm'], xs[i], y=pre[i])
+            assert np.array_equal(got[i], want), (trial, height, width, p0, tokens, i)
+    for trial in range(8):
+        d_model = int(rng.integers(1, 600))
+        d_ff = int(rng.integers(1, 900))
+        p0 = float(rng.choice([0.3, 0.9, 0.99]))
+        tokens = int(rng.choice([1, 4, 33, 300]))
+        stack, wi, wo = small_stack(oracle, 2, d_model, d_ff, p0, seed=6000 + trial)
+        prep = stack.prepare()
+        xs = so.f32_to_bf16_bits(rng.standard_normal((tokens, d_model)).astype(np.float32))
+        route = rng.integers(-1, 2, size=tokens).astype(np.int32)
+        y = prep.forward(bf16_dev(xs), torch.from_numpy(route).cuda())
+        got = bits_host(y)
+        for i in sorted(set([0, tokens // 2, tokens - 1])):
+            e = int(route[i])
+            want = xs[i] if e < 0 else oracle.expert_ffn(wi[e], wo[e], xs[i], order=2)[0]
+            assert np.array_equal(got[i], want), (trial, d_model, d_ff, p0, tokens, i)
