@@ -1581,7 +1581,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   // (the persistent kernel).  When even that leaves compute units idle (a
   // handful of tokens), the other kernel runs: a workgroup takes fewer slices
   // (8, 4, 2 or 1) and the wavefronts this frees share the slices, each
-  // starting from a column checkpoint.  plan_small picks the cut by estimate.
+  // starting from a position checkpoint.  plan_small picks the cut by estimate.
   const int want = (cus + tokens - 1) / tokens;   // tiles per token and projection
   int64_t first_slice = 0;
   bool idle_units = false;
@@ -1707,7 +1707,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   const size_t lds = lds_base + lds_partials;
   // Batches too small to occupy the GPU with a wavefront per slice go to the
   // latency kernel, everything else to the persistent one; either way at most
-  // a workgroup per compute unit (LDS holds the table once).
+  // a workgroup per compute unit (16 wavefronts of 72 to 80 registers each).
   const void *fn = small ? reinterpret_cast<const void *>(moe_prepared_small_kernel)
                          : reinterpret_cast<const void *>(moe_prepared_kernel);
   HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
