@@ -189,7 +189,12 @@ int sub1_moe_grouped(const sub1_moe_stack *stack, const int32_t *token_expert,
  * per group from zero, the partial sums added first group first; the same bits
  * for every batch size.  With few tokens several wavefronts share a row slice
  * (the buffer carries position checkpoints for that); the results do not
- * change.
+ * change.  A batch with several tokens per expert (at least four per expert
+ * and per compute unit on average) is grouped by expert on the GPU, and three
+ * or four tokens of an expert walk its streams together; the tables of that
+ * grouping live in the workspace; every token's result stays the same to the
+ * bit for finite activations (tokens that share a walk share dwords of the
+ * activation array: an infinity or NaN of one spoils its partner's sums).
  *
  * sub1_moe_prepared_decode writes the symbols (0, 1 = row min, 2 = row max) of
  * one matrix, read back from the stream, to tern_out (uint8 [rows, width] on
@@ -230,6 +235,8 @@ int sub1_moe_prepared_decode(const sub1_moe_prepared *prepared, int expert, int 
  * (count = 1: one Sub1Linear), then
  *     y[t, :] += W_m x[t, :],   m = token_matrix[t]  (NULL: matrix 0 for all),
  * the semantics of sub1_matvec_tokens, in one launch without a workspace.
+ * Without token_matrix and with enough tokens to occupy the GPU that way, the
+ * stream is walked once per four tokens (same results to the bit).
  * Tokens whose matrix index is negative or >= count are left alone.
  *
  *   meta_bytes = sub1_matrix_prepared_meta_bytes(count, height, width);

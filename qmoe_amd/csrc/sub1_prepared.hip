@@ -35,7 +35,6 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
-#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -414,6 +413,8 @@ struct PreparedArgs {
   const uint16_t *ckpt;       // position checkpoints, behind the stream
   KindArgs k[2];
   const int32_t *token_expert;   // NULL: every token uses matrix 0
+  const int32_t *order;          // fused kernel, tokens grouped by expert: token ids by expert,
+  const int2 *groups;            // and tiles (expert or -1, first index into order * 8 + tokens)
   const uint16_t *x;
   uint16_t *y;
   uint16_t *h;                   // kinds == 2 only
@@ -667,8 +668,11 @@ struct GroupSums {
   float v[kGroupTokens];
 };
 
-__device__ __forceinline__ void stage_group(uint32_t *xa, const uint16_t *x, int64_t ldx,
-                                            int tokens_left, int width) {
+struct GroupRows {
+  const uint16_t *row[kGroupTokens];   // NULL: no token in this place
+};
+
+__device__ __forceinline__ void stage_group(uint32_t *xa, const GroupRows &rows, int width) {
   const int npairs = (width + 1) / 2;
   const int step = blockDim.x;
   for (int z = threadIdx.x * kZeroPeriod; z < physical_columns(width); z += step * kZeroPeriod) {
@@ -680,8 +684,8 @@ __device__ __forceinline__ void stage_group(uint32_t *xa, const uint16_t *x, int
 #pragma unroll
     for (int t = 0; t < kGroupTokens; t++) {
       v[t] = 0u;
-      if (t < tokens_left) {
-        const uint16_t *row = x + t * ldx;
+      const uint16_t *row = rows.row[t];
+      if (row) {
         if ((reinterpret_cast<uintptr_t>(row) & 3u) == 0 && 2 * m + 1 < width) {
           v[t] = *reinterpret_cast<const uint32_t *>(row + 2 * m);
         } else {
@@ -729,16 +733,31 @@ __device__ __forceinline__ void add_chunk_group(uint2 cw, uint32_t &at, GroupSum
   }
 }
 
-// run_slice for four tokens: the same groups of 72 entries per token.
+// run_slice for four tokens: the same groups of 72 entries per token.  With
+// `part` the wavefront shares its slice and leaves each group's four partial
+// sums at part[group * 64 + lane].
 __device__ __forceinline__ GroupSums run_slice_group(SliceWalk &w, const uint2 *stream,
-                                                     const uint32_t *xa, int pass, int passes) {
+                                                     const uint32_t *xa, GroupSums *part,
+                                                     int pass, int passes) {
   w.nch = __builtin_amdgcn_readfirstlane(w.nch);
   const uint2 *p = chunk_pointer(stream, __builtin_amdgcn_readfirstlane(w.base));
+  const int lane = threadIdx.x & 63;
   const uint32_t w_min = w.minmax & 0xffffu, w_max = w.minmax >> 16;
   GroupSums sum = {{0.f, 0.f, 0.f, 0.f}}, partial = {{0.f, 0.f, 0.f, 0.f}};
-  uint32_t at = lds_address(xa);
-  progress_priority(pass, passes);
-  for (int c = 0; c < w.nch; c += kRing) {
+  uint32_t at = lds_address(xa) + 4u * static_cast<uint32_t>(w.j0);
+  int c = __builtin_amdgcn_readfirstlane(w.c0);
+  if (passes) progress_priority(pass, passes);
+  auto group_done = [&](int g) {
+    if (part) {
+      part[g * 64 + lane] = partial;
+    } else {
+#pragma unroll
+      for (int t = 0; t < kGroupTokens; t++) sum.v[t] += partial.v[t];
+    }
+#pragma unroll
+    for (int t = 0; t < kGroupTokens; t++) partial.v[t] = 0.f;
+  };
+  for (; c < w.nch; c += kRing) {
 #pragma unroll
     for (int i = 0; i < kRing; i++) {
       if (c + i < w.nch) {
@@ -748,16 +767,12 @@ __device__ __forceinline__ GroupSums run_slice_group(SliceWalk &w, const uint2 *
       }
     }
     if ((c + kRing) % kGroupChunks == 0) {
-      progress_priority(pass * w.nch + c + kRing, passes * w.nch);
-#pragma unroll
-      for (int t = 0; t < kGroupTokens; t++) {
-        sum.v[t] += partial.v[t];
-        partial.v[t] = 0.f;
-      }
+      if (passes) progress_priority(pass * w.nch + c + kRing, passes * w.nch);
+      group_done((c + kRing) / kGroupChunks - 1);
     }
   }
-#pragma unroll
-  for (int t = 0; t < kGroupTokens; t++) sum.v[t] += partial.v[t];   // the last, partial group
+  // the last, partial group, unless the loop has just closed it
+  if (c % kGroupChunks) group_done(c / kGroupChunks);
   return sum;
 }
 
@@ -1016,11 +1031,193 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
   }
 }
 
+// Tokens by expert, for the fused kernel when experts receive several tokens
+// each.  One workgroup: counts per expert (tokens that name no expert in a
+// bucket of their own), prefix sums, then every token takes a place among its
+// expert's tokens and, if its place starts one, writes a tile: four tokens of
+// an expert walk the stream together, three too; one or two left over go one
+// by one (a walk for four costs about as much as 2.3 single ones).
+//   tab: int32 [4, experts + 1]: counts, first place, first tile, next place
+// ctrl[3] receives the number of tiles, ctrl[2] the tokens whose expert id is
+// too large.  Which tokens share a walk depends on the order in which they
+// take their places (atomics) and may differ from run to run; each token's
+// result does not depend on it.
+__device__ __forceinline__ int32_t load_l2(const int32_t *p) {   // past the L1: atomics update L2 only
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__host__ __device__ constexpr int tiles_of(int n) {
+  return n / kGroupTokens + (n % kGroupTokens == 3 ? 1 : n % kGroupTokens);
+}
+
+__global__ __launch_bounds__(1024) void group_tokens_kernel(
+    const int32_t *__restrict__ token_expert, int tokens, int experts, int32_t *__restrict__ tab,
+    int32_t *__restrict__ order, int2 *__restrict__ groups, int32_t *__restrict__ ctrl) {
+  __shared__ int32_t seg_tokens[1024], seg_tiles[1024];
+  const int tid = threadIdx.x;
+  const int buckets = experts + 1;
+  int32_t *count = tab, *first = tab + buckets, *tile0 = tab + 2 * buckets,
+          *next = tab + 3 * buckets;
+  for (int b = tid; b < buckets; b += 1024) count[b] = 0;
+  __syncthreads();
+  int faults = 0;
+  for (int t = tid; t < tokens; t += 1024) {
+    const int e = token_expert[t];
+    if (e >= experts) faults++;
+    atomicAdd(&count[e < 0 || e >= experts ? experts : e], 1);
+  }
+  if (faults) atomicAdd(&ctrl[2], faults);
+  __syncthreads();
+  // prefix sums over the buckets: a run of buckets per thread, then the runs
+  const int seg = (buckets + 1023) / 1024;
+  const int lo = min(tid * seg, buckets), hi = min(lo + seg, buckets);
+  int32_t n_tok = 0, n_tile = 0;
+  for (int b = lo; b < hi; b++) {
+    const int n = load_l2(&count[b]);
+    n_tok += n;
+    n_tile += b == experts ? n : tiles_of(n);
+  }
+  seg_tokens[tid] = n_tok;
+  seg_tiles[tid] = n_tile;
+  __syncthreads();
+  for (int d = 1; d < 1024; d *= 2) {
+    const int32_t a0 = tid >= d ? seg_tokens[tid - d] : 0, a1 = tid >= d ? seg_tiles[tid - d] : 0;
+    __syncthreads();
+    seg_tokens[tid] += a0;
+    seg_tiles[tid] += a1;
+    __syncthreads();
+  }
+  int32_t run_tok = tid ? seg_tokens[tid - 1] : 0, run_tile = tid ? seg_tiles[tid - 1] : 0;
+  for (int b = lo; b < hi; b++) {
+    const int n = load_l2(&count[b]);
+    first[b] = run_tok;
+    next[b] = run_tok;
+    tile0[b] = run_tile;
+    run_tok += n;
+    run_tile += b == experts ? n : tiles_of(n);
+  }
+  if (tid == 1023) ctrl[3] = seg_tiles[1023];
+  __syncthreads();
+  for (int t = tid; t < tokens; t += 1024) {
+    const int e = token_expert[t];
+    const int b = e < 0 || e >= experts ? experts : e;
+    const int place = atomicAdd(&next[b], 1);
+    order[place] = t;
+    const int i = place - load_l2(&first[b]), n = load_l2(&count[b]);
+    const int t0 = load_l2(&tile0[b]);
+    const int whole = b == experts ? 0 : n / kGroupTokens * kGroupTokens;   // tokens in tiles of four
+    const int rest = n - whole;
+    if (i < whole) {
+      if (i % kGroupTokens == 0) groups[t0 + i / kGroupTokens] = make_int2(e, place * 8 + kGroupTokens);
+    } else if (b != experts && rest == 3) {
+      if (i == whole) groups[t0 + whole / kGroupTokens] = make_int2(e, place * 8 + 3);
+    } else {
+      groups[t0 + whole / kGroupTokens + (i - whole)] = make_int2(b == experts ? -1 : e, place * 8 + 1);
+    }
+  }
+}
+
+// A tile of the fused kernel with three or four tokens of one expert: the
+// same two phases, both walked once for all of them (see "four tokens per
+// walk").  order[place ..] are the tokens; h sits in LDS as (h0, h1), (h2, h3)
+// per physical column.  Ends before the loop's barrier.
+template <class FetchNext>
+__device__ __forceinline__ void fused_group_tile(const PreparedArgs &a, uint32_t *xa, uint32_t *ha,
+                                                 int e, int place, int n, FetchNext &&fetch_next) {
+  const KindArgs &ki = a.k[0];
+  const KindArgs &ko = a.k[1];
+  const int waves = blockDim.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  int tok[kGroupTokens];
+  GroupRows rows;
+#pragma unroll
+  for (int k = 0; k < kGroupTokens; k++) {
+    tok[k] = k < n ? __builtin_amdgcn_readfirstlane(a.order[place + k]) : -1;
+    rows.row[k] = k < n ? a.x + static_cast<int64_t>(tok[k]) * a.ldx : nullptr;
+  }
+  // wi: x -> relu(h) into LDS
+  const int64_t first_i = static_cast<int64_t>(e) * ki.slices;
+  int s = slice_of_pass(0, wave, waves, ki.slices);
+  SliceWalk cur;
+  if (s < ki.slices) cur = load_slice(a, ki, first_i + s);
+  stage_group(xa, rows, ki.width);
+  __syncthreads();
+  for (int pass = 0; s < ki.slices; pass++) {
+    const int s_next = slice_of_pass(pass + 1, wave, waves, ki.slices);
+    SliceWalk nxt;
+    if (s_next < ki.slices) nxt = load_slice(a, ki, first_i + s_next);
+    const GroupSums res = run_slice_group(cur, a.stream, xa, nullptr, pass,
+                                          (ki.slices + waves - 1) / waves);
+    if (cur.ridx != 0xffff) {
+      uint32_t out[kGroupTokens];
+#pragma unroll
+      for (int k = 0; k < kGroupTokens; k++) {
+        out[k] = f32_to_bf16(res.v[k]);
+        if (out[k] & 0x8000u) out[k] = 0;   // relu between the projections, on the bf16 value
+      }
+      uint32_t *p = ha + 2 * physical_column(cur.ridx);
+      p[0] = out[0] | (out[1] << 16);
+      p[1] = out[2] | (out[3] << 16);
+    }
+    if (s_next < ki.slices) cur = nxt;
+    s = s_next;
+  }
+  fetch_next();
+  // wo: h -> y, the short last pass shared out as for a single token
+  const int whole = ko.tail_split ? ko.slices - ko.slices % waves : ko.slices;
+  const int64_t first = static_cast<int64_t>(e) * ko.slices;
+  s = slice_of_pass(0, wave, waves, whole);
+  if (s < whole) cur = load_slice(a, ko, first + s);
+  __syncthreads();
+  auto write_rows = [&](int ridx, const GroupSums &res) {
+#pragma unroll
+    for (int k = 0; k < kGroupTokens; k++)
+      if (k < n) write_row(a.y + static_cast<int64_t>(tok[k]) * a.ldy, ridx, res.v[k], kStore);
+  };
+  for (int pass = 0; s < whole; pass++) {
+    const int s_next = slice_of_pass(pass + 1, wave, waves, whole);
+    SliceWalk nxt;
+    if (s_next < whole) nxt = load_slice(a, ko, first + s_next);
+    const GroupSums res = run_slice_group(cur, a.stream, ha, nullptr, pass, (whole + waves - 1) / waves);
+    write_rows(cur.ridx, res);
+    if (s_next < whole) cur = nxt;
+    s = s_next;
+  }
+  __builtin_amdgcn_s_setprio(0);
+  if (ko.tail_split) {
+    const int sl = whole + wave / ko.tail_split;
+    const int sub = wave % ko.tail_split;
+    GroupSums *mine = reinterpret_cast<GroupSums *>(xa) + (wave / ko.tail_split) * ko.groups_max * 64;
+    int groups = 0;
+    if (sl < ko.slices) {
+      groups = (__builtin_amdgcn_readfirstlane(ko.slice_nch[first + sl]) + kGroupChunks - 1) /
+               kGroupChunks;
+      const int g_lo = sub * groups / ko.tail_split, g_hi = (sub + 1) * groups / ko.tail_split;
+      if (g_lo < g_hi) {
+        SliceWalk tail = load_slice(a, ko, first + sl, g_lo, g_hi);
+        run_slice_group(tail, a.stream, ha, mine, 0, 0);
+      }
+    }
+    __syncthreads();
+    if (sub == 0 && sl < ko.slices) {
+      GroupSums sum = {{0.f, 0.f, 0.f, 0.f}};
+      for (int g = 0; g < groups; g++) {
+        const GroupSums v = mine[g * 64 + lane];
+#pragma unroll
+        for (int k = 0; k < kGroupTokens; k++) sum.v[k] += v.v[k];
+      }
+      write_rows(ko.row_idx[(first + sl) * 64 + lane], sum);
+    }
+  }
+}
+
 // Streaming form for batches of at least one token per compute unit: a tile is
 // a token, and the workgroup runs wi, ReLU and wo back to back with h kept in
 // LDS, already in the layout wo reads its activations from.  No workspace
 // traffic for h, no waiting between workgroups; tickets only balance the load.
 // LDS: x (wi's activations) | h (wo's activations).
+template <bool kGrouped>
 __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(PreparedArgs a) {
   extern __shared__ __align__(16) uint32_t lds[];
   __shared__ int s_ticket;
@@ -1034,6 +1231,8 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
   // h: the lanes overwrite the two value dwords of their rows; the zeros between
   // them stay for the whole launch
   for (int i = threadIdx.x; i < a.hdwords; i += threads) ha[i] = 0u;
+  // tokens grouped by expert: the tiles are in a.groups, ctrl[3] of them
+  const int n_tiles = kGrouped ? __builtin_amdgcn_readfirstlane(a.ctrl[3]) : a.tokens;
   int next_ticket = 0;
   auto fetch_next = [&]() {
     if (threadIdx.x == 0)
@@ -1045,17 +1244,30 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
     __syncthreads();   // the previous token's wo has read h; s_ticket is free
     if (threadIdx.x == 0) s_ticket = next_ticket;
     __syncthreads();
-    const int t = __builtin_amdgcn_readfirstlane(s_ticket);
-    if (t >= a.tokens) break;
-    int e = __builtin_amdgcn_readfirstlane(a.token_expert[t]);
-    if (e >= a.experts) {
-      if (threadIdx.x == 0)
-        __hip_atomic_fetch_add(&a.ctrl[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      e = -1;
+    const int tile = __builtin_amdgcn_readfirstlane(s_ticket);
+    if (tile >= n_tiles) break;
+    int t = tile, e, n = 1, place = 0;
+    if (kGrouped) {
+      const int2 rec = a.groups[tile];
+      e = __builtin_amdgcn_readfirstlane(rec.x);
+      place = __builtin_amdgcn_readfirstlane(rec.y >> 3);
+      n = __builtin_amdgcn_readfirstlane(rec.y & 7);
+      t = __builtin_amdgcn_readfirstlane(a.order[place]);
+    } else {
+      e = __builtin_amdgcn_readfirstlane(a.token_expert[t]);
+      if (e >= a.experts) {
+        if (threadIdx.x == 0)
+          __hip_atomic_fetch_add(&a.ctrl[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        e = -1;
+      }
     }
     if (e < 0) {
       pass_through(a, ko, t, 0, ko.slices);
       fetch_next();
+      continue;
+    }
+    if (kGrouped && n > 2) {
+      fused_group_tile(a, xa, ha, e, place, n, fetch_next);
       continue;
     }
     // wi: x -> relu(h) into LDS
@@ -1214,13 +1426,17 @@ __global__ __launch_bounds__(kMaxThreads) void matvec_group_kernel(PreparedArgs 
     SliceWalk cur;
     if (s < count) cur = load_slice(a, k, s_lo + s);
     __syncthreads();   // the previous tile has read its activations
-    stage_group(xa, a.x + static_cast<int64_t>(t0) * a.ldx, a.ldx, left, k.width);
+    GroupRows rows;
+#pragma unroll
+    for (int t = 0; t < kGroupTokens; t++)
+      rows.row[t] = t < left ? a.x + static_cast<int64_t>(t0 + t) * a.ldx : nullptr;
+    stage_group(xa, rows, k.width);
     __syncthreads();
     for (int pass = 0; s < count; pass++) {
       const int s_next = slice_of_pass(pass + 1, wave, waves, count);
       SliceWalk nxt;
       if (s_next < count) nxt = load_slice(a, k, s_lo + s_next);
-      const GroupSums res = run_slice_group(cur, a.stream, xa, pass, passes);
+      const GroupSums res = run_slice_group(cur, a.stream, xa, nullptr, pass, passes);
 #pragma unroll
       for (int t = 0; t < kGroupTokens; t++)
         if (t < left)
@@ -1563,6 +1779,8 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   a.ldy = ldy;
   a.ctrl = nullptr;
   a.h = nullptr;
+  a.order = nullptr;
+  a.groups = nullptr;
   if (p.kinds == 2) {
     a.ctrl = static_cast<int32_t *>(workspace);
     int64_t ctrl_bytes = (static_cast<int64_t>(kCtrlHeader + tokens) * 4 + 255) / 256 * 256;
@@ -1616,12 +1834,8 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   // 2048, break-even between 50 and 400 tokens depending on the shape).
   const int groups = (tokens + kGroupTokens - 1) / kGroupTokens;
   const int group_parts = (a.k[0].slices + waves - 1) / waves;
-  bool by_groups = p.kinds == 1 && !token_matrix &&
+  const bool by_groups = p.kinds == 1 && !token_matrix &&
                    static_cast<int64_t>(groups) * group_parts * 2 >= cus;
-#ifdef SUB1_TUNE
-  if (const char *env = getenv("SUB1_GROUP_MIN"))
-    by_groups = p.kinds == 1 && !token_matrix && tokens >= atoi(env);
-#endif
   if (by_groups) {
     KindArgs &k = a.k[0];
     const int max_parts = group_parts;
@@ -1679,28 +1893,54 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   if (fused) {
     a.xdwords = activation_dwords(a.k[0].width);
     a.hdwords = activation_dwords(a.k[1].width);
+    // Several tokens per expert: three or four tokens of one expert walk its
+    // streams together (measured on the Switch shapes: nothing to gain below
+    // four tokens per expert and four per compute unit, 1.1 to 1.3 times faster
+    // at 8 to 16 per expert, 1.7 to 1.95 at 32 to 64).  The tables of the
+    // grouping go where the other kernels keep h (this one keeps it in LDS).
+    const int64_t table_ints = 4 * (static_cast<int64_t>(p.count) + 1);
+    const int64_t order_ints = (tokens + 1) / 2 * 2;
+    const int64_t group_bytes = (table_ints + order_ints) * 4 + static_cast<int64_t>(tokens) * 8;
+    const bool grouped = tokens >= 4 * static_cast<int64_t>(p.count) && tokens >= 4 * cus &&
+                         group_bytes <= static_cast<int64_t>(tokens) * d_ff * 2;
     // wo's last pass: with at most half the wavefronts busy, the idle ones take
     // groups of those slices (partial sums go where x was)
     KindArgs &ko = a.k[1];
-    // Two workgroups of 8 wavefronts per compute unit, where two fit LDS and
-    // there are tokens for both: one's barriers between the phases of a token
-    // fall into the other's work (measured 3% faster than one of 16).
-    const int per_cu = 2 * lds_fused <= lds_limit && tokens >= 2 * cus ? 2 : 1;
+    // Two workgroups of 8 wavefronts per compute unit, where two fit LDS: one's
+    // barriers between the phases of a token fall into the other's work
+    // (measured 3% faster than one of 16 on 2048 tokens).
+    // Whole rounds count: 568 tokens are three rounds of workgroups of 16 but
+    // two (each twice as long) of workgroups of 8.
+    const int64_t rounds16 = (tokens + cus - 1) / cus, rounds8 = (tokens + 2 * cus - 1) / (2 * cus);
+    const int per_cu = 2 * lds_fused <= lds_limit && 1.94 * rounds8 < rounds16 ? 2 : 1;
     const int fw = waves / per_cu;   // wavefronts per workgroup
     const int rest = ko.slices % fw;
     if (rest > 0 && rest * 2 <= fw && ko.groups_max > 1) {
       int split = 1;
       while (split * 2 * rest <= fw && split * 2 <= ko.groups_max) split *= 2;
-      if (split > 1 &&
-          static_cast<size_t>(rest) * ko.groups_max * 256 <= static_cast<size_t>(a.xdwords) * 4)
-        ko.tail_split = split;
+      // a partial sum per group of chunks and lane, four with grouped tokens
+      const size_t partials = static_cast<size_t>(rest) * ko.groups_max * (grouped ? 1024 : 256);
+      if (split > 1 && partials <= static_cast<size_t>(a.xdwords) * 4) ko.tail_split = split;
     }
-    const void *fn = reinterpret_cast<const void *>(moe_prepared_fused_kernel);
+    const void *fn = grouped ? reinterpret_cast<const void *>(moe_prepared_fused_kernel<true>)
+                             : reinterpret_cast<const void *>(moe_prepared_fused_kernel<false>);
     HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(lds_fused)));
     zero_words_kernel<<<1, 256, 0, s>>>(a.ctrl, kCtrlHeader);
+    if (grouped) {
+      int32_t *tab = reinterpret_cast<int32_t *>(a.h);
+      int32_t *order = tab + table_ints;
+      int2 *groups = reinterpret_cast<int2 *>(order + order_ints);
+      group_tokens_kernel<<<1, 1024, 0, s>>>(token_matrix, tokens, p.count, tab, order, groups,
+                                              a.ctrl);
+      a.order = order;
+      a.groups = groups;
+    }
     const int grid = tokens < cus * per_cu ? tokens : cus * per_cu;
-    moe_prepared_fused_kernel<<<grid, 64 * fw, lds_fused, s>>>(a);
+    if (grouped)
+      moe_prepared_fused_kernel<true><<<grid, 64 * fw, lds_fused, s>>>(a);
+    else
+      moe_prepared_fused_kernel<false><<<grid, 64 * fw, lds_fused, s>>>(a);
     HIP_TRY(hipGetLastError());
     return SUB1_OK;
   }

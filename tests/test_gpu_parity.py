@@ -699,3 +699,36 @@ def test_prepared_paths_on_random_shapes(gpu, oracle):
             e = int(route[i])
             want = xs[i] if e < 0 else oracle.expert_ffn(wi[e], wo[e], xs[i], order=2)[0]
             assert np.array_equal(got[i], want), (trial, d_model, d_ff, p0, tokens, i)
+
+
+def test_tokens_of_an_expert_walk_together(gpu, oracle):
+    """A batch with many tokens per expert: the launch groups the tokens by
+    expert on the GPU and walks an expert's streams once for four (or three)
+    of them.  Every token must equal what it gives in a small batch, dropped
+    tokens pass through, expert ids that name no expert are counted, and
+    sampled tokens equal the oracle."""
+    from qmoe_amd import synthetic
+    experts, d_model, d_ff, tokens = 6, 200, 333, 1500
+    stack, wi, wo = small_stack(oracle, experts, d_model, d_ff, 0.8, seed=8100)
+    prep = stack.prepare()
+    rng = np.random.default_rng(81)
+    xs = so.f32_to_bf16_bits(rng.standard_normal((tokens, d_model)).astype(np.float32))
+    # counts per expert with every remainder modulo four; expert 5 gets nothing
+    route = np.concatenate([np.full(400, 0), np.full(401, 1), np.full(402, 2), np.full(283, 3),
+                            np.full(1, 4), np.full(8, -1), np.full(5, experts + 3)]).astype(np.int32)
+    assert route.shape[0] == tokens
+    rng.shuffle(route)
+    x = bf16_dev(xs)
+    te = torch.from_numpy(route).cuda()
+    y = prep.forward(x, te)
+    assert prep.launch_faults(tokens) == (0, 5)
+    for rep in range(2):
+        assert torch.equal(prep.forward(x, te), y)
+    small = torch.cat([prep.forward(x[lo:lo + 50].contiguous(), te[lo:lo + 50].contiguous())
+                       for lo in range(0, tokens, 50)])
+    assert torch.equal(y, small)
+    got = bits_host(y)
+    for i in range(0, tokens, 97):
+        e = int(route[i])
+        want = xs[i] if e < 0 or e >= experts else oracle.expert_ffn(wi[e], wo[e], xs[i], order=2)[0]
+        assert np.array_equal(got[i], want), (i, e)
