@@ -404,6 +404,15 @@ def main():
                      'GBps_cache_resident': round(ab / us_s / 1e3, 1)}
             if name == 'large128' and not args.no_dense:
                 entry['dense_bf16_gemv_us_per_layer'] = round(dense_gemv_us(st, xs, n_e) * n_e, 1)
+            if name == 'base128':
+                # a large batch: 4096 tokens routed uniformly (32 per expert on
+                # average), grouped by expert on the GPU, four tokens per walk
+                gb = torch.Generator().manual_seed(args.seed + 12)
+                xb = synthetic.activations(4096, dm, args.seed + 13)
+                rb = torch.randint(0, n_e, (4096,), generator=gb).to(torch.int32).cuda()
+                yb = torch.empty_like(xb)
+                _, us_b = time_launches(lambda: pr.forward(xb, rb, yb), 30, 5, stream_ptr)
+                entry['tokens4096_us_per_layer'] = round(us_b, 1)
             also[name] = entry
             del st, pr
     if not args.no_dense:
