@@ -812,15 +812,20 @@ __device__ __forceinline__ SplitWalk split_begin(const PreparedArgs &a, const Ki
   r.w.nch = 0;
   r.w.minmax = 0u;
   r.w.ridx = 0xffff;
+  // both words of the slice's description in one round trip (a slice that
+  // exists is read also where this wavefront has none)
+  const int64_t described = r.mine ? r.sl : static_cast<int64_t>(e) * k.slices + s0;
+  const int nch_word = k.slice_nch[described];
+  const uint32_t base_word = k.slice_base[described];
   if (r.mine) {
-    const int nch_all = __builtin_amdgcn_readfirstlane(k.slice_nch[r.sl]);
+    const int nch_all = __builtin_amdgcn_readfirstlane(nch_word);
     r.ngroups = (nch_all + kGroupChunks - 1) / kGroupChunks;
     r.g_lo = sub * r.ngroups / k.split;
     r.g_hi = (sub + 1) * r.ngroups / k.split;
     r.w.minmax = k.minmax[r.sl * 64 + lane];
     if (sub == 0) r.w.ridx = k.row_idx[r.sl * 64 + lane];   // it will write the slice's rows
     if (r.g_lo < r.g_hi) {
-      const uint32_t base = __builtin_amdgcn_readfirstlane(k.slice_base[r.sl]);
+      const uint32_t base = __builtin_amdgcn_readfirstlane(base_word);
       r.w.base = base;
       const uint2 *p = chunk_pointer(a.stream, base);
       const int c_lo = r.g_lo * kGroupChunks;
