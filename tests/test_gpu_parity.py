@@ -732,3 +732,39 @@ def test_tokens_of_an_expert_walk_together(gpu, oracle):
         e = int(route[i])
         want = xs[i] if e < 0 or e >= experts else oracle.expert_ffn(wi[e], wo[e], xs[i], order=2)[0]
         assert np.array_equal(got[i], want), (i, e)
+
+
+def test_full_size_c2048_layer_properties(gpu, oracle):
+    """The benchmark's own workload (2048 experts of 6144x2080 and 2080x6144,
+    one token each: 52 G weights) is too large for the oracle; what can be
+    checked at full size without it: the prepared stream holds every weight of
+    sampled experts (decoded back and compared with the packed codes decoded
+    by the other kernel), zero activations give zero, doubling the activations
+    doubles the output exactly (a power of two commutes with every rounding and
+    with ReLU), the sweep agrees with the packed-layout kernel to the stated
+    tolerance, and sampled tokens equal the oracle to the bit."""
+    sub1, op = gpu
+    from qmoe_amd import synthetic
+    experts = 2048
+    d_model, d_ff = synthetic.SHAPES['c2048']
+    stack = synthetic.build_stack(experts, d_model, d_ff, 0.9, seed=20231116)
+    prep = stack.prepare()
+    x = synthetic.activations(experts, d_model, seed=3)
+    route = torch.arange(experts, dtype=torch.int32, device='cuda')
+    y = prep.forward(x, route).clone()
+    assert prep.launch_faults(experts) == (0, 0)
+    assert torch.equal(prep.forward(torch.zeros_like(x), route), torch.zeros_like(x))
+    assert torch.equal(prep.forward(x * 2, route), y * 2)
+    assert close(y, stack.forward(x, route))
+    xs = bits_host(x)
+    got = bits_host(y)
+    for e in (0, 1023, 2047):
+        wi, wo = synthetic.expert_layers(stack, e)
+        for proj, layer, width in ((0, wi, d_model), (1, wo, d_ff)):
+            tern, _, bad = op.sub1decode(sub1.DEC[0], layer[0], layer[1], layer[2], width, want_w=False)
+            assert bad == 0
+            assert torch.equal(prep.decode(e, proj), tern), (e, proj)
+        host = [tuple(bits_host(t) if t.dtype != torch.int32 else t.cpu().numpy() for t in l)
+                for l in (wi, wo)]
+        want, _ = oracle.expert_ffn(host[0], host[1], xs[e], order=2)
+        assert np.array_equal(got[e], want), e
