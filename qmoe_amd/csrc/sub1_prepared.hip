@@ -889,14 +889,16 @@ __device__ __forceinline__ void await_activations(const PreparedArgs &a, const K
   if (kind == 1) {
     if (threadIdx.x == 0) {
       int spins = 0;
-      while (__hip_atomic_load(&a.ctrl[kCtrlHeader + t], __ATOMIC_ACQUIRE,
+      while (__hip_atomic_load(&a.ctrl[kCtrlHeader + t], __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT) < a.k[0].parts) {
         if (++spins > a.spin_limit) {
           __hip_atomic_fetch_add(&a.ctrl[1], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }
-        __builtin_amdgcn_s_sleep(8);
+        __builtin_amdgcn_s_sleep(2);
       }
+      // one acquire when the count is there, not one per look at it
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     }
     __syncthreads();
   }
