@@ -424,6 +424,7 @@ struct PreparedArgs {
   int tokens, experts;
   int xdwords;                   // LDS dwords reserved for the activations
   int hdwords;                   // fused kernel: LDS dwords of h (wo's activations)
+  int tail_room;                 // persistent kernel: partial sums (groups x 64 lanes) LDS has room for
   int spin_limit;
 };
 
@@ -1023,8 +1024,16 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
       uint16_t *dst = tile_output(a, k, kind, t, mode);
       // the first loads of the stream go out before the wait and the staging
       {
-        const int count = s_hi - s_lo;
-        const int passes = (count + waves - 1) / waves;
+        const int all = s_hi - s_lo;
+        // A short last pass (at most half the wavefronts busy) is shared out:
+        // `split` wavefronts per slice, each a run of its chunk groups, partial
+        // sums behind the activations in LDS (a.tail_room of them).
+        int split = 1;
+        const int rest = all % waves;
+        if (rest > 0 && rest * 2 <= waves && rest * k.groups_max <= a.tail_room)
+          while (split * 2 * rest <= waves && split * 2 <= k.groups_max) split *= 2;
+        const int count = split > 1 ? all - rest : all;
+        const int passes = (count + waves - 1) / waves + (split > 1);
         const int64_t first = static_cast<int64_t>(e) * k.slices + s_lo;
         int s = slice_of_pass(0, wave, waves, count);
         SliceWalk cur;
@@ -1038,6 +1047,29 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
           write_row(dst, cur.ridx, res, mode);
           if (s_next < count) cur = nxt;
           s = s_next;
+        }
+        if (split > 1) {
+          __builtin_amdgcn_s_setprio(0);
+          const int lane = threadIdx.x & 63;
+          const int sl = count + wave / split;
+          const int sub = wave % split;
+          float *mine = reinterpret_cast<float *>(xa + a.xdwords) + (wave / split) * k.groups_max * 64;
+          int groups = 0;
+          if (sl < all) {
+            groups = (__builtin_amdgcn_readfirstlane(k.slice_nch[first + sl]) + kGroupChunks - 1) /
+                     kGroupChunks;
+            const int g_lo = sub * groups / split, g_hi = (sub + 1) * groups / split;
+            if (g_lo < g_hi) {
+              SliceWalk tail = load_slice(a, k, first + sl, g_lo, g_hi);
+              run_slice(tail, a.stream, xa, mine);
+            }
+          }
+          __syncthreads();
+          if (sub == 0 && sl < all) {
+            float sum = 0.f;
+            for (int g = 0; g < groups; g++) sum += mine[g * 64 + lane];
+            write_row(dst, k.row_idx[(first + sl) * 64 + lane], sum, mode);
+          }
         }
       }
     }
@@ -1733,6 +1765,21 @@ size_t plan_small(PreparedArgs &a, int kinds, int tokens, int cus, int waves, si
   return partials;
 }
 
+// Passes a workgroup needs for a tile of `slices` slices (a pass = one slice per
+// wavefront); a last pass of at most half the wavefronts is shared out between
+// all of them by chunk groups and costs a fraction of one.
+double tile_passes(int slices, int waves, int groups_max) {
+  const int rest = slices % waves;
+  double passes = slices / waves;
+  if (rest > 0) {
+    int split = 1;
+    if (rest * 2 <= waves)
+      while (split * 2 * rest <= waves && split * 2 <= groups_max) split *= 2;
+    passes += split > 1 ? 1.0 / split + 0.1 : 1.0;
+  }
+  return passes;
+}
+
 // Launch of the prepared kernels.  kinds == 2: y = wo(relu(wi x)) per token,
 // workspace required; kinds == 1: y += W x per token, no workspace.
 int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *x, int64_t ldx,
@@ -1805,6 +1852,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   a.experts = p.count;
   a.xdwords = activation_dwords(wmax);
   a.hdwords = 0;
+  a.tail_room = 0;
   a.spin_limit = 1 << 24;
   const size_t lds_limit = 160 * 1024 - 64;
   const size_t lds_base = static_cast<size_t>(a.xdwords) * 4;
@@ -1829,13 +1877,14 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     if (want > max_parts) idle_units = true;
     // Parts per matrix for the streaming kernel: the count that needs the fewest
     // passes of a workgroup per compute unit (a pass = one slice per wavefront;
-    // 33 slices are 3 passes as one part but 1.5 rounds of 1 pass as three).
+    // a last pass of at most 8 slices is shared out between the wavefronts and
+    // costs a fraction of one).
     double best = 1e30;
     for (int parts = 1; parts <= max_parts; parts++) {
       const int per_tile = (k.slices + parts - 1) / parts;
       const int64_t rounds = (static_cast<int64_t>(tokens) * parts + cus - 1) / cus;
       // a quarter of a pass per tile for staging its activations
-      const double cost = rounds * ((per_tile + waves - 1) / waves + 0.25);
+      const double cost = rounds * (tile_passes(per_tile, waves, k.groups_max) + 0.25);
       if (cost < best - 1e-9) {
         best = cost;
         k.parts = parts;
@@ -1873,6 +1922,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     HIP_TRY(hipGetLastError());
     return SUB1_OK;
   }
+  const int stream_parts[2] = {a.k[0].parts, a.k[1].parts};   // plan_small may change them
   size_t lds_partials = 0;
   double small_us = 0.0;
   if (idle_units)
@@ -1881,23 +1931,41 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   int64_t tiles = 0;
   for (int i = 0; i < p.kinds; i++) tiles += static_cast<int64_t>(tokens) * a.k[i].parts;
   if (tiles > INT32_MAX - (1 << 20)) return fail(SUB1_ERR_SHAPE, "%s: too many tiles", who);
-  // At least a token per compute unit: a workgroup takes whole tokens and keeps
-  // h in LDS, if x + h fit.
+  // Whole tokens per workgroup with h in LDS (the fused kernel), or the matrices
+  // cut into tiles?  By estimate, in microseconds, from measurements on the
+  // Switch shapes.  One token on one compute unit takes about 8 us + entries /
+  // 23400 per us; the fused kernel takes that per round of workgroups (1.94
+  // times that with two workgroups of 8 wavefronts per compute unit).  The cut
+  // versions pay about 8 us per launch and, per round of tiles of a projection,
+  // 3 us for staging plus the tile's passes, a pass of 16 slices weighing in the
+  // token's time by its share of the chunks; where wavefronts share slices
+  // (plan_small) their own estimate + 13 us if that is less.
   const size_t lds_fused = (static_cast<size_t>(activation_dwords(a.k[0].width)) +
                             activation_dwords(a.k[1].width)) * 4;
-  bool fused = p.kinds == 2 && !small && a.k[0].parts == 1 && a.k[1].parts == 1 &&
-               lds_fused <= lds_limit;
-  if (!fused && p.kinds == 2 && lds_fused <= lds_limit && tokens < cus) {
-    // Fewer tokens than compute units: whole tokens per workgroup leave units
-    // idle but pay nothing for cutting the matrices (per-tile staging, h through
-    // memory, waiting).  The fused kernel then takes the time of one token,
-    // measured on the Switch shapes as about 8 us + entries / 23400 per us; the
-    // cut versions take the estimate above when wavefronts share slices and
-    // about 33 us + tokens / units x (time of one token) otherwise.
+  bool fused = false;
+  int fused_per_cu = 1;
+  if (p.kinds == 2 && lds_fused <= lds_limit) {
     const double token_us = 8.0 + static_cast<double>(p.total_chunks) * (64.0 * kFields) /
                                       p.count / 23400.0;
-    const double cut_us = small ? small_us + kLaunchUs : 33.0 + token_us * tokens / cus;
-    if (token_us < cut_us) {
+    const int64_t rounds16 = (tokens + cus - 1) / cus, rounds8 = (tokens + 2 * cus - 1) / (2 * cus);
+    double fused_us = rounds16 * token_us;
+    if (2 * lds_fused <= lds_limit && 1.94 * rounds8 < rounds16) {
+      fused_us = 1.94 * rounds8 * token_us;
+      fused_per_cu = 2;
+    }
+    double weight = 0.0;
+    for (int i = 0; i < 2; i++) weight += static_cast<double>(a.k[i].slices) * p.max_chunks[i];
+    double cut_us = 8.0;
+    for (int i = 0; i < 2; i++) {
+      const KindArgs &k = a.k[i];
+      const int per_tile = (k.slices + stream_parts[i] - 1) / stream_parts[i];
+      const int64_t rounds = (static_cast<int64_t>(tokens) * stream_parts[i] + cus - 1) / cus;
+      const double pass_us = (token_us - 8.0) * waves * p.max_chunks[i] / weight;
+      cut_us += rounds * (tile_passes(per_tile, waves, k.groups_max) * pass_us + 3.0);
+    }
+    cut_us *= 1.05;   // the estimate ran 5 to 8% low where tiles take several rounds
+    if (small) cut_us = std::min(cut_us, small_us + kLaunchUs);
+    if (fused_us < cut_us) {
       fused = true;
       for (int i = 0; i < 2; i++) {
         a.k[i].parts = 1;
@@ -1921,13 +1989,12 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     // wo's last pass: with at most half the wavefronts busy, the idle ones take
     // groups of those slices (partial sums go where x was)
     KindArgs &ko = a.k[1];
-    // Two workgroups of 8 wavefronts per compute unit, where two fit LDS: one's
+    // Two workgroups of 8 wavefronts per compute unit, where two fit LDS and it
+    // costs no round of workgroups more (568 tokens are three rounds of
+    // workgroups of 16 but two, each twice as long, of workgroups of 8): one's
     // barriers between the phases of a token fall into the other's work
     // (measured 3% faster than one of 16 on 2048 tokens).
-    // Whole rounds count: 568 tokens are three rounds of workgroups of 16 but
-    // two (each twice as long) of workgroups of 8.
-    const int64_t rounds16 = (tokens + cus - 1) / cus, rounds8 = (tokens + 2 * cus - 1) / (2 * cus);
-    const int per_cu = 2 * lds_fused <= lds_limit && 1.94 * rounds8 < rounds16 ? 2 : 1;
+    const int per_cu = fused_per_cu;
     const int fw = waves / per_cu;   // wavefronts per workgroup
     const int rest = ko.slices % fw;
     if (rest > 0 && rest * 2 <= fw && ko.groups_max > 1) {
@@ -1959,7 +2026,20 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     HIP_TRY(hipGetLastError());
     return SUB1_OK;
   }
-  const size_t lds = lds_base + lds_partials;
+  // the persistent kernel shares out a tile's short last pass: room for the
+  // partial sums of up to half the wavefronts' slices
+  size_t lds_tail = 0;
+  a.tail_room = 0;
+  if (!small) {
+    int groups_max = 0;
+    for (int i = 0; i < p.kinds; i++) groups_max = std::max(groups_max, a.k[i].groups_max);
+    lds_tail = static_cast<size_t>(waves / 2) * groups_max * 256;
+    if (lds_base + lds_tail <= lds_limit)
+      a.tail_room = (waves / 2) * groups_max;
+    else
+      lds_tail = 0;
+  }
+  const size_t lds = lds_base + lds_partials + lds_tail;
   // Batches too small to occupy the GPU with a wavefront per slice go to the
   // latency kernel, everything else to the persistent one; either way at most
   // a workgroup per compute unit (16 wavefronts of 72 to 80 registers each).
