@@ -350,7 +350,7 @@ def main():
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS,
                      'unit': 'GB/s', 'frac': round(achieved / HBM_PEAK_GBS, 4),
                      'traffic': MEASURED_TRAFFIC.get(args.workload) if not args.experts else None,
-                     'kernel': 'moe_prepared_fused_kernel',
+                     'kernel': 'moe_prepared_fused_kernel<false>',
                      'algorithmic_bytes': abytes, 'us_per_launch': round(us_launch, 2)},
     }
 
