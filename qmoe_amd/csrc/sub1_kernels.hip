@@ -380,15 +380,19 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
               a.wi_minmax[static_cast<int64_t>(e) * a.d_ff + row], s1, s2);
           uint16_t hb = f32_to_bf16(res);
           if (hb & 0x8000u) hb = 0;  // relu
-          a.h[static_cast<int64_t>(t) * a.d_ff + row] = hb;
+          // stored at agent scope: written through this die's L2, where the
+          // workgroups on other dies will read it
+          __hip_atomic_store(&a.h[static_cast<int64_t>(t) * a.d_ff + row], hb, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
         }
       }
-      // every wavefront's h stores reach L2, then the barrier, then thread 0's
-      // release writes L2 back for the other dies to see
+      // every wavefront waits for its h stores to be acknowledged, then the
+      // barrier, then thread 0 counts the tile (a release fence here would write
+      // back the whole L2)
       sub1::drain_stores();
       __syncthreads();
       if (threadIdx.x == 0)
-        __hip_atomic_fetch_add(&a.ctrl[kCtrlHeader + t], 1, __ATOMIC_RELEASE,
+        __hip_atomic_fetch_add(&a.ctrl[kCtrlHeader + t], 1, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
     } else {
       const int j = ticket - n_wi;
@@ -410,15 +414,16 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
       }
       if (threadIdx.x == 0) {
         int spins = 0;
-        while (__hip_atomic_load(&a.ctrl[kCtrlHeader + t], __ATOMIC_ACQUIRE,
+        while (__hip_atomic_load(&a.ctrl[kCtrlHeader + t], __ATOMIC_RELAXED,
                                  __HIP_MEMORY_SCOPE_AGENT) < a.wi_tiles) {
           if (++spins > a.spin_limit) {
             __hip_atomic_fetch_add(&a.ctrl[1], 1, __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
             break;
           }
-          __builtin_amdgcn_s_sleep(8);
+          __builtin_amdgcn_s_sleep(2);
         }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // once, when the count is there
       }
       __syncthreads();  // thread 0's acquire now covers the whole workgroup
       stage_activations<kThreads>(lds, a.h + static_cast<int64_t>(t) * a.d_ff, a.d_ff);
