@@ -163,8 +163,10 @@ class FasterMLP(nn.Module):
     module: `mlp.router` and `mlp.experts` (a ModuleDict of modules with
     `wi`/`wo` Sub1Linear layers).
 
-    Differences from the reference: the experts run in one launch (built from
-    the layers' buffers on first use, rebuilt if they are replaced or written);
+    Differences from the reference: the experts run in one launch, from a
+    stacked copy of the layers' buffers made on first use (remade after .to(),
+    load_state_dict or `refresh()`; the per-call check looks at four of the
+    experts' tensors only, so other writes to the buffers need `refresh()`);
     tokens stay on their GPU (one GPU here, the reference moves them to the
     layer's GPU and back, sub1.py:307-320)."""
 
@@ -176,11 +178,30 @@ class FasterMLP(nn.Module):
         self.experts = nn.ModuleList(mlp.experts.values())
         self.gpu = gpu
 
+    def _sentinels(self):
+        # a few of the experts' tensors stand for all of them in the per-call
+        # check (looking at every tensor of 2048 experts costs milliseconds)
+        first, last = self.experts[0], self.experts[len(self.experts) - 1]
+        return [first.wi.w_comp, first.wi.ter_minmax, last.wo.w_comp, last.wo.ter_minmax]
+
+    def refresh(self):
+        """Forget the stacked copy of the experts; the next forward rebuilds it.
+        Call it after writing to or replacing expert buffers (moving the module
+        with .to()/.cuda() and load_state_dict do it themselves)."""
+        self._launcher_cache = None
+
+    def _apply(self, fn, *args, **kwargs):
+        self._launcher_cache = None
+        return super()._apply(fn, *args, **kwargs)
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self._launcher_cache = None
+        return super()._load_from_state_dict(*args, **kwargs)
+
     def _launcher(self):
-        live = [t for e in self.experts for l in (e.wi, e.wo)
-                for t in (l.w_comp, l.row_off, l.ter_minmax)]
-        key = tuple((t.data_ptr(), t._version, t.numel()) for t in live)
         cached = getattr(self, '_launcher_cache', None)
+        live = self._sentinels()
+        key = tuple((t.data_ptr(), t._version, t.numel()) for t in live)
         if cached is None or cached[0] != key:
             stack = Sub1Experts([e.wi for e in self.experts], [e.wo for e in self.experts]).stack
             # the aliases keep the keyed addresses from being reused while cached
@@ -196,9 +217,9 @@ class FasterMLP(nn.Module):
         router_mask, router_probs, router_logits = _router_outputs(
             self.router(hidden_states), len(self.experts))
         expert_index = torch.argmax(router_mask, dim=-1)
-        routed = router_mask.sum(dim=-1) > 0
-        route = torch.where(routed, expert_index, torch.full_like(expert_index, -1))
+        # a token the capacity limit dropped has an all-zero mask row: expert -1
+        route = torch.where(router_mask.any(dim=-1), expert_index, -1).to(torch.int32)
         x = hidden_states.reshape(-1, hidden_states.shape[-1]).to(torch.bfloat16).contiguous()
-        next_states = self._launcher().forward(x, route.reshape(-1).to(torch.int32).contiguous())
+        next_states = self._launcher().forward(x, route.reshape(-1))
         hidden_states = router_probs * next_states.view(hidden_states.shape).to(hidden_states.dtype)
         return hidden_states, (router_logits, expert_index)

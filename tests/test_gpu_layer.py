@@ -121,7 +121,18 @@ def test_faster_mlp_equals_the_expert_loop(gpu, order):
     assert torch.equal(index, torch.argmax(mask, dim=-1))
     assert torch.equal(logits, outs[2])
     # a second call reuses the stacked experts
+    stacked = fast._launcher()
     assert torch.equal(fast(hidden)[0], want)
+    assert fast._launcher() is stacked
+    # writing to an expert in the middle is seen after refresh(); moving the module remakes the copy too
+    mid = layers['expert_2']
+    mid.wo.ter_minmax.mul_(2)
+    fast.refresh()
+    assert fast._launcher() is not stacked
+    assert torch.equal(fast(hidden)[0], expert_loop())
+    stacked = fast._launcher()
+    fast.cuda()
+    assert fast._launcher() is not stacked
 
 
 def test_checkpoint_directory_to_one_launch_layer(gpu, tmp_path):
