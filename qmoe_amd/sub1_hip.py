@@ -21,7 +21,27 @@ PREPARED_MAX_WIDTH = _lib.PREPARED_MAX_WIDTH
 
 
 def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    """torch's current stream on the current device, as the C ABI takes it."""
+    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice()))
+
+
+class _on_device:
+    """`with _on_device(dev):` makes dev the current device for the launch; a
+    device that already is costs two cheap calls instead of torch's guard."""
+
+    def __init__(self, device):
+        self.want = device.index if device.index is not None else torch._C._cuda_getDevice()
+        self.guard = None
+
+    def __enter__(self):
+        if torch._C._cuda_getDevice() != self.want:
+            self.guard = torch.cuda.device(self.want)
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
+        return False
 
 
 def _need(t, dtype, name, device=None, numel=None, dim=None):
@@ -64,7 +84,7 @@ def sub1matvec(dec, w_comp, row_off, ter_minmax, x, y):
         _need(x, torch.bfloat16, 'x', dev),
         _need(y, torch.bfloat16, 'y', dev),
     ]
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(_lib.load().sub1_matvec(*args, height, width, _stream()))
 
 
@@ -83,7 +103,7 @@ def sub1matvec_tokens(dec, w_comp, row_off, ter_minmax, x, y):
     height = row_off.numel() - 1
     if y.shape != (tokens, height) or ter_minmax.numel() != 2 * height:
         raise ValueError('y must be [%d, %d] and ter_minmax [%d]' % (tokens, height, 2 * height))
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(_lib.load().sub1_matvec_tokens(*args, height, width, tokens,
                                                   width, height, _stream()))
 
@@ -98,7 +118,7 @@ def sub1pack(trie, w_tern, row_off):
     height, width = w_tern.shape
     p_ro = _need(row_off, torch.int32, 'row_off', dev, numel=height + 1)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(lib.sub1_pack_count(p_trie, p_w, p_ro, height, width, _stream()))
         total = int(row_off[height].item())      # the one host sync, as in the reference
         w_comp = torch.empty(total, dtype=torch.int16, device=dev)
@@ -119,7 +139,7 @@ def sub1decode(dec, w_comp, row_off, ter_minmax, width, want_tern=True, want_w=T
     tern = torch.zeros((height, width), dtype=torch.uint8, device=dev) if want_tern else None
     w = torch.zeros((height, width), dtype=torch.bfloat16, device=dev) if want_w else None
     bad = torch.zeros(1, dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(_lib.load().sub1_decode(
             p_dec, p_wc, p_ro, p_mm, tern.data_ptr() if want_tern else None,
             w.data_ptr() if want_w else None, bad.data_ptr(), height, width, _stream()))
@@ -200,7 +220,7 @@ class ExpertStack:
             return y
         p_y = _need(y, torch.bfloat16, 'y', dev, numel=x.numel())
         ws = self.workspace(tokens)
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             _lib.check(_lib.load().sub1_moe_grouped(
                 ctypes.byref(self._c), p_te, p_x, p_y, tokens, ws.data_ptr(),
                 ws.numel(), _stream()))
@@ -242,7 +262,7 @@ class PreparedStack:
             raise ValueError('bad stack dimensions')
         self.meta = torch.empty(meta_bytes, dtype=torch.uint8, device=dev)
         self._c = _lib.MoePrepared()
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             _lib.check(lib.sub1_moe_prepare_layout(ctypes.byref(stack._c), self.meta.data_ptr(),
                                                    meta_bytes, ctypes.byref(self._c), _stream()))
             self.code_bytes = self._c.code_bytes
@@ -272,7 +292,7 @@ class PreparedStack:
             return y
         p_y = _need(y, torch.bfloat16, 'y', dev, numel=x.numel())
         ws = self.workspace(tokens)
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             _lib.check(_lib.load().sub1_moe_grouped_prepared(
                 ctypes.byref(self._c), p_te, p_x, p_y, tokens, ws.data_ptr(), ws.numel(),
                 _stream()))
@@ -287,7 +307,7 @@ class PreparedStack:
         1 = wo) read back from the prepared stream."""
         rows, width = (self.d_ff, self.d_model) if projection == 0 else (self.d_model, self.d_ff)
         out = torch.empty(rows, width, dtype=torch.uint8, device=self.device)
-        with torch.cuda.device(self.device):
+        with _on_device(self.device):
             _lib.check(_lib.load().sub1_moe_prepared_decode(
                 ctypes.byref(self._c), expert, projection, out.data_ptr(), _stream()))
         return out
@@ -327,7 +347,7 @@ class PreparedMatrix:
             raise ValueError('bad matrix dimensions')
         self.meta = torch.empty(meta_bytes, dtype=torch.uint8, device=dev)
         self._c = _lib.MatrixPrepared()
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             _lib.check(lib.sub1_matrix_prepare_layout(ctypes.byref(src), self.meta.data_ptr(),
                                                       meta_bytes, ctypes.byref(self._c), _stream()))
             self.codes = torch.empty(max(self._c.code_bytes, 256), dtype=torch.uint8, device=dev)
@@ -348,7 +368,7 @@ class PreparedMatrix:
                                                        dev, numel=tokens)
         if tokens == 0:
             return
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             _lib.check(_lib.load().sub1_matvec_prepared(
                 ctypes.byref(self._c), p_tm, p_x, self.width, p_y, self.height, tokens, _stream()))
 
@@ -356,7 +376,7 @@ class PreparedMatrix:
         """uint8 [height, width]: the symbols of one matrix read back from the
         prepared stream."""
         out = torch.empty(self.height, self.width, dtype=torch.uint8, device=self.device)
-        with torch.cuda.device(self.device):
+        with _on_device(self.device):
             _lib.check(_lib.load().sub1_matrix_prepared_decode(
                 ctypes.byref(self._c), matrix, out.data_ptr(), _stream()))
         return out
