@@ -128,8 +128,25 @@ class Sub1Experts(nn.Module):
             [(l.w_comp, l.row_off, l.ter_minmax) for l in wi_layers],
             [(l.w_comp, l.row_off, l.ter_minmax) for l in wo_layers])
 
+    # forward() goes through the prepared stream of the experts' non-zero
+    # weights, made on first use (about as much memory again as the stack); set
+    # to False to run from the packed buffers.  The stack is taken as fixed: after
+    # writing to its tensors call refresh().
+    fast = True
+
+    def refresh(self):
+        self._prepared = None
+
+    def _launcher(self):
+        if not (self.fast and self.stack.can_prepare()):
+            return self.stack
+        if getattr(self, '_prepared', None) is None:
+            self._prepared = self.stack.prepare()
+        return self._prepared
+
     def forward(self, x, expert_index):
-        return self.stack.forward(x.contiguous(), expert_index.to(torch.int32).contiguous())
+        return self._launcher().forward(x.contiguous(),
+                                        expert_index.to(torch.int32).contiguous())
 
 
 def _router_outputs(outputs, experts):
@@ -203,10 +220,9 @@ class FasterMLP(nn.Module):
         live = self._sentinels()
         key = tuple((t.data_ptr(), t._version, t.numel()) for t in live)
         if cached is None or cached[0] != key:
-            stack = Sub1Experts([e.wi for e in self.experts], [e.wo for e in self.experts]).stack
+            layer = Sub1Experts([e.wi for e in self.experts], [e.wo for e in self.experts])
             # the aliases keep the keyed addresses from being reused while cached
-            cached = (key, stack.prepare() if stack.can_prepare() else stack,
-                      [t.detach() for t in live])
+            cached = (key, layer._launcher(), [t.detach() for t in live])
             self._launcher_cache = cached
         return cached[1]
 
