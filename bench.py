@@ -127,6 +127,36 @@ def cpu_single_matrix_us(seed):
     return (time.perf_counter() - tick) / reps * 1e6
 
 
+def cpu_python_decode_matmul_us(seed):
+    """The reference's own host path for the first configuration
+    (test.py:103-115 and :180): the codes of a 3072 x 768 matrix expanded to
+    dense values in interpreted Python through the entry strings, then one
+    bf16 torch.matmul on the host.  Microseconds for the pair; nearly all of
+    it is the expansion."""
+    import torch
+    from oracle import sub1_oracle as so
+    o = so.COracle()
+    o.tables()
+    entries, _ = o.entries()
+    t, mm = so.synthetic_ternary(3072, 768, 0.9, seed)
+    codes, row_off = o.encode(t)
+    xv = torch.from_numpy(so.bf16_bits_to_f32(so.synthetic_activation(768, seed + 1))).to(torch.bfloat16)
+    levels = so.bf16_bits_to_f32(mm).reshape(-1, 2)
+    tick = time.perf_counter()
+    dense = []
+    for r in range(3072):
+        lo, hi = float(levels[r, 0]), float(levels[r, 1])
+        table = (0.0, lo, hi)
+        dense.extend(table[s] for s in so.expand_codes(codes[row_off[r]:row_off[r + 1]], entries, 768))
+    w = torch.tensor(dense, dtype=torch.float32).reshape(3072, 768).to(torch.bfloat16)
+    y = torch.matmul(w, xv)
+    spent = time.perf_counter() - tick
+    want = so.bf16_bits_to_f32(o.matvec_lanes(codes, row_off, mm, so.synthetic_activation(768, seed + 1)))
+    err = float((y.float() - torch.from_numpy(want)).norm() / torch.from_numpy(want).norm())
+    assert err < 1e-2, 'python decode + matmul differs from the C oracle by %g' % err
+    return spent * 1e6
+
+
 def dense_gemv_us(stack, x, experts):
     """Dense bf16 batched GEMV (torch.bmm -> hipBLASLt/rocBLAS) on the decoded
     weights of the first `experts` experts, microseconds per expert FFN."""
@@ -431,7 +461,8 @@ def main():
                       '%.1f s, extrapolated to the layer' % (done, experts, cores, cores, spent),
             'one_core_us_per_layer': round(spent1 / done1 * experts * 1e6, 1),
             'one_core_sample': '%d expert FFNs, %.1f s' % (done1, spent1),
-            'base_wi_3072x768_one_core_us': round(cpu_single_matrix_us(args.seed + 20), 1)}
+            'base_wi_3072x768_one_core_us': round(cpu_single_matrix_us(args.seed + 20), 1),
+            'base_wi_3072x768_python_decode_matmul_us': round(cpu_python_decode_matmul_us(args.seed + 20), 1)}
     print(json.dumps(out))
 
 
