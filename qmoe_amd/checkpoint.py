@@ -12,7 +12,9 @@ and reads it (sub1.py:169-214 `Sub1CheckpointManager`, sub1.py:217-292
 with expert names '<encoder|decoder>.block.<i>.layer.<1|2>.mlp.experts.expert_<j>'
 (reference switch.py:424-426).  The writer here takes packed layers directly
 (no HuggingFace model needed); the reader returns, per MoE layer, the experts'
-layers in index order, ready for `Sub1Experts` / `FasterMLP`.
+layers in index order, ready for `Sub1Experts` / `FasterMLP`, or, for models
+too large to hold twice, the layers already prepared with the packed form
+dropped (`load_prepared_experts`).
 
 Files are read with `torch.load(..., weights_only=True)`: tensors and plain
 containers only.
@@ -113,6 +115,67 @@ def load_expert_layers(path, device=None):
                 raise ValueError('%s: expert %d is missing or incomplete' % (layer_name, j))
             pairs.append((experts[j]['wi'], experts[j]['wo']))
         out[layer_name] = pairs
+    return out
+
+
+def load_prepared_experts(path, device):
+    """{layer name: Sub1Experts} on `device`, each holding only the prepared
+    stream of its experts' weights.  For checkpoints whose packed form and
+    prepared form do not fit the GPU side by side: the files are read one at a
+    time, a layer is stacked, prepared and its packed tensors dropped as soon
+    as its last expert has arrived, so the GPU holds the prepared layers plus
+    the experts of layers still incomplete.  Expert counts come from sizes.pt
+    (reference sub1.py:250); a layer with experts missing raises at the end."""
+    sizes = torch.load(os.path.join(path, 'sizes.pt'), weights_only=True)
+    want = {}
+    for key in sizes:
+        name, tag = key.rsplit('.', 1)
+        m = _EXPERT.match(name)
+        if not m or tag not in ('wi', 'wo'):
+            raise ValueError('unexpected entry in sizes.pt: %r' % key)
+        want.setdefault(m.group('layer'), set()).add(int(m.group('index')))
+    for layer_name, have in want.items():
+        if have != set(range(len(have))):
+            raise ValueError('%s: expert indices in sizes.pt are not 0..%d'
+                             % (layer_name, len(have) - 1))
+    pending, out = {}, {}
+    for filename in sorted(os.listdir(path)):
+        if filename in _FILES_SKIPPED or filename == 'noexp.pt' or not filename.endswith('.pt'):
+            continue
+        tensors = torch.load(os.path.join(path, filename), weights_only=True)
+        for key in [k for k in tensors if k.endswith('.w_comp')]:
+            stem = key[:-len('.w_comp')]
+            name, tag = stem.rsplit('.', 1)
+            m = _EXPERT.match(name)
+            if not m or tag not in ('wi', 'wo') or stem not in sizes:
+                raise ValueError('%s holds %r, which sizes.pt does not list' % (filename, key))
+            try:
+                w_comp, row_off = tensors[key], tensors[stem + '.row_off']
+                ter_minmax = tensors[stem + '.ter_minmax']
+            except KeyError as err:
+                raise ValueError('checkpoint lacks %s' % err.args[0])
+            if w_comp.numel() != sizes[stem] or int(row_off[-1]) != sizes[stem]:
+                raise ValueError('%s: %d codewords stored, sizes.pt says %d, row_off ends at %d'
+                                 % (stem, w_comp.numel(), sizes[stem], int(row_off[-1])))
+            layer = sub1.Sub1Linear(row_off.numel() - 1, w_comp.numel())
+            layer.w_comp.data = w_comp.to(torch.int16)
+            layer.row_off.data = row_off.to(torch.int32)
+            layer.ter_minmax.data = ter_minmax.to(torch.bfloat16)
+            pending.setdefault(m.group('layer'), {}).setdefault(int(m.group('index')), {})[tag] = \
+                layer.to(device)
+        del tensors
+        for layer_name in list(pending):
+            experts = pending[layer_name]
+            if len(experts) == len(want[layer_name]) and \
+                    all(set(e) == {'wi', 'wo'} for e in experts.values()):
+                stacked = sub1.Sub1Experts([experts[j]['wi'] for j in range(len(experts))],
+                                           [experts[j]['wo'] for j in range(len(experts))])
+                stacked.release_packed()
+                out[layer_name] = stacked
+                del pending[layer_name]
+    if pending or set(out) != set(want):
+        missing = sorted(set(want) - set(out))
+        raise ValueError('incomplete layers in %s: %s' % (path, ', '.join(missing)))
     return out
 
 

@@ -135,9 +135,26 @@ class Sub1Experts(nn.Module):
     fast = True
 
     def refresh(self):
+        if self.stack is None:
+            raise RuntimeError('the packed stack was released; build the layer again')
         self._prepared = None
 
+    def release_packed(self):
+        """Keep only the prepared stream: makes it if need be and frees the
+        stacked copy of the packed buffers (the larger half of the layer's
+        memory; the per-expert tensors the layer was built from are the
+        caller's to drop).  What is lost is the way back: no refresh(), no run
+        from the packed buffers.  A c-2048 model's 30 layers are ~135 GB packed
+        and ~150 GB prepared: one 288 GB GPU holds one of the two."""
+        if not self.stack.can_prepare():
+            raise RuntimeError('these shapes have no prepared form; the packed stack stays')
+        self.fast = True
+        self._launcher()
+        self.stack = None
+
     def _launcher(self):
+        if self.stack is None:
+            return self._prepared
         if not (self.fast and self.stack.can_prepare()):
             return self.stack
         if getattr(self, '_prepared', None) is None:
@@ -205,18 +222,44 @@ class FasterMLP(nn.Module):
         """Forget the stacked copy of the experts; the next forward rebuilds it.
         Call it after writing to or replacing expert buffers (moving the module
         with .to()/.cuda() and load_state_dict do it themselves)."""
+        self._forget()
+
+    def release_packed(self):
+        """Keep only the prepared stream of this layer's experts: builds it if
+        need be, then empties the experts' `w_comp`, `row_off` and `ter_minmax`
+        buffers, which frees about half of the layer's memory.  From then on
+        the layer can run and nothing else: saving it stores empty buffers, and
+        moving, loading or refresh() raise."""
+        launcher = self._launcher()
+        if not isinstance(launcher, sub1_hip.PreparedStack):
+            raise RuntimeError('these shapes have no prepared form; the packed buffers stay')
+        self._released = True
+        self._launcher_cache = (None, launcher, [])     # no aliases of expert tensors
+        for expert in self.experts:
+            for layer in (expert.wi, expert.wo):
+                for name in ('w_comp', 'row_off', 'ter_minmax'):
+                    old = getattr(layer, name)
+                    setattr(layer, name, torch.zeros(0, dtype=old.dtype, device=old.device))
+                layer._prepared_cache = None
+
+    def _forget(self):
+        if getattr(self, '_released', False):
+            raise RuntimeError('the packed buffers of this layer were released; '
+                               'it cannot be moved, reloaded or refreshed')
         self._launcher_cache = None
 
     def _apply(self, fn, *args, **kwargs):
-        self._launcher_cache = None
+        self._forget()
         return super()._apply(fn, *args, **kwargs)
 
     def _load_from_state_dict(self, *args, **kwargs):
-        self._launcher_cache = None
+        self._forget()
         return super()._load_from_state_dict(*args, **kwargs)
 
     def _launcher(self):
         cached = getattr(self, '_launcher_cache', None)
+        if getattr(self, '_released', False):
+            return cached[1]
         live = self._sentinels()
         key = tuple((t.data_ptr(), t._version, t.numel()) for t in live)
         if cached is None or cached[0] != key:

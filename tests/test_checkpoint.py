@@ -96,6 +96,23 @@ def test_reader_rejects_damage(written):
         checkpoint.load_expert_layers(path)          # expert 1 of 0..2 missing
 
 
+def test_prepared_only_reader_checks_the_directory_first(written):
+    """The streaming reader reads sizes.pt before any expert file: entries
+    that are not experts' wi / wo, and expert indices with holes, raise before
+    anything is put on a GPU (none is needed to get that far)."""
+    path, _ = written
+    sizes = torch.load(os.path.join(path, 'sizes.pt'), weights_only=True)
+    bad = {k: v for k, v in sizes.items() if not k.startswith(expert_name('decoder', 3, 1))}
+    torch.save(bad, os.path.join(path, 'sizes.pt'))
+    with pytest.raises(ValueError, match='indices'):
+        checkpoint.load_prepared_experts(path, 'cpu')
+    bad = dict(sizes)
+    bad['encoder.block.1.layer.1.mlp.router.classifier'] = 3
+    torch.save(bad, os.path.join(path, 'sizes.pt'))
+    with pytest.raises(ValueError, match='unexpected'):
+        checkpoint.load_prepared_experts(path, 'cpu')
+
+
 def test_writer_rejects_other_names(tmp_path, oracle):
     mgr = checkpoint.Sub1CheckpointManager(str(tmp_path))
     layer = packed_layer(oracle, 8, 8, 1)

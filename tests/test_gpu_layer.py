@@ -2,6 +2,7 @@
 the sparse-MLP module (router, one-launch experts, probability scaling) against
 the reference's per-expert loop (sub1.py:306-321) restated with per-layer
 calls."""
+import os
 import types
 
 import pytest
@@ -159,6 +160,75 @@ def test_checkpoint_directory_to_one_launch_layer(gpu, tmp_path):
         e = int(route[t])
         want = x[t:t + 1] if e < 0 else made[e](x[t:t + 1])
         assert torch.equal(y[t:t + 1], want), t
+
+
+def test_checkpoint_directory_to_prepared_only_layers(gpu, tmp_path):
+    """The loader for models too large to hold twice: two layers whose experts
+    are spread over three files, out of order, come back as prepared-only
+    layers that give the bits of the stacked layers and hold no packed copy."""
+    from qmoe_amd import checkpoint, sub1, sub1_hip
+    d_model, d_ff, experts = 128, 320, 4
+    g = torch.Generator(device='cuda').manual_seed(53)
+    mgr = checkpoint.Sub1CheckpointManager(str(tmp_path), config={'d_model': d_model})
+    names = [('encoder.block.1.layer.1.mlp', j) for j in (3, 0, 2, 1)] + \
+            [('decoder.block.1.layer.2.mlp', j) for j in (1, 0, 3, 2)]
+    for n, (layer_name, j) in enumerate(names):
+        wi = sub1.Sub1Linear.make(ternary_dense(d_ff, d_model, 0.8, g))
+        wo = sub1.Sub1Linear.make(ternary_dense(d_model, d_ff, 0.8, g))
+        mgr.add_expert('%s.experts.expert_%d' % (layer_name, j), wi, wo)
+        if n in (2, 5):                      # files end in the middle of a layer
+            mgr.save_experts()
+    mgr.finalize()
+    assert sorted(f for f in os.listdir(str(tmp_path)) if f.startswith('exp')) == \
+        ['exp00.pt', 'exp01.pt', 'exp02.pt']
+    stacks = checkpoint.load_expert_stacks(str(tmp_path), 'cuda:0')
+    lean = checkpoint.load_prepared_experts(str(tmp_path), 'cuda:0')
+    assert set(lean) == set(stacks) and len(lean) == 2
+    x = torch.randn((9, d_model), generator=g, device='cuda').bfloat16()
+    route = torch.tensor([0, 3, 1, 2, 2, -1, 0, 3, 1], dtype=torch.int32, device='cuda')
+    for name, layer in lean.items():
+        assert layer.stack is None and isinstance(layer._launcher(), sub1_hip.PreparedStack)
+        assert torch.equal(layer(x, route), stacks[name](x, route)), name
+        with pytest.raises(RuntimeError):
+            layer.refresh()
+    # a layer with an expert missing from the files
+    os.remove(os.path.join(str(tmp_path), 'exp01.pt'))
+    with pytest.raises(ValueError):
+        checkpoint.load_prepared_experts(str(tmp_path), 'cuda:0')
+
+
+def test_faster_mlp_release_packed(gpu):
+    """release_packed() frees the experts' packed buffers (the memory in use
+    drops by their size), the layer keeps giving the same bits, and what can
+    no longer work raises."""
+    sub1 = gpu
+    d_model, d_ff, n = 256, 640, 16
+    g = torch.Generator(device='cuda').manual_seed(57)
+    experts = nn.ModuleDict()
+    for j in range(n):
+        experts['expert_%d' % j] = Expert(
+            sub1.Sub1Linear.make(ternary_dense(d_ff, d_model, 0.85, g)),
+            sub1.Sub1Linear.make(ternary_dense(d_model, d_ff, 0.85, g)))
+    mlp = types.SimpleNamespace(router=Top1Router(d_model, n, 3, 'probs_first').cuda(),
+                                experts=experts)
+    fast = sub1.FasterMLP(mlp)
+    hidden = torch.randn((2, 24, d_model), generator=g, device='cuda').bfloat16()
+    want = fast(hidden)[0].clone()
+    packed = sum(t.numel() * t.element_size() for e in fast.experts for l in (e.wi, e.wo)
+                 for t in (l.w_comp, l.row_off, l.ter_minmax))
+    del experts, mlp
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    fast.release_packed()
+    torch.cuda.synchronize()
+    freed = before - torch.cuda.memory_allocated()
+    assert freed >= 0.9 * packed, (freed, packed)
+    assert all(e.wi.w_comp.numel() == 0 and e.wo.ter_minmax.numel() == 0 for e in fast.experts)
+    assert torch.equal(fast(hidden)[0], want)
+    assert torch.equal(fast(hidden)[0], want)
+    for broken in (fast.refresh, fast.cuda, lambda: fast.load_state_dict(fast.state_dict())):
+        with pytest.raises(RuntimeError):
+            broken()
 
 
 def test_layer_launch_replays_from_a_graph(gpu):
