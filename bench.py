@@ -56,13 +56,25 @@ def rel_diff(a, b):
     return float('%.3g' % (torch.linalg.norm(a - b) / torch.linalg.norm(b)).item())
 
 
-def time_launches(fn, steps, warmup, stream_ptr):
+PREHEAT_S = 0.1
+
+
+def time_launches(fn, steps, warmup, stream_ptr, preheat_s=PREHEAT_S):
     """(wall seconds for `steps` calls, average microseconds per call from HIP
-    events recorded on the launch stream)."""
+    events recorded on the launch stream).  Before the `warmup` untimed calls
+    the same call is repeated, untimed, for `preheat_s` seconds: from idle the
+    GPU takes about 40 ms of load to reach its clocks (the c-2048 sweep reads
+    1250 us in its first ten launches, 1000 us from the fortieth on), and a
+    short warm-up would time that ramp instead of the kernel."""
     import ctypes
     import torch
     from qmoe_amd import _lib
     lib = _lib.load()
+    tick = time.perf_counter()
+    while time.perf_counter() - tick < preheat_s:
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -255,8 +267,8 @@ def single_matrix_protocol(seed, stream_ptr):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=20)
-    ap.add_argument('--warmup', type=int, default=3)
+    ap.add_argument('--steps', type=int, default=100)
+    ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--workload', default='c2048-sweep', choices=sorted(WORKLOADS))
     ap.add_argument('--experts', type=int, default=0, help='override the expert count (debugging)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline')
@@ -367,6 +379,7 @@ def main():
         'value': round(ms_per_step * 1e3, 2),
         'unit': 'us/layer',
         'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'preheat_s': PREHEAT_S,       # untimed repeats of the step before the warm-up: clock ramp
         'ms_per_step': round(ms_per_step, 4),
         'higher_is_better': False, 'scaling': 'weak', 'vs_baseline': None,
         'dtype': 'bf16 in/out, fp32 accumulate, u16 codes transcoded to 7-bit gap entries',
