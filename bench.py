@@ -393,7 +393,10 @@ def main():
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS,
                      'unit': 'GB/s', 'frac': round(achieved / HBM_PEAK_GBS, 4),
                      'traffic': MEASURED_TRAFFIC.get(args.workload) if not args.experts else None,
-                     'kernel': 'moe_prepared_fused_kernel<false>',
+                     # the library picks the kernel: a token per workgroup from one token
+                     # per compute unit on, several workgroups per token below half of that
+                     'kernel': ('moe_prepared_fused_kernel<false>' if experts >= 256
+                                else 'moe_prepared_shared_kernel'),
                      'algorithmic_bytes': abytes, 'us_per_launch': round(us_launch, 2)},
     }
 

@@ -25,13 +25,16 @@
 // row's (min, max) pair, which adds x * min or x * max onto the row's fp32 sum;
 // no cross-lane traffic at all.  They compute what reference
 // sub1_cuda_kernel.cu:163-201 computes per row.
-// Three kernels share that loop and give the same bits:
+// Four kernels share that loop and give the same bits:
 // moe_prepared_fused_kernel streams whole tokens (wi, ReLU, wo in one
 // workgroup, h kept in LDS) when there is at least a token per compute unit;
+// moe_prepared_shared_kernel lets several workgroups share a token, each in
+// both projections, when there are fewer tokens than half the compute units;
 // moe_prepared_kernel streams tiles of one matrix (persistent grid, a wavefront
-// per slice, the next slice's loads in flight) for smaller batches and for
-// single matrices; moe_prepared_small_kernel is the latency form for a handful
-// of tokens (wavefronts share a slice from position checkpoints).
+// per slice, the next slice's loads in flight) for the batches in between and
+// for single matrices; moe_prepared_small_kernel is the latency form for a
+// handful of tokens through single matrices (wavefronts share a slice from
+// position checkpoints).
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -966,6 +969,65 @@ __device__ __forceinline__ void publish_h(const PreparedArgs &a, int t) {
                            __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// The wavefronts of a workgroup walk `all` slices of one matrix: slice `first`
+// of the stream's slices and every `stride`-th after it.  `before()` runs once
+// the first loads of the stream are out (it stages the activations `act` and
+// ends with a barrier); `out(row, sum)` takes every row's result.  A short last
+// pass (at most half the wavefronts busy) is shared out: `split` wavefronts per
+// slice, each a run of its chunk groups, partial sums in `partials`
+// (a.tail_room groups of 64 lanes).
+template <class Before, class Out>
+__device__ __forceinline__ void walk_tile(const PreparedArgs &a, const KindArgs &k, int64_t first,
+                                          int stride, int all, const uint32_t *act,
+                                          float *partials, Before &&before, Out &&out) {
+  const int waves = blockDim.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  int split = 1;
+  const int rest = all % waves;
+  if (rest > 0 && rest * 2 <= waves && rest * k.groups_max <= a.tail_room)
+    while (split * 2 * rest <= waves && split * 2 <= k.groups_max) split *= 2;
+  const int count = split > 1 ? all - rest : all;
+  const int passes = (count + waves - 1) / waves + (split > 1);
+  int s = slice_of_pass(0, wave, waves, count);
+  SliceWalk cur;
+  // the first loads of the stream go out before the wait and the staging
+  if (s < count) cur = load_slice(a, k, first + static_cast<int64_t>(s) * stride);
+  before();
+  for (int pass = 0; s < count; pass++) {
+    const int s_next = slice_of_pass(pass + 1, wave, waves, count);
+    SliceWalk nxt;
+    if (s_next < count) nxt = load_slice(a, k, first + static_cast<int64_t>(s_next) * stride);
+    const float res = run_slice(cur, a.stream, act, nullptr, pass, passes);
+    out(cur.ridx, res);
+    if (s_next < count) cur = nxt;
+    s = s_next;
+  }
+  if (split > 1) {
+    __builtin_amdgcn_s_setprio(0);
+    const int lane = threadIdx.x & 63;
+    const int sl = count + wave / split;
+    const int sub = wave % split;
+    const int64_t slice = first + static_cast<int64_t>(sl) * stride;
+    float *mine = partials + (wave / split) * k.groups_max * 64;
+    int groups = 0;
+    if (sl < all) {
+      groups = (__builtin_amdgcn_readfirstlane(k.slice_nch[slice]) + kGroupChunks - 1) /
+               kGroupChunks;
+      const int g_lo = sub * groups / split, g_hi = (sub + 1) * groups / split;
+      if (g_lo < g_hi) {
+        SliceWalk tail = load_slice(a, k, slice, g_lo, g_hi);
+        run_slice(tail, a.stream, act, mine);
+      }
+    }
+    __syncthreads();
+    if (sub == 0 && sl < all) {
+      float sum = 0.f;
+      for (int g = 0; g < groups; g++) sum += mine[g * 64 + lane];
+      out(k.row_idx[slice * 64 + lane], sum);
+    }
+  }
+}
+
 // Persistent grid.  A tile is (token, projection, part): the slices of one
 // matrix, or of one of `parts` equal ranges of them when there are too few
 // tokens to occupy the GPU otherwise; a workgroup stages the token's
@@ -981,11 +1043,8 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
   extern __shared__ __align__(16) uint32_t lds[];
   __shared__ int s_ticket;
   uint32_t *xa = lds;
-  const int threads = blockDim.x;
-  const int waves = threads >> 6;
   const int n_wi = a.tokens * a.k[0].parts;
   const int n_all = n_wi + (a.kinds == 2 ? a.tokens * a.k[1].parts : 0);
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const bool dynamic = a.ctrl != nullptr;
   // dynamic order: thread 0 asks for the next ticket when its own part of the
   // tile is done, so that the atomic's round trip overlaps the tile's tail (any
@@ -1022,56 +1081,10 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
     if (e >= 0) {
       int mode;
       uint16_t *dst = tile_output(a, k, kind, t, mode);
-      // the first loads of the stream go out before the wait and the staging
-      {
-        const int all = s_hi - s_lo;
-        // A short last pass (at most half the wavefronts busy) is shared out:
-        // `split` wavefronts per slice, each a run of its chunk groups, partial
-        // sums behind the activations in LDS (a.tail_room of them).
-        int split = 1;
-        const int rest = all % waves;
-        if (rest > 0 && rest * 2 <= waves && rest * k.groups_max <= a.tail_room)
-          while (split * 2 * rest <= waves && split * 2 <= k.groups_max) split *= 2;
-        const int count = split > 1 ? all - rest : all;
-        const int passes = (count + waves - 1) / waves + (split > 1);
-        const int64_t first = static_cast<int64_t>(e) * k.slices + s_lo;
-        int s = slice_of_pass(0, wave, waves, count);
-        SliceWalk cur;
-        if (s < count) cur = load_slice(a, k, first + s);
-        await_activations(a, k, kind, t, xa);
-        for (int pass = 0; s < count; pass++) {
-          const int s_next = slice_of_pass(pass + 1, wave, waves, count);
-          SliceWalk nxt;
-          if (s_next < count) nxt = load_slice(a, k, first + s_next);
-          const float res = run_slice(cur, a.stream, xa, nullptr, pass, passes);
-          write_row(dst, cur.ridx, res, mode);
-          if (s_next < count) cur = nxt;
-          s = s_next;
-        }
-        if (split > 1) {
-          __builtin_amdgcn_s_setprio(0);
-          const int lane = threadIdx.x & 63;
-          const int sl = count + wave / split;
-          const int sub = wave % split;
-          float *mine = reinterpret_cast<float *>(xa + a.xdwords) + (wave / split) * k.groups_max * 64;
-          int groups = 0;
-          if (sl < all) {
-            groups = (__builtin_amdgcn_readfirstlane(k.slice_nch[first + sl]) + kGroupChunks - 1) /
-                     kGroupChunks;
-            const int g_lo = sub * groups / split, g_hi = (sub + 1) * groups / split;
-            if (g_lo < g_hi) {
-              SliceWalk tail = load_slice(a, k, first + sl, g_lo, g_hi);
-              run_slice(tail, a.stream, xa, mine);
-            }
-          }
-          __syncthreads();
-          if (sub == 0 && sl < all) {
-            float sum = 0.f;
-            for (int g = 0; g < groups; g++) sum += mine[g * 64 + lane];
-            write_row(dst, k.row_idx[(first + sl) * 64 + lane], sum, mode);
-          }
-        }
-      }
+      walk_tile(a, k, static_cast<int64_t>(e) * k.slices + s_lo, 1, s_hi - s_lo, xa,
+                reinterpret_cast<float *>(xa + a.xdwords),
+                [&]() { await_activations(a, k, kind, t, xa); },
+                [&](int ridx, float res) { write_row(dst, ridx, res, mode); });
     }
     fetch_next();
     if (a.kinds == 2 && kind == 0) publish_h(a, t);
@@ -1387,6 +1400,49 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
       }
     }
   }
+}
+
+// Between the latency form and a token per workgroup: with fewer tokens than
+// half the compute units, `parts` workgroups share a token.  Each takes every
+// parts-th slice of wi (the slices are ordered longest first, so the shares are
+// even), writes its rows of relu(h) to the workspace, counts itself done, waits
+// for the others of its token, stages the whole of h and takes every parts-th
+// slice of wo.  Unlike tiles of one projection handed out by ticket, every
+// workgroup works in both phases, the token's activations are staged once per
+// phase and workgroup, and h crosses memory once.
+// The workgroups of a token wait for each other: the grid (tokens x parts) must
+// fit the GPU at once, which the launch makes sure of (at most one workgroup
+// per compute unit); the wait is bounded like the other kernels'.
+__global__ __launch_bounds__(kMaxThreads) void moe_prepared_shared_kernel(PreparedArgs a) {
+  extern __shared__ __align__(16) uint32_t lds[];
+  uint32_t *xa = lds;
+  float *partials = reinterpret_cast<float *>(xa + a.xdwords);
+  const KindArgs &ki = a.k[0];
+  const KindArgs &ko = a.k[1];
+  const int parts = ki.parts;
+  const int t = blockIdx.x / parts;
+  const int part = blockIdx.x - t * parts;
+  int e = __builtin_amdgcn_readfirstlane(a.token_expert[t]);
+  if (e >= a.experts) {
+    if (part == 0 && threadIdx.x == 0)
+      __hip_atomic_fetch_add(&a.ctrl[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    e = -1;
+  }
+  if (e < 0) {
+    if (part == 0) pass_through(a, ko, t, 0, ko.slices);
+    return;
+  }
+  uint16_t *h = a.h + static_cast<int64_t>(t) * ki.height;
+  walk_tile(a, ki, static_cast<int64_t>(e) * ki.slices + part, parts,
+            (ki.slices - part + parts - 1) / parts, xa, partials,
+            [&]() { await_activations(a, ki, 0, t, xa); },
+            [&](int ridx, float res) { write_row(h, ridx, res, kStoreRelu); });
+  publish_h(a, t);
+  uint16_t *y = a.y + static_cast<int64_t>(t) * a.ldy;
+  walk_tile(a, ko, static_cast<int64_t>(e) * ko.slices + part, parts,
+            (ko.slices - part + parts - 1) / parts, xa, partials,
+            [&]() { await_activations(a, ko, 1, t, xa); },
+            [&](int ridx, float res) { write_row(y, ridx, res, kStore); });
 }
 
 // For the batches too small to occupy the GPU with a wavefront per slice: built
@@ -1780,6 +1836,23 @@ double tile_passes(int slices, int waves, int groups_max) {
   return passes;
 }
 
+// The time, in units of a full pass (16 wavefronts, a slice each), that a
+// workgroup of `waves` wavefronts needs for `slices` slices: whole passes, then
+// the rest either as a pass of its own or, if it is at most half the
+// wavefronts, shared out `split` ways.  A pass with few wavefronts in it is
+// faster than a full one (less contention for LDS), down to about 0.3 of it.
+double part_passes(int slices, int waves, int groups_max) {
+  const int rest = slices % waves;
+  double passes = slices / waves;
+  if (rest > 0) {
+    int split = 1;
+    if (rest * 2 <= waves)
+      while (split * 2 * rest <= waves && split * 2 <= groups_max) split *= 2;
+    passes += std::max(static_cast<double>(rest * split) / waves, 0.3) / split;
+  }
+  return passes;
+}
+
 // Launch of the prepared kernels.  kinds == 2: y = wo(relu(wi x)) per token,
 // workspace required; kinds == 1: y += W x per token, no workspace.
 int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *x, int64_t ldx,
@@ -1944,6 +2017,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
                             activation_dwords(a.k[1].width)) * 4;
   bool fused = false;
   int fused_per_cu = 1;
+  int shared_parts = 0;
   if (p.kinds == 2 && lds_fused <= lds_limit) {
     const double token_us = 8.0 + static_cast<double>(p.total_chunks) * (64.0 * kFields) /
                                       p.count / 23400.0;
@@ -1965,13 +2039,56 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     }
     cut_us *= 1.05;   // the estimate ran 5 to 8% low where tiles take several rounds
     if (small) cut_us = std::min(cut_us, small_us + kLaunchUs);
-    if (fused_us < cut_us) {
+    // Up to half a token per compute unit: several workgroups per token, each
+    // in both projections (moe_prepared_shared_kernel).  All of them must be on
+    // the GPU at once, one per compute unit.  Fixed costs of 8 us plus staging
+    // (by the widths), the walk of the largest share, and what more workgroups
+    // cost in dispatch and in waiting for each other; measured on the Switch
+    // shapes it is the fastest form from 2 tokens (1 for the smaller shapes) to
+    // half the compute units: 1.1 to 1.5 times faster than cutting by projection.
+    const size_t lds_shared = lds_base + static_cast<size_t>(waves / 2) *
+                                             std::max(a.k[0].groups_max, a.k[1].groups_max) * 256;
+    if (2 * static_cast<int64_t>(tokens) <= cus && lds_shared <= lds_limit) {
+      double best_us = 1e30;
+      int best_parts = 0;
+      for (int parts = 2; parts <= 64 && static_cast<int64_t>(tokens) * parts <= cus; parts++) {
+        double us = 8.0 + (a.k[0].width + a.k[1].width) / 2700.0 + 0.03 * parts +
+                    0.008 * tokens * parts;
+        for (int i = 0; i < 2; i++) {
+          const KindArgs &k = a.k[i];
+          const double pass_us = (token_us - 8.0) * waves * p.max_chunks[i] / weight;
+          us += part_passes((k.slices + parts - 1) / parts, waves, k.groups_max) * pass_us + 0.5;
+        }
+        if (us < best_us) {
+          best_us = us;
+          best_parts = parts;
+        }
+      }
+      if (best_parts && best_us < cut_us && best_us < fused_us) shared_parts = best_parts;
+    }
+    if (!shared_parts && fused_us < cut_us) {
       fused = true;
       for (int i = 0; i < 2; i++) {
         a.k[i].parts = 1;
         a.k[i].split = 1;
       }
     }
+  }
+  if (shared_parts) {
+    for (int i = 0; i < 2; i++) {
+      a.k[i].parts = shared_parts;
+      a.k[i].split = 1;
+    }
+    a.tail_room = (waves / 2) * std::max(a.k[0].groups_max, a.k[1].groups_max);
+    const size_t lds_shared = lds_base + static_cast<size_t>(a.tail_room) * 256;
+    const void *fn = reinterpret_cast<const void *>(moe_prepared_shared_kernel);
+    HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(lds_shared)));
+    const int nctrl = kCtrlHeader + tokens;
+    zero_words_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl);
+    moe_prepared_shared_kernel<<<tokens * shared_parts, 64 * waves, lds_shared, s>>>(a);
+    HIP_TRY(hipGetLastError());
+    return SUB1_OK;
   }
   if (fused) {
     a.xdwords = activation_dwords(a.k[0].width);

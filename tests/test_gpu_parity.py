@@ -466,6 +466,44 @@ def test_token_per_workgroup_tiles_with_dropped_tokens(gpu, oracle):
     assert close(y, stack.forward(x, route))
 
 
+@pytest.mark.parametrize('d_model,d_ff,p0', [(2080, 6144, 0.9), (200, 330, 0.8), (64, 4096, 0.9)])
+def test_tokens_shared_between_workgroups(gpu, oracle, d_model, d_ff, p0):
+    """Fewer tokens than half the compute units: several workgroups share a
+    token, each taking every n-th slice of both projections, the intermediate
+    activations crossing memory once.  Shapes with fewer slices than
+    workgroups per token (some get nothing to walk) and rows that do not fill
+    the last slice; dropped tokens pass through, out-of-range expert ids are
+    counted; every token equals its single-token launch to the bit and the
+    oracle's sum in the stream's order."""
+    from qmoe_amd import synthetic
+    experts = 4
+    stack = synthetic.build_stack(experts, d_model, d_ff, p0, seed=31)
+    prep = stack.prepare()
+    for tokens in (2, 3, 7, 30, 100, 128):
+        x = synthetic.activations(tokens, d_model, seed=32 + tokens)
+        route = (torch.arange(tokens, dtype=torch.int32, device='cuda') * 3) % experts
+        bad = 0
+        if tokens >= 7:
+            route[1] = -1
+            route[5] = experts + 2
+            bad = 1
+        y = prep.forward(x, route)
+        assert prep.launch_faults(tokens) == (0, bad)
+        for t in range(tokens):
+            if int(route[t]) < 0 or int(route[t]) >= experts:
+                assert torch.equal(y[t], x[t]), (tokens, t)
+        for t in sorted({0, min(2, tokens - 1), tokens // 2, tokens - 1}):
+            one = prep.forward(x[t:t + 1].contiguous(), route[t:t + 1].contiguous())
+            assert torch.equal(one[0], y[t]), (tokens, t)
+        assert close(y, stack.forward(x, route))
+    t = 2
+    wi, wo = synthetic.expert_layers(stack, int(route[t]))
+    host = [tuple(bits_host(v) if v.dtype != torch.int32 else v.cpu().numpy() for v in l)
+            for l in (wi, wo)]
+    ref, _ = oracle.expert_ffn(host[0], host[1], bits_host(x[t]), order=2)
+    assert np.array_equal(bits_host(y[t]), ref)
+
+
 @pytest.mark.parametrize('d_model,d_ff', [(64, 12288), (12288, 64), (2, 2)])
 def test_extreme_widths_in_every_batch_regime(gpu, oracle, d_model, d_ff):
     """The widest activations the fast layout takes and the narrowest, from one
