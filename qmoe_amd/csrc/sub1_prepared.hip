@@ -1410,9 +1410,13 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
 // slice of wo.  Unlike tiles of one projection handed out by ticket, every
 // workgroup works in both phases, the token's activations are staged once per
 // phase and workgroup, and h crosses memory once.
-// The workgroups of a token wait for each other: the grid (tokens x parts) must
-// fit the GPU at once, which the launch makes sure of (at most one workgroup
-// per compute unit); the wait is bounded like the other kernels'.
+// The workgroups of a token wait for each other.  The launch keeps the grid
+// (tokens x parts) within one workgroup per compute unit, so that all of them
+// run at once.  Where they cannot (other work on the GPU), the waits still end:
+// the workgroups of a token have consecutive indices and workgroups start in
+// index order, so at most one token of a launch is ever partly on the GPU; all
+// others run to completion and make room.  The wait is bounded like the other
+// kernels' in any case.
 __global__ __launch_bounds__(kMaxThreads) void moe_prepared_shared_kernel(PreparedArgs a) {
   extern __shared__ __align__(16) uint32_t lds[];
   uint32_t *xa = lds;
