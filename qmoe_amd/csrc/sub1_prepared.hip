@@ -2043,26 +2043,32 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     }
     cut_us *= 1.05;   // the estimate ran 5 to 8% low where tiles take several rounds
     if (small) cut_us = std::min(cut_us, small_us + kLaunchUs);
-    // Up to half a token per compute unit: several workgroups per token, each
-    // in both projections (moe_prepared_shared_kernel).  All of them must be on
-    // the GPU at once, one per compute unit.  Fixed costs of 8 us plus staging
-    // (by the widths), the walk of the largest share, and what more workgroups
-    // cost in dispatch and in waiting for each other; measured on the Switch
-    // shapes it is the fastest form from 2 tokens (1 for the smaller shapes) to
-    // half the compute units: 1.1 to 1.5 times faster than cutting by projection.
+    // Up to a token per compute unit: several workgroups per token, each in
+    // both projections (moe_prepared_shared_kernel), one workgroup per compute
+    // unit at a time.  Up to half a token per unit that is all of them at once;
+    // up to one, two rounds can still beat whole tokens on half the units (they
+    // do for the c-2048 shapes at 129 to 170 tokens).  Fixed costs of 8 us plus
+    // staging (by the widths), the walk of the largest share, and what more
+    // workgroups cost in dispatch and in waiting for each other; measured on
+    // the Switch shapes it is the fastest form from 2 tokens (1 for the smaller
+    // shapes) to half the compute units: 1.1 to 1.5 times faster than cutting
+    // by projection.
     const size_t lds_shared = lds_base + static_cast<size_t>(waves / 2) *
                                              std::max(a.k[0].groups_max, a.k[1].groups_max) * 256;
-    if (2 * static_cast<int64_t>(tokens) <= cus && lds_shared <= lds_limit) {
+    if (tokens <= cus && lds_shared <= lds_limit) {
       double best_us = 1e30;
       int best_parts = 0;
-      for (int parts = 2; parts <= 64 && static_cast<int64_t>(tokens) * parts <= cus; parts++) {
-        double us = 8.0 + (a.k[0].width + a.k[1].width) / 2700.0 + 0.03 * parts +
-                    0.008 * tokens * parts;
+      for (int parts = 2; parts <= 64 && static_cast<int64_t>(tokens) * parts <= 2 * cus; parts++) {
+        // beyond one workgroup per compute unit the rest of the grid starts as
+        // the first tokens finish: two rounds, measured 7% above twice one
+        const int rounds = static_cast<int64_t>(tokens) * parts > cus ? 2 : 1;
+        double task = (a.k[0].width + a.k[1].width) / 2700.0 + 0.03 * parts;
         for (int i = 0; i < 2; i++) {
           const KindArgs &k = a.k[i];
           const double pass_us = (token_us - 8.0) * waves * p.max_chunks[i] / weight;
-          us += part_passes((k.slices + parts - 1) / parts, waves, k.groups_max) * pass_us + 0.5;
+          task += part_passes((k.slices + parts - 1) / parts, waves, k.groups_max) * pass_us + 0.5;
         }
+        const double us = 8.0 + (rounds == 2 ? 2.24 : 1.0) * task + 0.008 * tokens * parts;
         if (us < best_us) {
           best_us = us;
           best_parts = parts;

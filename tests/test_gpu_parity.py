@@ -468,7 +468,8 @@ def test_token_per_workgroup_tiles_with_dropped_tokens(gpu, oracle):
 
 @pytest.mark.parametrize('d_model,d_ff,p0', [(2080, 6144, 0.9), (200, 330, 0.8), (64, 4096, 0.9)])
 def test_tokens_shared_between_workgroups(gpu, oracle, d_model, d_ff, p0):
-    """Fewer tokens than half the compute units: several workgroups share a
+    """Fewer tokens than half the compute units (for large experts up to two
+    thirds, in two rounds of workgroups): several workgroups share a
     token, each taking every n-th slice of both projections, the intermediate
     activations crossing memory once.  Shapes with fewer slices than
     workgroups per token (some get nothing to walk) and rows that do not fill
@@ -479,7 +480,7 @@ def test_tokens_shared_between_workgroups(gpu, oracle, d_model, d_ff, p0):
     experts = 4
     stack = synthetic.build_stack(experts, d_model, d_ff, p0, seed=31)
     prep = stack.prepare()
-    for tokens in (2, 3, 7, 30, 100, 128):
+    for tokens in (2, 3, 7, 30, 100, 128, 150):
         x = synthetic.activations(tokens, d_model, seed=32 + tokens)
         route = (torch.arange(tokens, dtype=torch.int32, device='cuda') * 3) % experts
         bad = 0
