@@ -392,9 +392,11 @@ __global__ void fill_bytes_kernel(uint8_t *p, int64_t n, uint8_t v) {
   if (i < n) p[i] = v;
 }
 
-__global__ void zero_words_kernel(int32_t *p, int n) {
+// keep_faults: leave words 1 and 2 (the fault counts of the control words) as
+// an earlier launch of the same call left them.
+__global__ void zero_words_kernel(int32_t *p, int n, bool keep_faults = false) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) p[i] = 0;
+  if (i < n && !(keep_faults && (i == 1 || i == 2))) p[i] = 0;
 }
 
 // ------------------------------------------------------------- main kernel --
@@ -1859,9 +1861,12 @@ double part_passes(int slices, int waves, int groups_max) {
 
 // Launch of the prepared kernels.  kinds == 2: y = wo(relu(wi x)) per token,
 // workspace required; kinds == 1: y += W x per token, no workspace.
+// `piece`: 0 for a caller's launch; 1 and 2 for the first and the later pieces
+// when a launch is split in two (a piece is not split again, and a later piece
+// keeps the fault counts of the first).
 int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *x, int64_t ldx,
                     void *y, int64_t ldy, int tokens, void *workspace, int64_t workspace_bytes,
-                    hipStream_t s, const char *who) {
+                    hipStream_t s, const char *who, int piece = 0) {
   if (!p.meta || !p.codes || !x || !y) return fail(SUB1_ERR_NULL, "%s: NULL argument", who);
   if (p.kinds == 2 && !token_matrix) return fail(SUB1_ERR_NULL, "%s: NULL token_expert", who);
   if (tokens < 0 || tokens > (1 << 20))
@@ -2025,12 +2030,16 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   if (p.kinds == 2 && lds_fused <= lds_limit) {
     const double token_us = 8.0 + static_cast<double>(p.total_chunks) * (64.0 * kFields) /
                                       p.count / 23400.0;
-    const int64_t rounds16 = (tokens + cus - 1) / cus, rounds8 = (tokens + 2 * cus - 1) / (2 * cus);
-    double fused_us = rounds16 * token_us;
-    if (2 * lds_fused <= lds_limit && 1.94 * rounds8 < rounds16) {
-      fused_us = 1.94 * rounds8 * token_us;
-      fused_per_cu = 2;
-    }
+    auto fused_estimate = [&](int64_t n, int *per_cu) {
+      const int64_t rounds16 = (n + cus - 1) / cus, rounds8 = (n + 2 * cus - 1) / (2 * cus);
+      *per_cu = 1;
+      if (2 * lds_fused <= lds_limit && 1.94 * rounds8 < rounds16) {
+        *per_cu = 2;
+        return 1.94 * rounds8 * token_us;
+      }
+      return rounds16 * token_us;
+    };
+    const double fused_us = fused_estimate(tokens, &fused_per_cu);
     double weight = 0.0;
     for (int i = 0; i < 2; i++) weight += static_cast<double>(a.k[i].slices) * p.max_chunks[i];
     double cut_us = 8.0;
@@ -2055,26 +2064,54 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     // by projection.
     const size_t lds_shared = lds_base + static_cast<size_t>(waves / 2) *
                                              std::max(a.k[0].groups_max, a.k[1].groups_max) * 256;
-    if (tokens <= cus && lds_shared <= lds_limit) {
+    auto shared_estimate = [&](int64_t n, int *best_parts) {
       double best_us = 1e30;
-      int best_parts = 0;
-      for (int parts = 2; parts <= 64 && static_cast<int64_t>(tokens) * parts <= 2 * cus; parts++) {
+      *best_parts = 0;
+      if (n > cus || lds_shared > lds_limit) return best_us;
+      for (int parts = 2; parts <= 64 && n * parts <= 2 * cus; parts++) {
         // beyond one workgroup per compute unit the rest of the grid starts as
         // the first tokens finish: two rounds, measured 7% above twice one
-        const int rounds = static_cast<int64_t>(tokens) * parts > cus ? 2 : 1;
+        const int rounds = n * parts > cus ? 2 : 1;
         double task = (a.k[0].width + a.k[1].width) / 2700.0 + 0.03 * parts;
         for (int i = 0; i < 2; i++) {
           const KindArgs &k = a.k[i];
           const double pass_us = (token_us - 8.0) * waves * p.max_chunks[i] / weight;
           task += part_passes((k.slices + parts - 1) / parts, waves, k.groups_max) * pass_us + 0.5;
         }
-        const double us = 8.0 + (rounds == 2 ? 2.24 : 1.0) * task + 0.008 * tokens * parts;
+        const double us = 8.0 + (rounds == 2 ? 2.24 : 1.0) * task + 0.008 * n * parts;
         if (us < best_us) {
           best_us = us;
-          best_parts = parts;
+          *best_parts = parts;
         }
       }
-      if (best_parts && best_us < cut_us && best_us < fused_us) shared_parts = best_parts;
+      return best_us;
+    };
+    int best_parts = 0;
+    const double shared_us = shared_estimate(tokens, &best_parts);
+    if (best_parts && shared_us < cut_us && shared_us < fused_us) shared_parts = best_parts;
+    // More than a token per compute unit, and a last round of whole tokens that
+    // would be mostly empty: whole rounds as they are, the rest as shared
+    // tokens in a launch of its own (300 tokens on 256 units: 256 whole and 44
+    // shared instead of cut tiles or two rounds; measured 5 to 25% faster just
+    // above a whole number of rounds).  The second launch is taken as 6 us, and
+    // the split must promise 7%: the estimates are no better than that.  Not
+    // where tokens are grouped by expert, which wants them all in one launch.
+    if (piece == 0 && tokens > cus && tokens % cus != 0 &&
+        !(tokens >= 4 * static_cast<int64_t>(p.count) && tokens >= 4 * cus)) {
+      const int whole = tokens / cus * cus;
+      int unused = 0, rest_parts = 0;
+      const double split_us = fused_estimate(whole, &unused) +
+                              shared_estimate(tokens - whole, &rest_parts) + 6.0;
+      if (rest_parts && split_us < 0.93 * std::min(cut_us, fused_us)) {
+        const uint16_t *xs = static_cast<const uint16_t *>(x);
+        uint16_t *ys = static_cast<uint16_t *>(y);
+        const int rc = launch_prepared(p, token_matrix, xs, ldx, ys, ldy, whole, workspace,
+                                       workspace_bytes, s, who, 1);
+        if (rc) return rc;
+        return launch_prepared(p, token_matrix + whole, xs + static_cast<int64_t>(whole) * ldx, ldx,
+                               ys + static_cast<int64_t>(whole) * ldy, ldy, tokens - whole,
+                               workspace, workspace_bytes, s, who, 2);
+      }
     }
     if (!shared_parts && fused_us < cut_us) {
       fused = true;
@@ -2095,7 +2132,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(lds_shared)));
     const int nctrl = kCtrlHeader + tokens;
-    zero_words_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl);
+    zero_words_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl, piece == 2);
     moe_prepared_shared_kernel<<<tokens * shared_parts, 64 * waves, lds_shared, s>>>(a);
     HIP_TRY(hipGetLastError());
     return SUB1_OK;
@@ -2135,7 +2172,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
                              : reinterpret_cast<const void *>(moe_prepared_fused_kernel<false>);
     HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(lds_fused)));
-    zero_words_kernel<<<1, 256, 0, s>>>(a.ctrl, kCtrlHeader);
+    zero_words_kernel<<<1, 256, 0, s>>>(a.ctrl, kCtrlHeader, piece == 2);
     if (grouped) {
       int32_t *tab = reinterpret_cast<int32_t *>(a.h);
       int32_t *order = tab + table_ints;
@@ -2176,7 +2213,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
                               static_cast<int>(lds)));
   if (a.ctrl) {
     int nctrl = kCtrlHeader + tokens;
-    zero_words_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl);
+    zero_words_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl, piece == 2);
   }
   if (small) {
     const int64_t grid = tiles < cus ? tiles : cus;
