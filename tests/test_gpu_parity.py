@@ -505,6 +505,34 @@ def test_tokens_shared_between_workgroups(gpu, oracle, d_model, d_ff, p0):
     assert np.array_equal(bits_host(y[t]), ref)
 
 
+def test_shared_token_launches_on_several_streams(gpu):
+    """Launches whose workgroups wait for each other (several per token) from
+    three streams at once: together they ask for three times the compute
+    units, so none has all its workgroups on the GPU at the start.  Every
+    launch still completes without running into its wait limit, with the
+    results of the same launches made one after the other."""
+    from qmoe_amd import synthetic
+    d_model, d_ff = synthetic.SHAPES['large']
+    tokens = 128
+    preps = [synthetic.build_stack(16, d_model, d_ff, 0.88, seed=81 + i).prepare() for i in range(3)]
+    xs = [synthetic.activations(tokens, d_model, seed=85 + i) for i in range(3)]
+    route = (torch.arange(tokens, dtype=torch.int32, device='cuda') * 5) % 16
+    want = [p.forward(x, route).clone() for p, x in zip(preps, xs)]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in preps]
+    ys = [torch.empty_like(x) for x in xs]
+    for s in streams:
+        s.wait_stream(torch.cuda.current_stream())
+    for rep in range(40):
+        for p, x, y, s in zip(preps, xs, ys, streams):
+            with torch.cuda.stream(s):
+                p.forward(x, route, y)
+    torch.cuda.synchronize()
+    for p, y, ref in zip(preps, ys, want):
+        assert p.launch_faults(tokens) == (0, 0)
+        assert torch.equal(y, ref)
+
+
 @pytest.mark.parametrize('d_model,d_ff', [(64, 12288), (12288, 64), (2, 2)])
 def test_extreme_widths_in_every_batch_regime(gpu, oracle, d_model, d_ff):
     """The widest activations the fast layout takes and the narrowest, from one
