@@ -211,6 +211,12 @@ class FasterMLP(nn.Module):
         self.router = mlp.router
         self.experts = nn.ModuleList(mlp.experts.values())
         self.gpu = gpu
+        # the launch applies ReLU between wi and wo, as Switch's experts do
+        # (HuggingFace's DenseActDense keeps its activation in `act`)
+        for expert in self.experts:
+            act = getattr(expert, 'act', None)
+            if act is not None and not isinstance(act, nn.ReLU):
+                raise ValueError('FasterMLP runs ReLU experts; this one has %r' % (act,))
 
     def _sentinels(self):
         # a few of the experts' tensors stand for all of them in the per-call

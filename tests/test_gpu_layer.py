@@ -136,6 +136,22 @@ def test_faster_mlp_equals_the_expert_loop(gpu, order):
     assert fast._launcher() is not stacked
 
 
+def test_faster_mlp_refuses_other_activations(gpu):
+    """The launch computes ReLU between the projections; an expert that says it
+    uses another activation (HuggingFace keeps it in `act`) is refused."""
+    sub1 = gpu
+    g = torch.Generator(device='cuda').manual_seed(59)
+    expert = Expert(sub1.Sub1Linear.make(ternary_dense(64, 32, 0.8, g)),
+                    sub1.Sub1Linear.make(ternary_dense(32, 64, 0.8, g)))
+    expert.act = nn.GELU()
+    mlp = types.SimpleNamespace(router=Top1Router(32, 1, 4, 'probs_first').cuda(),
+                                experts=nn.ModuleDict({'expert_0': expert}))
+    with pytest.raises(ValueError, match='ReLU'):
+        sub1.FasterMLP(mlp)
+    expert.act = nn.ReLU()
+    sub1.FasterMLP(mlp)
+
+
 def test_checkpoint_directory_to_one_launch_layer(gpu, tmp_path):
     """Experts written in the reference's directory format come back as one
     stacked layer whose output equals the per-expert layers' output."""
