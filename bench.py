@@ -291,6 +291,9 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py measures one GPU: this build has no multi-GPU path (--gpus 1 only)')
+    from qmoe_amd import _lib, build as _build
+    if not os.path.exists(_lib.LIB_PATH):      # uses what is built; builds only if nothing is
+        _build.build_library()
     if args.calibrate_copy:
         import torch
         n = args.calibrate_copy << 20

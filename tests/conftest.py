@@ -10,6 +10,12 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line('markers', 'gpu: needs a real MI355X (run with -m gpu)')
+    # The package refuses to import without its library (there is no CPU
+    # fallback).  The tests use what is built and build only if nothing is.
+    from qmoe_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from qmoe_amd import build
+        build.build_library()
 
 
 @pytest.fixture(scope='session')
