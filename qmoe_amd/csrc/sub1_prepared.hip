@@ -530,10 +530,11 @@ typedef Walk<kRing> SliceWalk;
 
 // g_lo, g_hi: the run of chunk groups to walk, for a wavefront that shares the
 // slice with others (it then starts from the position checkpoint of group g_lo).
-__device__ __forceinline__ SliceWalk load_slice(const PreparedArgs &a, const KindArgs &k,
-                                                int64_t sl, int g_lo = 0, int g_hi = 1 << 20) {
+template <int R = kRing>
+__device__ __forceinline__ Walk<R> load_slice(const PreparedArgs &a, const KindArgs &k,
+                                              int64_t sl, int g_lo = 0, int g_hi = 1 << 20) {
   const int lane = threadIdx.x & 63;
-  SliceWalk w;
+  Walk<R> w;
   const int nch_all = __builtin_amdgcn_readfirstlane(k.slice_nch[sl]);
   w.nch = min(g_hi * kGroupChunks, nch_all);
   w.c0 = g_lo * kGroupChunks;
@@ -545,7 +546,7 @@ __device__ __forceinline__ SliceWalk load_slice(const PreparedArgs &a, const Kin
     w.j0 = a.ckpt[(checkpoint_entry(w.base, k.first_slice + sl) + g_lo) * 64 + lane];
   const uint2 *p = chunk_pointer(a.stream, w.base);
 #pragma unroll
-  for (int i = 0; i < kRing; i++) w.ring[i] = p[min(w.c0 + i, w.nch - 1) * 64];
+  for (int i = 0; i < R; i++) w.ring[i] = p[min(w.c0 + i, w.nch - 1) * 64];
   return w;
 }
 
@@ -593,8 +594,10 @@ __device__ __forceinline__ void progress_priority(int done, int total) {
 // sum at part[group * 64 + lane] for the wavefront that adds them up.
 // pass / passes (passes != 0): this slice is the wavefront's pass-th of `passes`
 // about equal ones in the current phase; sets the priority by progress.
-__device__ __forceinline__ float run_slice(SliceWalk &w, const uint2 *stream, const uint32_t *xa,
+template <int R>
+__device__ __forceinline__ float run_slice(Walk<R> &w, const uint2 *stream, const uint32_t *xa,
                                            float *part = nullptr, int pass = 0, int passes = 0) {
+  static_assert(kGroupChunks % R == 0, "a group of chunks is a whole number of ring turns");
   // a walk that went through `cur = nxt` may sit in vector registers: put what
   // is the same in all lanes back into scalar ones, for scalar loop control
   // and scalar address arithmetic
@@ -607,22 +610,22 @@ __device__ __forceinline__ float run_slice(SliceWalk &w, const uint2 *stream, co
   int c = __builtin_amdgcn_readfirstlane(w.c0);
   if (passes) progress_priority(pass, passes);
   auto group_done = [&]() {
-    if (passes) progress_priority(pass * w.nch + c + kRing, passes * w.nch);
+    if (passes) progress_priority(pass * w.nch + c + R, passes * w.nch);
     if (part) {
-      part[((c + kRing) / kGroupChunks - 1) * 64 + lane] = partial;
+      part[((c + R) / kGroupChunks - 1) * 64 + lane] = partial;
     } else {
       sum += partial;
     }
     partial = 0.f;
   };
-  for (; c + kRing <= w.nch; c += kRing) {
+  for (; c + R <= w.nch; c += R) {
     run_chunks<false>(w, p, c, at, partial, minmax);
-    if ((c + kRing) % kGroupChunks == 0) group_done();
+    if ((c + R) % kGroupChunks == 0) group_done();
   }
   if (c < w.nch) {
     run_chunks<true>(w, p, c, at, partial, minmax);
-    if ((c + kRing) % kGroupChunks == 0) group_done();
-    c += kRing;
+    if ((c + R) % kGroupChunks == 0) group_done();
+    c += R;
   }
   if (part) {
     // the slice's last group, unless the loop has just closed it
@@ -987,7 +990,7 @@ __device__ __forceinline__ void walk_tile(const PreparedArgs &a, const KindArgs 
   int split = 1;
   const int rest = all % waves;
   if (rest > 0 && rest * 2 <= waves && rest * k.groups_max <= a.tail_room)
-    while (split * 2 * rest <= waves && split * 2 <= k.groups_max) split *= 2;
+    split = min(waves / rest, k.groups_max);
   const int count = split > 1 ? all - rest : all;
   const int passes = (count + waves - 1) / waves + (split > 1);
   int s = slice_of_pass(0, wave, waves, count);
@@ -1017,8 +1020,15 @@ __device__ __forceinline__ void walk_tile(const PreparedArgs &a, const KindArgs 
                kGroupChunks;
       const int g_lo = sub * groups / split, g_hi = (sub + 1) * groups / split;
       if (g_lo < g_hi) {
-        SliceWalk tail = load_slice(a, k, slice, g_lo, g_hi);
-        run_slice(tail, a.stream, act, mine);
+        if (count == 0) {
+          // this pass is all there is (a few tokens): the walk is a chain of
+          // memory round trips, so a whole group of chunks is kept in flight
+          Walk<kSplitRing> tail = load_slice<kSplitRing>(a, k, slice, g_lo, g_hi);
+          run_slice(tail, a.stream, act, mine);
+        } else {
+          SliceWalk tail = load_slice(a, k, slice, g_lo, g_hi);
+          run_slice(tail, a.stream, act, mine);
+        }
       }
     }
     __syncthreads();
@@ -1852,8 +1862,7 @@ double part_passes(int slices, int waves, int groups_max) {
   double passes = slices / waves;
   if (rest > 0) {
     int split = 1;
-    if (rest * 2 <= waves)
-      while (split * 2 * rest <= waves && split * 2 <= groups_max) split *= 2;
+    if (rest * 2 <= waves) split = std::max(1, std::min(waves / rest, groups_max));
     passes += std::max(static_cast<double>(rest * split) / waves, 0.3) / split;
   }
   return passes;
