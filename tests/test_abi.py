@@ -87,3 +87,15 @@ def test_python_surface_imports_without_a_gpu():
     assert lin.w_comp.dtype.__str__() == 'torch.int16' and lin.row_off.shape == (17,)
     assert lin.ter_minmax.shape == (32,) and lin.weight.numel() == 0
     assert callable(sub1_hip.sub1matvec) and callable(sub1_hip.sub1pack)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it exits with a message that
+    says so, before touching any GPU."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, 'bench.py'), '--gpus', '2'],
+                         capture_output=True, text=True, timeout=120)
+    assert res.returncode != 0
+    assert 'one GPU' in res.stderr
