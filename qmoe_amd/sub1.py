@@ -167,27 +167,38 @@ class Sub1Experts(nn.Module):
 
 
 def _router_outputs(outputs, experts):
-    """(one-hot routing mask [.., E], probabilities [.., 1], logits [.., E])
-    from a Switch top-1 router's 3-tuple, whatever its order: transformers
-    4.28 returns (mask, probs, logits) (reference sub1.py:310), later versions
-    put the probabilities first.  The probabilities are the entry whose last
-    dimension is 1; of the two [.., E] entries the mask is the integer one."""
-    probs = [o for o in outputs if o.shape[-1] == 1 and experts != 1]
-    wide = [o for o in outputs if o.shape[-1] == experts and not any(o is p for p in probs)]
-    if experts == 1:
-        wide = list(outputs)
-        floats = [o for o in wide if o.is_floating_point()]
-        mask = [o for o in wide if not o.is_floating_point()]
-        if len(mask) != 1 or len(floats) != 2:
-            raise ValueError('cannot tell the router outputs apart')
-        # with one expert the top-1 probability is softmax of one logit = 1
-        return mask[0], floats[0], floats[1]
-    mask = [o for o in wide if not o.is_floating_point()]
-    logits = [o for o in wide if o.is_floating_point()]
-    if len(probs) != 1 or len(mask) != 1 or len(logits) != 1:
-        raise ValueError('cannot tell the router outputs apart: shapes %s'
+    """(one-hot routing mask [.., E], top-1 probabilities [.., 1], the third
+    output) from a Switch top-1 router's 3-tuple, in whichever form the
+    installed transformers returns it:
+
+      4.28 (reference sub1.py:310)  (mask [.., E] int, probs [.., 1], logits [.., E])
+      5.x                           (probs [.., 1], mask [.., 1, E] int64, max prob [.., 1])
+
+    The mask is the one integer tensor; a singleton top-k axis in front of its
+    expert axis is squeezed.  Of the two floating tensors the probabilities are
+    the one whose last dimension is 1; where both are (5.x, or a single
+    expert), the one that comes first in the tuple."""
+    outputs = tuple(outputs)
+    if len(outputs) != 3:
+        raise ValueError('a Switch top-1 router returns three tensors, got %d' % len(outputs))
+    masks = [o for o in outputs if not o.is_floating_point()]
+    floats = [o for o in outputs if o.is_floating_point()]
+    if len(masks) != 1 or len(floats) != 2 or masks[0].shape[-1] != experts:
+        raise ValueError('cannot tell the router outputs apart: %s'
+                         % [(tuple(o.shape), o.dtype) for o in outputs])
+    mask = masks[0]
+    narrow = [o for o in floats if o.shape[-1] == 1]
+    if not narrow:
+        raise ValueError('no [.., 1] probabilities among the router outputs: %s'
                          % [tuple(o.shape) for o in outputs])
-    return mask[0], probs[0], logits[0]
+    probs = narrow[0]
+    other = floats[1] if floats[0] is probs else floats[0]
+    if mask.dim() == probs.dim() + 1 and mask.shape[-2] == 1:
+        mask = mask.squeeze(-2)
+    if mask.shape[:-1] != probs.shape[:-1]:
+        raise ValueError('router mask %s and probabilities %s do not describe the same tokens'
+                         % (tuple(mask.shape), tuple(probs.shape)))
+    return mask, probs, other
 
 
 class FasterMLP(nn.Module):
@@ -202,15 +213,26 @@ class FasterMLP(nn.Module):
     load_state_dict or `refresh()`; the per-call check looks at four of the
     experts' tensors only, so other writes to the buffers need `refresh()`);
     tokens stay on their GPU (one GPU here, the reference moves them to the
-    layer's GPU and back, sub1.py:307-320)."""
+    layer's GPU and back, sub1.py:307-320).
 
-    def __init__(self, mlp, gpu=None):
+    `router_outputs`: what forward() returns.  True: the reference's pair
+    `(hidden_states, (router_logits, expert_index))`, which the Switch block of
+    transformers 4.28 unpacks; False: `hidden_states` alone, which the block of
+    transformers 5.x adds to its residual.  None (default) follows the wrapped
+    module: a sparse MLP whose forward is annotated to return a tensor gets the
+    tensor, anything else the reference's pair."""
+
+    def __init__(self, mlp, gpu=None, router_outputs=None):
         super().__init__()
         if gpu is not None:
             mlp = mlp.to(gpu)
         self.router = mlp.router
         self.experts = nn.ModuleList(mlp.experts.values())
         self.gpu = gpu
+        if router_outputs is None:
+            returns = getattr(getattr(type(mlp), 'forward', None), '__annotations__', {}).get('return')
+            router_outputs = returns not in (torch.Tensor, 'torch.Tensor')
+        self.router_outputs = bool(router_outputs)
         # the launch applies ReLU between wi and wo, as Switch's experts do
         # (HuggingFace's DenseActDense keeps its activation in `act`)
         for expert in self.experts:
@@ -276,9 +298,10 @@ class FasterMLP(nn.Module):
         return cached[1]
 
     def forward(self, hidden_states):
-        """hidden_states [B, S, d_model] -> (router_probs * expert output,
-        (router_logits, expert_index)); tokens that the router's capacity
-        limit dropped keep their input (reference sub1.py:312-318)."""
+        """hidden_states [B, S, d_model] -> router_probs * expert output (with
+        `router_outputs` also (router_logits, expert_index), reference
+        sub1.py:321); tokens that the router's capacity limit dropped keep
+        their input (reference sub1.py:312-318)."""
         router_mask, router_probs, router_logits = _router_outputs(
             self.router(hidden_states), len(self.experts))
         expert_index = torch.argmax(router_mask, dim=-1)
@@ -287,4 +310,6 @@ class FasterMLP(nn.Module):
         x = hidden_states.reshape(-1, hidden_states.shape[-1]).to(torch.bfloat16).contiguous()
         next_states = self._launcher().forward(x, route.reshape(-1))
         hidden_states = router_probs * next_states.view(hidden_states.shape).to(hidden_states.dtype)
-        return hidden_states, (router_logits, expert_index)
+        if self.router_outputs:
+            return hidden_states, (router_logits, expert_index)
+        return hidden_states

@@ -136,6 +136,59 @@ def test_faster_mlp_equals_the_expert_loop(gpu, order):
     assert fast._launcher() is not stacked
 
 
+def test_faster_mlp_in_a_huggingface_sparse_mlp(gpu):
+    """A SwitchTransformersSparseMLP of the installed transformers, built from
+    a config (nothing is fetched), its experts' wi/wo replaced by
+    Sub1Linear.make(...): FasterMLP around it equals the reference's loop
+    (sub1.py:306-321) on the same modules bit for bit, returns what the
+    installed Switch block expects from its mlp, and agrees with HuggingFace's
+    own expert loop on the compressed experts to bf16 rounding."""
+    pytest.importorskip('transformers')
+    from transformers.models.switch_transformers import modeling_switch_transformers as hf
+    from qmoe_amd import sub1
+    d_model, d_ff, experts, batch, seq = 256, 512, 8, 2, 40
+    cfg = hf.SwitchTransformersConfig(d_model=d_model, d_ff=d_ff, num_experts=experts,
+                                      expert_capacity=64, num_layers=2,
+                                      num_sparse_encoder_layers=1, num_heads=4, d_kv=64,
+                                      vocab_size=128, router_jitter_noise=0.0, dropout_rate=0.0)
+    torch.manual_seed(43)
+    block = hf.SwitchTransformersLayerFF(cfg, is_sparse=True).cuda().bfloat16().eval()
+    mlp = block.mlp
+    assert isinstance(mlp, hf.SwitchTransformersSparseMLP)
+    g = torch.Generator(device='cuda').manual_seed(44)
+    for e in range(experts):
+        expert = mlp.experts['expert_%d' % e]
+        expert.wi = sub1.Sub1Linear.make(ternary_dense(d_ff, d_model, 0.85, g))
+        expert.wo = sub1.Sub1Linear.make(ternary_dense(d_model, d_ff, 0.85, g))
+    hidden = torch.randn((batch, seq, d_model), generator=g, device='cuda').bfloat16()
+    fast = sub1.FasterMLP(mlp)
+    with torch.no_grad():
+        got = fast(hidden)
+        router_mask, router_probs, _ = sub1._router_outputs(mlp.router(hidden), experts)
+        # reference sub1.py:311-318 on the same modules
+        next_states = hidden.clone()
+        for e in torch.nonzero(router_mask.sum(dim=(0, 1)), as_tuple=True)[0]:
+            sel = router_mask[:, :, e].bool()
+            next_states[sel] = mlp.experts['expert_%d' % int(e)](hidden[sel])
+        want = router_probs * next_states
+        theirs = mlp(hidden)
+    pair = isinstance(theirs, tuple)
+    assert fast.router_outputs is pair
+    if pair:
+        got, theirs = got[0], theirs[0]
+    assert len(torch.unique(router_mask.argmax(-1))) > 1      # several experts hit
+    assert torch.equal(got, want)
+    assert torch.linalg.norm(got.float() - theirs.float()) <= 1e-2 * torch.linalg.norm(theirs.float())
+    # plugged into the block: layer norm, the compressed sparse MLP, residual
+    with torch.no_grad():
+        plain = block(hidden)
+        block.mlp = fast
+        plugged = block(hidden)
+    plain = plain[0] if isinstance(plain, tuple) else plain
+    plugged = plugged[0] if isinstance(plugged, tuple) else plugged
+    assert torch.linalg.norm(plugged.float() - plain.float()) <= 1e-2 * torch.linalg.norm(plain.float())
+
+
 def test_faster_mlp_refuses_other_activations(gpu):
     """The launch computes ReLU between the projections; an expert that says it
     uses another activation (HuggingFace keeps it in `act`) is refused."""
