@@ -22,10 +22,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 counter runs of this same
-# command (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a 1 GiB device copy reads on
-# those counters); the summaries are under profiles/.  None where no run was made.
-MEASURED_TRAFFIC = {'c2048-sweep': 4.905e9 + 0.057e9}
+# HBM bytes per launch of the dominant kernel.  A recorded figure, not measured by this run:
+# it comes from rocprofv3 counter runs of this same command (FETCH_SIZE x 2.0 + WRITE_SIZE x
+# 1.0, the factors a 1 GiB device copy reads on those counters), summarised in the file
+# named beside it.  None where no such run was made.
+MEASURED_TRAFFIC = {'c2048-sweep': (4.905e9 + 0.057e9,
+                                    'profiles/moe_prepared_fused_kernel_c2048_sweep.txt')}
 
 WORKLOADS = {
     # name: (shape key, experts, p_zero, description)
@@ -281,48 +283,16 @@ def main():
                          '`--steps` times, for a profiler')
     ap.add_argument('--single-matrix-only', action='store_true',
                     help='instead of the benchmark, run only the one-product-per-shape protocol')
-    ap.add_argument('--probe-gathers', action='store_true',
-                    help='instead of the benchmark, measure the time per random-gather '
-                         'instruction from LDS and from global tables (the bound of the inner loop)')
     ap.add_argument('--seed', type=int, default=20231116)
-    ap.add_argument('--calibrate-copy', type=int, default=0, metavar='MIB',
-                    help='instead of the benchmark, run a plain device copy of this many MiB '
-                         '(to scale the FETCH_SIZE / WRITE_SIZE counters of a profiler run)')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py measures one GPU: this build has no multi-GPU path (--gpus 1 only)')
     from qmoe_amd import _lib, build as _build
     if not os.path.exists(_lib.LIB_PATH):      # uses what is built; builds only if nothing is
         _build.build_library()
-    if args.calibrate_copy:
-        import torch
-        n = args.calibrate_copy << 20
-        src = torch.ones(n, dtype=torch.uint8, device='cuda')
-        dst = torch.empty_like(src)
-        for _ in range(args.steps):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        print(json.dumps({'copy_bytes_read': n, 'copy_bytes_written': n, 'copies': args.steps}))
-        return
-
     import ctypes
     import torch
-    from qmoe_amd import synthetic
-
-    if args.probe_gathers:
-        from qmoe_amd import _lib
-        lib = _lib.load()
-        torch.cuda.set_device(0)
-        stream_ptr = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-        rows = {}
-        for name, from_lds, words in (('lds_16k_words', 1, 16384), ('lds_32k_words', 1, 32768),
-                                      ('global_4KB', 0, 1024), ('global_16KB', 0, 4096),
-                                      ('global_64KB', 0, 16384), ('global_256KB', 0, 65536)):
-            c = ctypes.c_double()
-            _lib.check(lib.sub1_probe_gather(from_lds, words, 4000, ctypes.byref(c), stream_ptr))
-            rows[name] = round(c.value, 3)
-        print(json.dumps({'ns_per_wavefront_gather_per_compute_unit': rows}))
-        return
+    from qmoe_amd import _lib, synthetic
 
     if args.single_matrix_only:
         torch.cuda.set_device(0)
@@ -345,9 +315,10 @@ def main():
     tick = time.perf_counter()
     prep = stack.prepare()
     torch.cuda.synchronize()
+    prepare_ms = (time.perf_counter() - tick) * 1e3
     print('prepared in %.2f s: %.3f GB of interleaved gap entries (%.3f x the packed codes) + '
           '%.3f GB of position checkpoints' %
-          (time.perf_counter() - tick, prep.stream_bytes / 1e9,
+          (prepare_ms / 1e3, prep.stream_bytes / 1e9,
            prep.stream_bytes / (2.0 * stack.w_comp.numel()),
            (prep.code_bytes - prep.stream_bytes) / 1e9), file=sys.stderr)
 
@@ -372,10 +343,17 @@ def main():
 
     wall, us_launch = time_launches(lambda: prep.forward(x, route, y), args.steps,
                                     args.warmup, stream_ptr)
+    kernel = _lib.load().sub1_last_kernel().decode()      # what the library launched
     assert prep.launch_faults(experts) == (0, 0)
     ms_per_step = wall / args.steps * 1e3
     abytes = algorithmic_bytes(stack, range(experts))
     achieved = abytes / (us_launch * 1e-6) / 1e9
+    traffic, traffic_source = MEASURED_TRAFFIC.get(args.workload, (None, None)) \
+        if not args.experts else (None, None)
+    # what the kernel fetches: the entry stream once (the checkpoints behind it are not
+    # read by the streaming kernel), row order and min/max of every slice, x and y
+    fetched = int(prep.stream_bytes) + 6 * 64 * (-(-d_ff // 64) + -(-d_model // 64)) * experts \
+        + 4 * experts * d_model
 
     out = {
         'metric': 'us per compressed MoE layer (batch-1) + achieved HBM GB/s vs roofline',
@@ -390,17 +368,24 @@ def main():
         'config': {'workload': desc, 'experts': experts, 'd_model': d_model, 'd_ff': d_ff,
                    'p_zero': p_zero, 'tokens': experts,
                    'compressed_bytes': stack.compressed_bytes(),
-                   'prepared_stream_bytes': int(prep.stream_bytes),
                    'bits_per_weight': round(16.0 * stack.w_comp.numel()
-                                            / (2.0 * experts * d_model * d_ff), 4)},
+                                            / (2.0 * experts * d_model * d_ff), 4),
+                   # the timed kernel reads a stream made ONCE from the codes, untimed:
+                   'prepare_ms': round(prepare_ms, 1),
+                   'prepared_stream_bytes': int(prep.stream_bytes),
+                   'prepared_total_bytes': int(prep.code_bytes) + int(prep.meta.numel()),
+                   'prepared_bits_per_weight': round(
+                       8.0 * (int(prep.code_bytes) + int(prep.meta.numel()))
+                       / (2.0 * experts * d_model * d_ff), 4),
+                   'both_forms_resident': True},
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS,
                      'unit': 'GB/s', 'frac': round(achieved / HBM_PEAK_GBS, 4),
-                     'traffic': MEASURED_TRAFFIC.get(args.workload) if not args.experts else None,
-                     # the library picks the kernel: a token per workgroup from one token
-                     # per compute unit on, several workgroups per token below half of that
-                     'kernel': ('moe_prepared_fused_kernel<false>' if experts >= 256
-                                else 'moe_prepared_shared_kernel'),
-                     'algorithmic_bytes': abytes, 'us_per_launch': round(us_launch, 2)},
+                     'traffic': traffic, 'traffic_source': traffic_source,
+                     'kernel': kernel,
+                     'algorithmic_bytes': abytes, 'us_per_launch': round(us_launch, 2),
+                     'fetched_bytes_by_layout': fetched,
+                     'frac_on_fetched_bytes': round(
+                         (traffic or fetched) / (us_launch * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)},
     }
 
     if args.sweep_only:
@@ -417,6 +402,10 @@ def main():
     y2 = torch.empty_like(x)
     _, us_ref = time_launches(lambda: stack.forward(x, route, y2), 3, 1, stream_ptr)
     also['reference_layout_kernel_us'] = round(us_ref, 1)
+    # the same workload with the dictionary decoded inside the kernel, no preparation
+    out['roofline']['reference_layout'] = {
+        'kernel': _lib.load().sub1_last_kernel().decode(), 'us_per_launch': round(us_ref, 1),
+        'frac': round(abytes / (us_ref * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
     also['prepared_vs_reference_layout_rel_diff'] = rel_diff(y, y2)
     if not also['prepared_vs_reference_layout_rel_diff'] <= 1e-2:
         raise SystemExit('the prepared kernel and the packed-layout kernel disagree on the sweep')
@@ -433,9 +422,14 @@ def main():
     if not args.no_dense:
         n = min(experts, 128)
         d_us = dense_gemv_us(stack, x, n)
+        dense_bytes = experts * (4 * d_model * d_ff + 6 * d_model + 4 * d_ff)
         also['dense_bf16_gemv'] = {'us_per_expert_ffn': round(d_us, 2), 'experts_timed': n,
                                    'us_per_layer_extrapolated': round(d_us * experts, 1),
-                                   'sub1_us_per_expert_ffn': round(us_launch / experts, 2)}
+                                   'sub1_us_per_expert_ffn': round(us_launch / experts, 2),
+                                   # torch.bmm runs far below the HBM rate on these shapes; the
+                                   # bound a dense kernel cannot beat is its bytes at 8 TB/s
+                                   'dense_bytes': dense_bytes,
+                                   'us_per_layer_at_hbm_peak': round(dense_bytes / HBM_PEAK_GBS / 1e3, 1)}
     if not args.experts and args.workload == 'c2048-sweep':
         # the two smaller layers of the configuration list; their compressed stacks
         # (57 MB, 110 MB) fit the 256 MB last-level cache, so these are not HBM rates
@@ -469,11 +463,13 @@ def main():
     out['also'] = also
 
     if not args.no_cpu:
-        cores = min(16, len(os.sched_getaffinity(0)))
+        available = len(os.sched_getaffinity(0))
+        cores = min(16, available)          # threads used; a one-GPU box's share is 16
         done1, spent1 = cpu_baseline(stack, x, min(experts, 64), 1, budget_s=3.0)
         done, spent = cpu_baseline(stack, x, experts, cores)
         out['cpu_baseline'] = {
             'value': round(spent / done * experts * 1e6, 1), 'unit': 'us/layer', 'cores': cores,
+            'cores_available': available,
             'kind': 'port',
             'sample': '%d of %d expert FFNs of the same stack through the scalar C oracle in '
                       'the reference kernel\'s lane order, %d at a time on %d host threads, '

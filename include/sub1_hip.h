@@ -49,6 +49,14 @@ const char *sub1_last_error(void);
 int sub1_abi_version(void);
 
 /*
+ * Name of the kernel that the calling thread's last product or expert-layer
+ * entry point launched ("" before the first): the library picks among several
+ * by batch size, and a benchmark reports which one it timed.  A launch that
+ * was split in two reports the second.
+ */
+const char *sub1_last_kernel(void);
+
+/*
  * Build the fixed dictionary on the HOST: dec_host[131072], trie_host[65537*9].
  * Either may be NULL.  Replaces the Python `setup()` of reference
  * sub1.py:29-102 (same table bytes).  Deterministic, no GPU needed.
@@ -61,8 +69,9 @@ int sub1_build_tables(int32_t *dec_host, int32_t *trie_host);
  * (reference sub1_cuda.cpp:35-45, sub1_cuda_kernel.cu:70-88,129-202), which
  * handled six hard-coded shapes and silently did nothing for others.
  * The first call with a given `dec` pointer derives a compact device table
- * from it (one small kernel and one allocation, cached for the process; the
- * contents of `dec` must not change afterwards).
+ * from it (one allocation, two small kernels and a synchronisation, so not
+ * inside a stream capture; cached by the address of dec, see
+ * sub1_unregister_dec).
  */
 int sub1_matvec(const int32_t *dec, const int16_t *w_comp, const int32_t *row_off,
                 const void *ter_minmax, const void *x, void *y, int height,
@@ -294,14 +303,49 @@ int sub1_timing_begin(void *stream);
 int sub1_timing_end(void *stream, double *elapsed_us);
 
 /*
- * Gather-rate probe (no counterpart in the reference; for the benchmark's
- * bound): nanoseconds a compute unit needs per wavefront instruction that reads one
- * random dword per lane from a table of `words` dwords (a power of two), held
- * in LDS (from_lds != 0, words <= 32768) or in global memory, with 16
- * wavefronts per compute unit and four gathers in flight per lane, as in the
- * kernels' inner loop.  Allocates and frees its own buffers; synchronises.
+ * Faults that a launch cannot return (no counterpart in the reference, whose
+ * kernels do not wait for each other).  The grouped launches let workgroups
+ * wait for each other's part of h; every such wait is bounded in TIME (default
+ * 250 ms on the device's constant-rate clock, far above any wait of a healthy
+ * launch, which lasts microseconds).  A wait that reaches the bound gives up:
+ * the kernel carries on and exits normally, its output is wrong, and it sets a
+ * sticky flag in pinned host memory that no launch clears.  A second flag is
+ * set when a launch finds that `dec` no longer holds what the table cached for
+ * its address was derived from (see sub1_unregister_dec).
+ *
+ *   sub1_init()               allocates the flag words (pinned host memory) and
+ *                             prepares the current device; the other entry
+ *                             points do this themselves on first use, so it is
+ *                             only needed before a stream capture.  Safe to
+ *                             call again.
+ *   sub1_fault_flags(f)       f[0] = a wait gave up, f[1] = dec changed; read
+ *                             from host memory, no synchronisation: a flag is
+ *                             seen once the launch that set it has got that far.
+ *   sub1_fault_words_host()   the two flags as int32 words in host memory (NULL
+ *                             before sub1_init or a first launch): a caller
+ *                             that polls between launches reads them directly.
+ *   sub1_clear_faults()       resets both.
+ *   sub1_set_wait_limit_us(n) the bound, 1 .. 60 000 000 us, for later launches.
+ *   sub1_test_overstate_wait(k)  for tests of the above: later launches expect k
+ *                             more workgroups in every wait than will ever
+ *                             report, so each wait runs into the bound.
  */
-int sub1_probe_gather(int from_lds, int words, int steps, double *ns_per_gather, void *stream);
+int sub1_init(void);
+int sub1_fault_flags(int32_t *flags);
+const int32_t *sub1_fault_words_host(void);
+int sub1_clear_faults(void);
+int sub1_set_wait_limit_us(int64_t microseconds);
+int sub1_test_overstate_wait(int extra);
+
+/*
+ * sub1_matvec and sub1_moe_grouped keep the compact table they derive from
+ * `dec` by the ADDRESS of dec (per device).  Call this before freeing a dec
+ * buffer whose address may be handed out again for other contents; NULL drops
+ * every cached table.  Synchronises the device.  (A launch that finds other
+ * contents at a cached address sets the flag above and the next call derives
+ * the tables afresh.)
+ */
+int sub1_unregister_dec(const int32_t *dec);
 
 #ifdef __cplusplus
 }

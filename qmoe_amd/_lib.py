@@ -51,6 +51,7 @@ class MatrixPrepared(ctypes.Structure):
 PROTOTYPES = {
     'sub1_last_error': (ctypes.c_char_p, []),
     'sub1_abi_version': (_int, []),
+    'sub1_last_kernel': (ctypes.c_char_p, []),
     'sub1_build_tables': (_int, [_vp, _vp]),
     'sub1_matvec': (_int, [_vp] * 6 + [_int, _int, _vp]),
     'sub1_matvec_tokens': (_int, [_vp] * 6 + [_int, _int, _int, _i64, _i64, _vp]),
@@ -78,7 +79,13 @@ PROTOTYPES = {
     'sub1_matrix_prepared_decode': (_int, [ctypes.POINTER(MatrixPrepared), _int, _vp, _vp]),
     'sub1_timing_begin': (_int, [_vp]),
     'sub1_timing_end': (_int, [_vp, ctypes.POINTER(ctypes.c_double)]),
-    'sub1_probe_gather': (_int, [_int, _int, _int, ctypes.POINTER(ctypes.c_double), _vp]),
+    'sub1_init': (_int, []),
+    'sub1_fault_flags': (_int, [ctypes.POINTER(ctypes.c_int32)]),
+    'sub1_fault_words_host': (_vp, []),
+    'sub1_clear_faults': (_int, []),
+    'sub1_set_wait_limit_us': (_int, [_i64]),
+    'sub1_test_overstate_wait': (_int, [_int]),
+    'sub1_unregister_dec': (_int, [_vp]),
 }
 
 _lib = None
@@ -110,3 +117,37 @@ def load():
 def check(status):
     if status != SUB1_OK:
         raise Sub1Error(status, load().sub1_last_error().decode())
+
+
+class Sub1Fault(RuntimeError):
+    """A launch could not finish its work and said so through the library's
+    sticky fault flags; outputs since the last check may be wrong."""
+
+
+_fault_words = None
+
+
+def check_faults():
+    """Raise Sub1Fault if a launch has set a fault flag: a wait between
+    workgroups gave up at its time limit (that launch's output is wrong), or a
+    `dec` buffer changed under the table cached for its address.  Reads host
+    memory, synchronises nothing: it reports what the GPU has got to so far.
+    The flags stay up until clear_faults()."""
+    global _fault_words
+    if _fault_words is None:
+        lib = load()
+        check(lib.sub1_init())
+        _fault_words = (ctypes.c_int32 * 2).from_address(lib.sub1_fault_words_host())
+    if _fault_words[0] or _fault_words[1]:
+        what = []
+        if _fault_words[0]:
+            what.append('a wait between workgroups ran into its time limit, so the output of '
+                        'that launch is wrong')
+        if _fault_words[1]:
+            what.append('a dec tensor no longer holds what the table cached for its address '
+                        'was derived from (sub1_unregister_dec before freeing one)')
+        raise Sub1Fault('libsub1_hip: ' + '; '.join(what) + ' [sticky: clear_faults() resets]')
+
+
+def clear_faults():
+    check(load().sub1_clear_faults())

@@ -13,6 +13,7 @@
 //   sub1.py:306-321              expert loop      -> moe_kernel
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <mutex>
@@ -24,6 +25,9 @@
 namespace sub1 {
 
 thread_local std::string g_err;
+thread_local const char *g_kernel = "";
+
+void note_kernel(const char *name) { g_kernel = name; }
 
 int fail(int code, const char *fmt, ...) {
   char buf[512];
@@ -34,6 +38,54 @@ int fail(int code, const char *fmt, ...) {
   g_err = buf;
   return code;
 }
+
+namespace {
+std::mutex g_fault_mutex;
+int32_t *g_fault_host = nullptr;     // pinned, mapped: kFaultWords words
+int32_t *g_fault_device = nullptr;   // the same words as the GPUs address them
+std::atomic<int64_t> g_wait_limit_us{250000};
+std::atomic<int> g_expect_extra{0};
+std::atomic<int> g_clock_khz{0};     // rate of wall_clock64 on the device first asked
+}  // namespace
+
+int fault_words(int32_t **device_ptr, bool may_allocate) {
+  std::lock_guard<std::mutex> lock(g_fault_mutex);
+  if (!g_fault_host) {
+    if (!may_allocate)
+      return fail(SUB1_ERR_INTERNAL, "call sub1_init() once before an entry point that does not allocate");
+    void *host = nullptr, *dev = nullptr;
+    HIP_TRY(hipHostMalloc(&host, kFaultWords * sizeof(int32_t),
+                          hipHostMallocPortable | hipHostMallocMapped));
+    for (int i = 0; i < kFaultWords; i++) static_cast<int32_t *>(host)[i] = 0;
+    HIP_TRY(hipHostGetDevicePointer(&dev, host, 0));
+    g_fault_host = static_cast<int32_t *>(host);
+    g_fault_device = static_cast<int32_t *>(dev);
+  }
+  *device_ptr = g_fault_device;
+  return SUB1_OK;
+}
+
+bool fault_flag_host(int word) {
+  std::lock_guard<std::mutex> lock(g_fault_mutex);
+  return g_fault_host && *const_cast<volatile int32_t *>(&g_fault_host[word]) != 0;
+}
+
+int64_t wait_limit_ticks() {
+  int khz = g_clock_khz.load();
+  if (khz <= 0) {
+    int device = 0, rate = 0;
+    if (hipGetDevice(&device) == hipSuccess &&
+        hipDeviceGetAttribute(&rate, hipDeviceAttributeWallClockRate, device) == hipSuccess &&
+        rate > 0)
+      khz = rate;
+    else
+      khz = 100000;   // 100 MHz
+    g_clock_khz.store(khz);
+  }
+  return g_wait_limit_us.load() * khz / 1000;
+}
+
+int expect_extra() { return g_expect_extra.load(); }
 
 }  // namespace sub1
 
@@ -81,6 +133,27 @@ __global__ void derive_slot_table_kernel(const int32_t *__restrict__ dec,
   }
   tab[e] = out;
   if (bad) atomicOr(unsupported, 1);
+}
+
+// The cached table is found by the address of the caller's dec.  To notice an
+// address that now holds something else, 64 words of dec at fixed scattered
+// places are kept beside the table and compared by one wavefront of every
+// launch; a difference sets the sticky kFaultDec flag (the host then drops its
+// cached tables).
+constexpr int kPrintWords = 64;
+__host__ __device__ constexpr int print_index(int i) {
+  return (i * 4099 + 7) & (SUB1_DEC_WORDS - 1);
+}
+
+__global__ void capture_print_kernel(const int32_t *__restrict__ dec, int32_t *__restrict__ print) {
+  if (threadIdx.x < kPrintWords) print[threadIdx.x] = dec[print_index(threadIdx.x)];
+}
+
+__device__ __forceinline__ void compare_print(const int32_t *__restrict__ dec,
+                                              const int32_t *__restrict__ print,
+                                              int32_t *sticky) {
+  if (threadIdx.x < kPrintWords && dec[print_index(threadIdx.x)] != print[threadIdx.x])
+    sub1::raise_fault(sticky, sub1::kFaultDec);
 }
 
 // ----------------------------------------------- activations in LDS --------
@@ -188,8 +261,10 @@ __global__ __launch_bounds__(kThreads) void matvec_kernel(
     const uint32_t *__restrict__ tab, const uint16_t *__restrict__ w_comp,
     const int32_t *__restrict__ row_off, const uint32_t *__restrict__ minmax,
     const uint16_t *__restrict__ x, uint16_t *__restrict__ y, int height, int width,
-    int64_t ldx, int64_t ldy) {
+    int64_t ldx, int64_t ldy, const int32_t *__restrict__ dec,
+    const int32_t *__restrict__ print, int32_t *sticky) {
   extern __shared__ float lds[];
+  if (blockIdx.x == 0 && blockIdx.y == 0) compare_print(dec, print, sticky);
   x += static_cast<int64_t>(blockIdx.y) * ldx;
   y += static_cast<int64_t>(blockIdx.y) * ldy;
   stage_activations<kThreads>(lds, x, width);
@@ -340,7 +415,11 @@ struct MoeArgs {
                   // id >= experts (treated as dropped), [4+t] wi tiles done for t
   int tokens, d_model, d_ff, experts;
   int wi_tiles, wo_tiles;  // per token
-  int spin_limit;
+  int wi_expect;           // wi tiles a wo tile waits for (wi_tiles outside tests)
+  int64_t wait_ticks;      // longest wait, in ticks of wall_clock64
+  int32_t *sticky;         // fault flags in pinned host memory
+  const int32_t *dec;      // the caller's table and the words kept of it
+  const int32_t *print;
 };
 
 constexpr int kCtrlHeader = 4;
@@ -351,6 +430,7 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
   __shared__ int s_ticket;
   const int n_wi = a.tokens * a.wi_tiles;
   const int n_all = n_wi + a.tokens * a.wo_tiles;
+  if (blockIdx.x == 0) compare_print(a.dec, a.print, a.sticky);
   for (;;) {
     __syncthreads();  // previous tile's readers of lds and s_ticket are done
     if (threadIdx.x == 0)
@@ -412,19 +492,9 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
         }
         continue;
       }
-      if (threadIdx.x == 0) {
-        int spins = 0;
-        while (__hip_atomic_load(&a.ctrl[kCtrlHeader + t], __ATOMIC_RELAXED,
-                                 __HIP_MEMORY_SCOPE_AGENT) < a.wi_tiles) {
-          if (++spins > a.spin_limit) {
-            __hip_atomic_fetch_add(&a.ctrl[1], 1, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-            break;
-          }
-          __builtin_amdgcn_s_sleep(2);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // once, when the count is there
-      }
+      if (threadIdx.x == 0)
+        sub1::bounded_wait(&a.ctrl[kCtrlHeader + t], a.wi_expect, a.wait_ticks, a.sticky,
+                           &a.ctrl[1]);
       __syncthreads();  // thread 0's acquire now covers the whole workgroup
       stage_activations<kThreads>(lds, a.h + static_cast<int64_t>(t) * a.d_ff, a.d_ff);
       __syncthreads();
@@ -452,38 +522,67 @@ __global__ void zero_i32_kernel(int32_t *p, int n) {
 struct TableSlot {
   int device;
   const int32_t *dec;
-  uint32_t *tab;
+  uint32_t *tab;          // kDictEntries table words, a flag word, kPrintWords of dec
+  const int32_t *print;
 };
 
 std::mutex g_tab_mutex;
 std::vector<TableSlot> g_tabs;
+bool g_purged = false;   // the tables were dropped for the kFaultDec flag now standing
 
-int slot_table_for(const int32_t *dec, hipStream_t stream, const uint32_t **out) {
+void drop_tables_locked(const int32_t *dec, bool all) {
+  for (size_t i = 0; i < g_tabs.size();) {
+    if (all || g_tabs[i].dec == dec) {
+      (void)hipFree(g_tabs[i].tab);   // synchronises: no launch is still reading it
+      g_tabs.erase(g_tabs.begin() + i);
+    } else {
+      i++;
+    }
+  }
+}
+
+// The compact table for `dec` on the current device, and the fault flags.  The
+// first call with an address derives the table (one allocation, two small
+// kernels, one synchronisation: not for a stream that is being captured).
+int slot_table_for(const int32_t *dec, hipStream_t stream, TableSlot *out, int32_t **sticky) {
   int device = 0;
   HIP_TRY(hipGetDevice(&device));
+  int rc = sub1::fault_words(sticky, true);
+  if (rc) return rc;
   std::lock_guard<std::mutex> lock(g_tab_mutex);
+  // a launch found other contents at a cached address: every cached table is
+  // suspect, derive them afresh (once per raised flag)
+  const bool flagged = sub1::fault_flag_host(sub1::kFaultDec);
+  if (flagged && !g_purged) {
+    drop_tables_locked(nullptr, true);
+    g_purged = true;
+  }
+  if (!flagged) g_purged = false;
   for (const TableSlot &s : g_tabs)
     if (s.device == device && s.dec == dec) {
-      *out = s.tab;
+      *out = s;
       return SUB1_OK;
     }
   uint32_t *tab = nullptr;
-  HIP_TRY(hipMalloc(&tab, (SUB1_DICT_ENTRIES + 1) * sizeof(uint32_t)));
+  HIP_TRY(hipMalloc(&tab, (SUB1_DICT_ENTRIES + 64 + kPrintWords) * sizeof(uint32_t)));
   int32_t *flag = reinterpret_cast<int32_t *>(tab + SUB1_DICT_ENTRIES);
+  int32_t *print = flag + 64;
   zero_i32_kernel<<<1, 64, 0, stream>>>(flag, 1);
   derive_slot_table_kernel<<<SUB1_DICT_ENTRIES / 256, 256, 0, stream>>>(dec, tab, flag);
-  HIP_TRY(hipGetLastError());
+  capture_print_kernel<<<1, 64, 0, stream>>>(dec, print);
   int32_t bad = 0;
-  HIP_TRY(hipMemcpyAsync(&bad, flag, sizeof bad, hipMemcpyDeviceToHost, stream));
-  HIP_TRY(hipStreamSynchronize(stream));
-  if (bad) {
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) e = hipMemcpyAsync(&bad, flag, sizeof bad, hipMemcpyDeviceToHost, stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  if (e != hipSuccess || bad) {
     (void)hipFree(tab);
+    if (e != hipSuccess) return fail(SUB1_ERR_HIP, "deriving the table: %s", hipGetErrorString(e));
     return fail(SUB1_ERR_SHAPE,
                 "dec holds an entry with a digit 3 or more than %d non-zero weights",
                 kSlots);
   }
-  g_tabs.push_back({device, dec, tab});
-  *out = tab;
+  g_tabs.push_back({device, dec, tab, print});
+  *out = g_tabs.back();
   return SUB1_OK;
 }
 
@@ -507,7 +606,9 @@ hipEvent_t g_ev_begin = nullptr, g_ev_end = nullptr;
 
 extern "C" const char *sub1_last_error(void) { return sub1::g_err.c_str(); }
 
-extern "C" int sub1_abi_version(void) { return 2; }
+extern "C" const char *sub1_last_kernel(void) { return sub1::g_kernel; }
+
+extern "C" int sub1_abi_version(void) { return 3; }
 
 extern "C" int sub1_matvec_tokens(const int32_t *dec, const int16_t *w_comp,
                                   const int32_t *row_off, const void *ter_minmax,
@@ -528,17 +629,20 @@ extern "C" int sub1_matvec_tokens(const int32_t *dec, const int16_t *w_comp,
       misaligned(w_comp, 2) || misaligned(x, 2) || misaligned(y, 2))
     return fail(SUB1_ERR_ALIGN, "sub1_matvec: misaligned pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const uint32_t *tab = nullptr;
-  int rc = slot_table_for(dec, s, &tab);
+  TableSlot slot;
+  int32_t *sticky = nullptr;
+  int rc = slot_table_for(dec, s, &slot, &sticky);
   if (rc) return rc;
+  const uint32_t *tab = slot.tab;
   size_t lds = lds_dwords_for_width(width) * sizeof(float);
   rc = allow_lds(matvec_kernel<kMatvecThreads>, lds);
   if (rc) return rc;
   dim3 grid((height + kMatvecThreads - 1) / kMatvecThreads, tokens);
+  sub1::note_kernel("matvec_kernel<256>");
   matvec_kernel<kMatvecThreads><<<grid, kMatvecThreads, lds, s>>>(
       tab, reinterpret_cast<const uint16_t *>(w_comp), row_off,
       static_cast<const uint32_t *>(ter_minmax), static_cast<const uint16_t *>(x),
-      static_cast<uint16_t *>(y), height, width, ldx, ldy);
+      static_cast<uint16_t *>(y), height, width, ldx, ldy, dec, slot.print, sticky);
   HIP_TRY(hipGetLastError());
   return SUB1_OK;
 }
@@ -635,12 +739,16 @@ extern "C" int sub1_moe_grouped(const sub1_moe_stack *st, const int32_t *token_e
     return fail(SUB1_ERR_ALIGN, "sub1_moe_grouped: misaligned pointer");
 
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const uint32_t *tab = nullptr;
-  int rc = slot_table_for(st->dec, s, &tab);
+  TableSlot slot;
+  int32_t *sticky = nullptr;
+  int rc = slot_table_for(st->dec, s, &slot, &sticky);
   if (rc) return rc;
 
   MoeArgs a;
-  a.tab = tab;
+  a.tab = slot.tab;
+  a.dec = st->dec;
+  a.print = slot.print;
+  a.sticky = sticky;
   a.w_comp = reinterpret_cast<const uint16_t *>(st->w_comp);
   a.wi_code_base = st->wi_code_base;
   a.wo_code_base = st->wo_code_base;
@@ -660,7 +768,8 @@ extern "C" int sub1_moe_grouped(const sub1_moe_stack *st, const int32_t *token_e
   a.experts = st->experts;
   a.wi_tiles = (st->d_ff + kMoeThreads - 1) / kMoeThreads;
   a.wo_tiles = (st->d_model + kMoeThreads - 1) / kMoeThreads;
-  a.spin_limit = 1 << 24;
+  a.wi_expect = a.wi_tiles + sub1::expect_extra();
+  a.wait_ticks = sub1::wait_limit_ticks();
   int64_t tiles = static_cast<int64_t>(tokens) * (a.wi_tiles + a.wo_tiles);
   if (tiles > INT32_MAX - (1 << 20))
     return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped: too many tiles");
@@ -680,8 +789,55 @@ extern "C" int sub1_moe_grouped(const sub1_moe_stack *st, const int32_t *token_e
 
   int nctrl = kCtrlHeader + tokens;
   zero_i32_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl);
+  sub1::note_kernel("moe_kernel<256>");
   moe_kernel<kMoeThreads><<<static_cast<unsigned>(grid), kMoeThreads, lds, s>>>(a);
   HIP_TRY(hipGetLastError());
+  return SUB1_OK;
+}
+
+extern "C" int sub1_fault_flags(int32_t *flags) {
+  if (!flags) return fail(SUB1_ERR_NULL, "sub1_fault_flags: NULL argument");
+  flags[0] = sub1::fault_flag_host(sub1::kFaultWait) ? 1 : 0;
+  flags[1] = sub1::fault_flag_host(sub1::kFaultDec) ? 1 : 0;
+  return SUB1_OK;
+}
+
+extern "C" const int32_t *sub1_fault_words_host(void) {
+  std::lock_guard<std::mutex> lock(sub1::g_fault_mutex);
+  return sub1::g_fault_host;
+}
+
+extern "C" int sub1_clear_faults(void) {
+  // a standing kFaultDec flag means a cached table is stale: drop them all, so
+  // that the calls after the reset derive theirs afresh
+  if (sub1::fault_flag_host(sub1::kFaultDec)) {
+    std::lock_guard<std::mutex> lock(g_tab_mutex);
+    drop_tables_locked(nullptr, true);
+  }
+  std::lock_guard<std::mutex> lock(sub1::g_fault_mutex);
+  if (sub1::g_fault_host)
+    for (int i = 0; i < sub1::kFaultWords; i++)
+      *const_cast<volatile int32_t *>(&sub1::g_fault_host[i]) = 0;
+  return SUB1_OK;
+}
+
+extern "C" int sub1_set_wait_limit_us(int64_t microseconds) {
+  if (microseconds < 1 || microseconds > 60000000)
+    return fail(SUB1_ERR_SHAPE, "sub1_set_wait_limit_us: %lld outside 1..60000000",
+                static_cast<long long>(microseconds));
+  sub1::g_wait_limit_us.store(microseconds);
+  return SUB1_OK;
+}
+
+extern "C" int sub1_test_overstate_wait(int extra) {
+  if (extra < 0) return fail(SUB1_ERR_SHAPE, "sub1_test_overstate_wait: negative count");
+  sub1::g_expect_extra.store(extra);
+  return SUB1_OK;
+}
+
+extern "C" int sub1_unregister_dec(const int32_t *dec) {
+  std::lock_guard<std::mutex> lock(g_tab_mutex);
+  drop_tables_locked(dec, dec == nullptr);
   return SUB1_OK;
 }
 

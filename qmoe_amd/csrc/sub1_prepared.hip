@@ -430,7 +430,9 @@ struct PreparedArgs {
   int xdwords;                   // LDS dwords reserved for the activations
   int hdwords;                   // fused kernel: LDS dwords of h (wo's activations)
   int tail_room;                 // persistent kernel: partial sums (groups x 64 lanes) LDS has room for
-  int spin_limit;
+  int wi_expect;                 // workgroups of a token's wi a wait expects (k[0].parts outside tests)
+  int64_t wait_ticks;            // longest wait between workgroups, ticks of wall_clock64
+  int32_t *sticky;               // fault flags in pinned host memory
 };
 
 // Activations in LDS: two dwords per physical column, A = (x, 0) and B = (0, x)
@@ -896,19 +898,9 @@ __device__ __forceinline__ void split_run(const PreparedArgs &a, const KindArgs 
 __device__ __forceinline__ void await_activations(const PreparedArgs &a, const KindArgs &k,
                                                   int kind, int t, uint32_t *xa) {
   if (kind == 1) {
-    if (threadIdx.x == 0) {
-      int spins = 0;
-      while (__hip_atomic_load(&a.ctrl[kCtrlHeader + t], __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT) < a.k[0].parts) {
-        if (++spins > a.spin_limit) {
-          __hip_atomic_fetch_add(&a.ctrl[1], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          break;
-        }
-        __builtin_amdgcn_s_sleep(2);
-      }
-      // one acquire when the count is there, not one per look at it
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    }
+    if (threadIdx.x == 0)
+      sub1::bounded_wait(&a.ctrl[kCtrlHeader + t], a.wi_expect, a.wait_ticks, a.sticky,
+                         &a.ctrl[1]);
     __syncthreads();
   }
   const uint16_t *src = kind ? a.h + static_cast<int64_t>(t) * k.width
@@ -1568,19 +1560,10 @@ __global__ __launch_bounds__(kMaxThreads) void matvec_group_kernel(PreparedArgs 
 
 // ------------------------------------------------------------ host side --
 
-std::mutex g_mutex;
-std::vector<std::pair<int, const int32_t *>> g_checked_dec;   // (device, dec) known to be the fixed table
-
 // The prepare kernels read dec as the fixed dictionary's table (symbols 0..2,
-// unused digits zero): refuse any other.
+// unused digits zero): refuse any other.  Compared in full on every call (a
+// 512 KB copy and a synchronisation; preparing is a load-time step).
 int check_dec(const int32_t *dec, hipStream_t stream) {
-  int device = 0;
-  HIP_TRY(hipGetDevice(&device));
-  {
-    std::lock_guard<std::mutex> lock(g_mutex);
-    for (const auto &p : g_checked_dec)
-      if (p.first == device && p.second == dec) return SUB1_OK;
-  }
   std::vector<int32_t> want(SUB1_DEC_WORDS), got(SUB1_DEC_WORDS);
   int rc = sub1_build_tables(want.data(), nullptr);
   if (rc) return fail(rc, "sub1_build_tables failed");
@@ -1590,8 +1573,6 @@ int check_dec(const int32_t *dec, hipStream_t stream) {
   if (std::memcmp(want.data(), got.data(), want.size() * sizeof(int32_t)) != 0)
     return fail(SUB1_ERR_SHAPE,
                 "sub1_moe_prepare: dec is not the fixed dictionary; use sub1_moe_grouped");
-  std::lock_guard<std::mutex> lock(g_mutex);
-  g_checked_dec.push_back({device, dec});
   return SUB1_OK;
 }
 
@@ -1875,7 +1856,7 @@ double part_passes(int slices, int waves, int groups_max) {
 // keeps the fault counts of the first).
 int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *x, int64_t ldx,
                     void *y, int64_t ldy, int tokens, void *workspace, int64_t workspace_bytes,
-                    hipStream_t s, const char *who, int piece = 0) {
+                    hipStream_t s, const char *who, int piece = 0, bool may_allocate = true) {
   if (!p.meta || !p.codes || !x || !y) return fail(SUB1_ERR_NULL, "%s: NULL argument", who);
   if (p.kinds == 2 && !token_matrix) return fail(SUB1_ERR_NULL, "%s: NULL token_expert", who);
   if (tokens < 0 || tokens > (1 << 20))
@@ -1944,7 +1925,11 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   a.xdwords = activation_dwords(wmax);
   a.hdwords = 0;
   a.tail_room = 0;
-  a.spin_limit = 1 << 24;
+  a.wait_ticks = sub1::wait_limit_ticks();
+  {
+    const int rc = sub1::fault_words(&a.sticky, may_allocate);
+    if (rc) return rc;
+  }
   const size_t lds_limit = 160 * 1024 - 64;
   const size_t lds_base = static_cast<size_t>(a.xdwords) * 4;
   if (lds_base > lds_limit) return fail(SUB1_ERR_SHAPE, "%s: width %d does not fit LDS", who, wmax);
@@ -2008,6 +1993,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     const void *fn = reinterpret_cast<const void *>(matvec_group_kernel);
     HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(lds_base)));
+    sub1::note_kernel("matvec_group_kernel");
     matvec_group_kernel<<<static_cast<unsigned>(tiles < cus ? tiles : cus), 64 * waves, lds_base,
                           s>>>(a);
     HIP_TRY(hipGetLastError());
@@ -2115,11 +2101,11 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
         const uint16_t *xs = static_cast<const uint16_t *>(x);
         uint16_t *ys = static_cast<uint16_t *>(y);
         const int rc = launch_prepared(p, token_matrix, xs, ldx, ys, ldy, whole, workspace,
-                                       workspace_bytes, s, who, 1);
+                                       workspace_bytes, s, who, 1, may_allocate);
         if (rc) return rc;
         return launch_prepared(p, token_matrix + whole, xs + static_cast<int64_t>(whole) * ldx, ldx,
                                ys + static_cast<int64_t>(whole) * ldy, ldy, tokens - whole,
-                               workspace, workspace_bytes, s, who, 2);
+                               workspace, workspace_bytes, s, who, 2, may_allocate);
       }
     }
     if (!shared_parts && fused_us < cut_us) {
@@ -2136,12 +2122,14 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
       a.k[i].split = 1;
     }
     a.tail_room = (waves / 2) * std::max(a.k[0].groups_max, a.k[1].groups_max);
+    a.wi_expect = a.k[0].parts + sub1::expect_extra();
     const size_t lds_shared = lds_base + static_cast<size_t>(a.tail_room) * 256;
     const void *fn = reinterpret_cast<const void *>(moe_prepared_shared_kernel);
     HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(lds_shared)));
     const int nctrl = kCtrlHeader + tokens;
     zero_words_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl, piece == 2);
+    sub1::note_kernel("moe_prepared_shared_kernel");
     moe_prepared_shared_kernel<<<tokens * shared_parts, 64 * waves, lds_shared, s>>>(a);
     HIP_TRY(hipGetLastError());
     return SUB1_OK;
@@ -2192,6 +2180,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
       a.groups = groups;
     }
     const int grid = tokens < cus * per_cu ? tokens : cus * per_cu;
+    sub1::note_kernel(grouped ? "moe_prepared_fused_kernel<true>" : "moe_prepared_fused_kernel<false>");
     if (grouped)
       moe_prepared_fused_kernel<true><<<grid, 64 * fw, lds_fused, s>>>(a);
     else
@@ -2213,6 +2202,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
       lds_tail = 0;
   }
   const size_t lds = lds_base + lds_partials + lds_tail;
+  a.wi_expect = a.k[0].parts + sub1::expect_extra();
   // Batches too small to occupy the GPU with a wavefront per slice go to the
   // latency kernel, everything else to the persistent one; either way at most
   // a workgroup per compute unit (16 wavefronts of 72 to 80 registers each).
@@ -2226,9 +2216,11 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   }
   if (small) {
     const int64_t grid = tiles < cus ? tiles : cus;
+    sub1::note_kernel("moe_prepared_small_kernel");
     moe_prepared_small_kernel<<<static_cast<unsigned>(grid), 64 * waves, lds, s>>>(a);
   } else {
     const int64_t grid = tiles < cus ? tiles : cus;
+    sub1::note_kernel("moe_prepared_kernel");
     moe_prepared_kernel<<<static_cast<unsigned>(grid), 64 * waves, lds, s>>>(a);
   }
   HIP_TRY(hipGetLastError());
@@ -2275,6 +2267,7 @@ int check_matrix_set(const sub1_matrix_set *ms, const char *who) {
 }  // namespace
 
 // ================================================================ C ABI =====
+
 
 extern "C" int64_t sub1_moe_prepared_meta_bytes(int experts, int d_model, int d_ff) {
   if (experts < 1 || d_model < 1 || d_ff < 1) return 0;
@@ -2344,6 +2337,11 @@ bool bad_dims(int count, int h, int w) {
   return count < 1 || h < 1 || w < 1 || h > 65534 || w > SUB1_PREPARED_MAX_WIDTH;
 }
 }  // namespace
+
+extern "C" int sub1_init(void) {
+  int32_t *sticky = nullptr;
+  return sub1::fault_words(&sticky, true);
+}
 
 extern "C" int sub1_moe_prepare_codes(const sub1_moe_stack *st, const sub1_moe_prepared *p,
                                       void *stream) {

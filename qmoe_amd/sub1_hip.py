@@ -18,6 +18,9 @@ from . import _lib
 
 DICT_ENTRIES = _lib.DICT_ENTRIES
 PREPARED_MAX_WIDTH = _lib.PREPARED_MAX_WIDTH
+Sub1Fault = _lib.Sub1Fault
+check_faults = _lib.check_faults
+clear_faults = _lib.clear_faults
 
 
 def _stream():
@@ -75,6 +78,7 @@ def sub1matvec(dec, w_comp, row_off, ter_minmax, x, y):
     """y += W x for one compressed matrix; height = y.numel(), width =
     x.numel() (reference sub1_cuda_kernel.cu:78-79).  Any shape, in place."""
     dev = dec.device if isinstance(dec, torch.Tensor) else None
+    _lib.check_faults()
     height, width = y.numel(), x.numel()
     args = [
         _need(dec, torch.int32, 'dec', numel=_lib.DEC_WORDS),
@@ -174,7 +178,7 @@ class ExpertStack:
             _need(wi_minmax, torch.bfloat16, 'wi_minmax', dev, numel=experts * 2 * d_ff),
             _need(wo_minmax, torch.bfloat16, 'wo_minmax', dev, numel=experts * 2 * d_model),
             experts, d_model, d_ff)
-        self._ws = None
+        self._ws = {}
 
     @classmethod
     def from_layers(cls, dec, wi_layers, wo_layers):
@@ -199,16 +203,26 @@ class ExpertStack:
                 + 2 * self.wo_minmax.numel())
 
     def workspace(self, tokens):
+        """The launch's scratch memory (control words and h), one buffer per
+        stream: launches on different streams may run at once, launches on one
+        stream run in order and share theirs.  A buffer that has to grow is
+        replaced; the old one goes back to torch's allocator, which hands it
+        out again only in the order of the stream it was allocated on."""
         need = _lib.load().sub1_moe_workspace_bytes(tokens, self.d_ff)
-        if self._ws is None or self._ws.numel() < need:
-            self._ws = torch.empty(need, dtype=torch.uint8, device=self.device)
-        return self._ws
+        key = _stream().value
+        ws = self._ws.get(key)
+        if ws is None or ws.numel() < need:
+            with _on_device(self.device):
+                ws = torch.empty(need, dtype=torch.uint8, device=self.device)
+            self._ws[key] = ws
+        return ws
 
     def forward(self, x, token_expert, y=None):
         """y[t] = wo_e(relu(wi_e(x[t]))), e = token_expert[t]; tokens with a
         negative expert keep their input.  x bf16 [T, d_model], token_expert
         int32 [T]."""
         dev = self.device
+        _lib.check_faults()       # what earlier launches reported (host memory, no sync)
         p_x = _need(x, torch.bfloat16, 'x', dev, dim=2)
         tokens = x.shape[0]
         if x.shape[1] != self.d_model:
@@ -237,11 +251,15 @@ class ExpertStack:
         return PreparedStack(self)
 
     def launch_faults(self, tokens):
-        """(waits inside the last forward that gave up, tokens whose expert id
-        was >= experts and were passed through); both 0 when all is well.
-        Reads the control words of the workspace, synchronising."""
+        """(waits inside the last forward on this stream that gave up, tokens
+        whose expert id was >= experts and were passed through); both 0 when
+        all is well.  Reads the control words of the workspace, synchronising.
+        A wait that gave up is also reported, sticky, by check_faults() and by
+        the next forward()."""
         ctrl = self.workspace(tokens)[:16].view(torch.int32).tolist()
         return ctrl[1], ctrl[2]
+
+    check_faults = staticmethod(_lib.check_faults)
 
 
 class PreparedStack:
@@ -271,16 +289,26 @@ class PreparedStack:
             self._c.codes = self.codes.data_ptr()
             _lib.check(lib.sub1_moe_prepare_codes(ctypes.byref(stack._c), ctypes.byref(self._c),
                                                   _stream()))
-        self._ws = None
+        self._ws = {}
 
     def workspace(self, tokens):
+        """The launch's scratch memory (control words and h), one buffer per
+        stream: launches on different streams may run at once, launches on one
+        stream run in order and share theirs.  A buffer that has to grow is
+        replaced; the old one goes back to torch's allocator, which hands it
+        out again only in the order of the stream it was allocated on."""
         need = _lib.load().sub1_moe_workspace_bytes(tokens, self.d_ff)
-        if self._ws is None or self._ws.numel() < need:
-            self._ws = torch.empty(need, dtype=torch.uint8, device=self.device)
-        return self._ws
+        key = _stream().value
+        ws = self._ws.get(key)
+        if ws is None or ws.numel() < need:
+            with _on_device(self.device):
+                ws = torch.empty(need, dtype=torch.uint8, device=self.device)
+            self._ws[key] = ws
+        return ws
 
     def forward(self, x, token_expert, y=None):
         dev = self.device
+        _lib.check_faults()       # what earlier launches reported (host memory, no sync)
         p_x = _need(x, torch.bfloat16, 'x', dev, dim=2)
         tokens = x.shape[0]
         if x.shape[1] != self.d_model:
@@ -299,8 +327,11 @@ class PreparedStack:
         return y
 
     def launch_faults(self, tokens):
+        """As ExpertStack.launch_faults."""
         ctrl = self.workspace(tokens)[:16].view(torch.int32).tolist()
         return ctrl[1], ctrl[2]
+
+    check_faults = staticmethod(_lib.check_faults)
 
     def decode(self, expert, projection):
         """uint8 [rows, width]: the symbols of one matrix (projection 0 = wi,
