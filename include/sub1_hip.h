@@ -240,6 +240,26 @@ int sub1_moe_prepared_decode(const sub1_moe_prepared *prepared, int expert, int 
                              void *tern_out, void *stream);
 
 /*
+ * sub1_moe_grouped_prepared without the workspace argument, for callers that
+ * cannot allocate device memory: code under a HIP graph capture, tight serving
+ * loops, harnesses that forbid it.  No counterpart in the reference (whose
+ * kernels need no scratch memory).  The control words and h live in a static
+ * device array of SUB1_STATIC_SCRATCH_BYTES that every GPU the library runs on
+ * holds until the process ends; the call allocates nothing, on the device or
+ * pinned (so sub1_init() must have run once in the process), and refuses a
+ * batch whose sub1_moe_workspace_bytes(tokens, d_ff) exceeds the array (64
+ * tokens of a Switch-c-2048 layer fit).  Same kernels and same results as
+ * sub1_moe_grouped_prepared.  All calls on one GPU share the one array: two
+ * that overlap there (different streams, different threads) race; calls on one
+ * stream run in order and are safe.
+ */
+#define SUB1_STATIC_SCRATCH_BYTES (1 << 20)
+
+int sub1_moe_grouped_prepared_static(const sub1_moe_prepared *prepared,
+                                     const int32_t *token_expert, const void *x, void *y,
+                                     int tokens, void *stream);
+
+/*
  * The same preparation for plain products: `count` matrices of one shape
  * (count = 1: one Sub1Linear), then
  *     y[t, :] += W_m x[t, :],   m = token_matrix[t]  (NULL: matrix 0 for all),
@@ -316,8 +336,10 @@ int sub1_timing_end(void *stream, double *elapsed_us);
  *   sub1_init()               allocates the flag words (pinned host memory) and
  *                             prepares the current device; the other entry
  *                             points do this themselves on first use, so it is
- *                             only needed before a stream capture.  Safe to
- *                             call again.
+ *                             only needed before a stream capture or
+ *                             sub1_moe_grouped_prepared_static.  Safe to call
+ *                             again; call it once with each device current
+ *                             that will use the static scratch.
  *   sub1_fault_flags(f)       f[0] = a wait gave up, f[1] = dec changed; read
  *                             from host memory, no synchronisation: a flag is
  *                             seen once the launch that set it has got that far.

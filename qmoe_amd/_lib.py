@@ -68,6 +68,8 @@ PROTOTYPES = {
                                       _vp]),
     'sub1_moe_grouped_prepared': (_int, [ctypes.POINTER(MoePrepared), _vp, _vp, _vp, _int,
                                          _vp, _i64, _vp]),
+    'sub1_moe_grouped_prepared_static': (_int, [ctypes.POINTER(MoePrepared), _vp, _vp, _vp, _int,
+                                                _vp]),
     'sub1_moe_prepared_decode': (_int, [ctypes.POINTER(MoePrepared), _int, _int, _vp, _vp]),
     'sub1_matrix_prepared_meta_bytes': (_i64, [_int, _int, _int]),
     'sub1_matrix_prepare_layout': (_int, [ctypes.POINTER(MatrixSet), _vp, _i64,

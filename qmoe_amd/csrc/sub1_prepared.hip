@@ -2338,9 +2338,70 @@ bool bad_dims(int count, int h, int w) {
 }
 }  // namespace
 
+// ------------------------------------------------ launch without allocating --
+//
+// Scratch memory of sub1_moe_grouped_prepared_static: what the workspace
+// argument of sub1_moe_grouped_prepared brings in (control words, then h), held
+// by every GPU the library runs on until the process ends.  The name is a
+// host-side stand-in, not a device address: host code uses the per-device
+// address that hipGetSymbolAddress returns, never the name.
+static __device__ __align__(256) unsigned char scratch[SUB1_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};   // each GPU's own copy of `scratch`
+
+// The current device's address of the scratch array (resolved once per device,
+// with that device current; no allocation).
+int scratch_of_current_device(void **out) {
+  int device = 0;
+  HIP_TRY(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices)
+    return fail(SUB1_ERR_SHAPE, "device %d: the static scratch serves devices 0..%d", device,
+                kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[device]) {
+    void *ptr = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return fail(SUB1_ERR_HIP, "hipGetSymbolAddress returned no address for the scratch");
+    g_scratch_ptr[device] = ptr;
+  }
+  *out = g_scratch_ptr[device];
+  return SUB1_OK;
+}
+}  // namespace
+
 extern "C" int sub1_init(void) {
   int32_t *sticky = nullptr;
-  return sub1::fault_words(&sticky, true);
+  int rc = sub1::fault_words(&sticky, true);
+  if (rc) return rc;
+  void *ws = nullptr;
+  return scratch_of_current_device(&ws);
+}
+
+extern "C" int sub1_moe_grouped_prepared_static(const sub1_moe_prepared *p,
+                                                const int32_t *token_expert, const void *x,
+                                                void *y, int tokens, void *stream) {
+  const char *who = "sub1_moe_grouped_prepared_static";
+  if (!p) return fail(SUB1_ERR_NULL, "%s: NULL argument", who);
+  if (tokens == 0) return SUB1_OK;
+  if (bad_dims(p->experts, p->d_ff, p->d_model) || bad_dims(p->experts, p->d_model, p->d_ff))
+    return fail(SUB1_ERR_SHAPE, "%s: experts %d d_model %d d_ff %d", who, p->experts, p->d_model,
+                p->d_ff);
+  if (tokens < 0) return fail(SUB1_ERR_SHAPE, "%s: tokens %d", who, tokens);
+  const int64_t need = sub1_moe_workspace_bytes(tokens, p->d_ff);
+  if (need > SUB1_STATIC_SCRATCH_BYTES)
+    return fail(SUB1_ERR_SHAPE,
+                "%s: %d tokens of d_ff %d need %lld bytes of scratch, the static buffer holds "
+                "%d; use sub1_moe_grouped_prepared with a workspace",
+                who, tokens, p->d_ff, static_cast<long long>(need), SUB1_STATIC_SCRATCH_BYTES);
+  void *ws = nullptr;
+  const int rc = scratch_of_current_device(&ws);
+  if (rc) return rc;
+  return launch_prepared(from_moe(p), token_expert, x, p->d_model, y, p->d_model, tokens, ws,
+                         SUB1_STATIC_SCRATCH_BYTES, static_cast<hipStream_t>(stream), who, 0,
+                         /*may_allocate=*/false);
 }
 
 extern "C" int sub1_moe_prepare_codes(const sub1_moe_stack *st, const sub1_moe_prepared *p,

@@ -1,0 +1,69 @@
+"""sub1_moe_grouped_prepared_static: the expert-layer launch whose scratch
+memory (control words and h) is a static device array instead of a workspace
+argument, for callers that cannot allocate.  Called through the C ABI, its
+output must equal sub1_moe_grouped_prepared's bit for bit, on two calls in a
+row, the second on a smaller batch (the array keeps the first call's
+contents); batches beyond the array are refused."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import sub1_oracle as so
+from test_gpu_parity import bf16_dev, bits_host, small_stack
+
+pytestmark = pytest.mark.gpu
+
+
+def test_static_scratch_launch_equals_workspace_launch(oracle):
+    from qmoe_amd import _lib, sub1
+    assert torch.cuda.is_available() and sub1.DEC
+    lib = _lib.load()
+    _lib.check(lib.sub1_init())
+    experts, d_model, d_ff = 4, 768, 3072
+    stack, wi, wo = small_stack(oracle, experts, d_model, d_ff, 0.9, seed=1500)
+    prep = stack.prepare()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def both(route, seed):
+        tokens = len(route)
+        xs = np.stack([so.synthetic_activation(d_model, seed + i) for i in range(tokens)])
+        x = bf16_dev(xs)
+        te = torch.tensor(route, dtype=torch.int32, device='cuda')
+        want = prep.forward(x, te)                       # sub1_moe_grouped_prepared
+        got = torch.full_like(x, 7.0)
+        _lib.check(lib.sub1_moe_grouped_prepared_static(
+            ctypes.byref(prep._c), te.data_ptr(), x.data_ptr(), got.data_ptr(), tokens, stream))
+        torch.cuda.synchronize()
+        return xs, bits_host(got), bits_host(want)
+
+    # the first call: 40 tokens, some dropped, one with an expert that does not exist
+    route = [(3 * i) % experts for i in range(40)]
+    route[5], route[17], route[30] = -1, experts + 1, -1
+    xs, got, want = both(route, 1600)
+    assert np.array_equal(got, want)
+    for i in (0, 7, 39):
+        ref, _ = oracle.expert_ffn(wi[route[i]], wo[route[i]], xs[i], order=2)
+        assert np.array_equal(got[i], ref)
+    for i in (5, 17, 30):
+        assert np.array_equal(got[i], xs[i])
+    # the second, smaller, on the same array
+    route = [2, 0, 3]
+    xs, got, want = both(route, 1700)
+    assert np.array_equal(got, want)
+    for i, e in enumerate(route):
+        ref, _ = oracle.expert_ffn(wi[e], wo[e], xs[i], order=2)
+        assert np.array_equal(got[i], ref)
+    _lib.check_faults()
+
+    # more scratch than the array holds: refused, with the size in the message
+    tokens = 200
+    assert lib.sub1_moe_workspace_bytes(tokens, d_ff) > (1 << 20)
+    x = torch.zeros((tokens, d_model), dtype=torch.bfloat16, device='cuda')
+    te = torch.zeros(tokens, dtype=torch.int32, device='cuda')
+    rc = lib.sub1_moe_grouped_prepared_static(ctypes.byref(prep._c), te.data_ptr(), x.data_ptr(),
+                                              x.data_ptr(), tokens, stream)
+    assert rc == -2 and b'static buffer holds' in lib.sub1_last_error()
+    assert lib.sub1_moe_grouped_prepared_static(ctypes.byref(prep._c), te.data_ptr(), x.data_ptr(),
+                                                x.data_ptr(), 0, stream) == 0
