@@ -60,7 +60,7 @@ constexpr int kMaxStep = 127;        // the largest entry
 constexpr int kRing = 4;             // chunks in flight per lane (2 KB per wavefront)
 constexpr int kGroupChunks = 8;      // chunks (72 entries) per partial sum, a multiple of kRing
 constexpr int kSplitRing = 8;        // chunks in flight per lane where wavefronts share a slice
-constexpr int kMaxRowChunks = 4096;  // chunks per row the row ordering can count
+constexpr int kMaxRowEntries = 16383; // entries per row the row ordering can count (widths to 12288)
 constexpr int kCtrlHeader = 4;       // ctrl[0] ticket, [1] wait-limit hits, [2] bad expert ids
 
 // ------------------------------------------------------------- meta layout --
@@ -69,8 +69,8 @@ constexpr int kCtrlHeader = 4;       // ctrl[0] ticket, [1] wait-limit hits, [2]
 // Kind 0 = wi (rows d_ff, width d_model), kind 1 = wo.
 struct KindMeta {
   int64_t slice_base;   // u32 [E*S] (+1): this kind's part of the scanned counts
-  int64_t slice_nch;    // u16 [E*S]
-  int64_t row_chunks;   // u16 [E*H]: chunks of every row, in the matrix's own row order
+  int64_t slice_len;    // u16 [E*S]: entries of the slice's longest row
+  int64_t row_len;      // u16 [E*H]: entries of every row, in the matrix's own row order
   int64_t row_idx;      // u16 [E*S*64]
   int64_t minmax;       // u32 [E*S*64]
   int slices;           // S
@@ -109,8 +109,8 @@ MetaLayout meta_layout(int experts, int kinds, const int height[2], const int wi
     int64_t es = static_cast<int64_t>(experts) * k.slices;
     first[i] = nslices;
     nslices += es;
-    k.slice_nch = take(es * 2);
-    k.row_chunks = take(static_cast<int64_t>(experts) * height[i] * 2);
+    k.slice_len = take(es * 2);
+    k.row_len = take(static_cast<int64_t>(experts) * height[i] * 2);
     k.row_idx = take(es * 64 * 2);
     k.minmax = take(es * 64 * 4);
   }
@@ -158,6 +158,12 @@ __device__ __forceinline__ int for_each_nonzero(const uint16_t *codes, int n,
   }
   return col;
 }
+
+// A slice is as long as its longest row, counted in ENTRIES; its chunks, and how
+// many entries of the last one are walked (1..9; the rest of that chunk is
+// padding nobody reads).
+__host__ __device__ constexpr int chunks_of(int len) { return (len + kFields - 1) / kFields; }
+__host__ __device__ constexpr int last_entries_of(int len) { return len - kFields * (chunks_of(len) - 1); }
 
 // Positions.  The kernels keep the activations in LDS by physical column: real
 // column c is physical column q = c + c/16 + 1, so that every 17th physical
@@ -211,11 +217,12 @@ __device__ __forceinline__ const uint16_t *row_codes(const uint16_t *src, const 
   return src + (code_base ? code_base[e] : 0) + ro[r];   // one matrix: no base array
 }
 
-// One thread per row: how many chunks its entries fill.
+// One thread per row: how many entries its non-zeros take (the step onto a zero
+// column that a padded row makes after them is not counted: it fits the padding).
 __global__ __launch_bounds__(256) void count_entries_kernel(
     const uint16_t *__restrict__ src, const int64_t *__restrict__ code_base,
     const int32_t *__restrict__ row_off_all, const int32_t *__restrict__ dec,
-    uint16_t *__restrict__ row_chunks, int32_t *__restrict__ status, int height, int width,
+    uint16_t *__restrict__ row_len, int32_t *__restrict__ status, int height, int width,
     int64_t rows_total) {
   const int64_t g = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (g >= rows_total) return;
@@ -228,40 +235,43 @@ __global__ __launch_bounds__(256) void count_entries_kernel(
   EntryWriter wr;
   const int covered =
       for_each_nonzero(codes, n, dec, width, [&](int col, int sym) { wr.nonzero(col, sym, emit); });
-  wr.park(emit);
   // a row's codes cover its width rounded up to a whole pair, exactly
   if (covered != ((width + 1) & ~1)) atomicAdd(&status[0], 1);
-  row_chunks[g] = static_cast<uint16_t>((entries + kFields - 1) / kFields);
+  row_len[g] = static_cast<uint16_t>(min(entries, kMaxRowEntries));
 }
 
-// One workgroup per matrix: order the rows by chunk count, longest first, and
+// One workgroup per matrix: order the rows by entry count, longest first, and
 // describe the 64-row slices.  The order is a counting sort carried out by one
-// thread, so it is the same on every run.
+// thread, so it is the same on every run.  Dynamic LDS: the histogram
+// (kMaxRowEntries + 2 counters), then the entry count of the first row of up to
+// 1024 slices.
+constexpr size_t kOrderRowsLds = (kMaxRowEntries + 2 + 1024) * sizeof(int);
 __global__ __launch_bounds__(256) void order_rows_kernel(
-    const uint16_t *__restrict__ row_chunks_all, const uint32_t *__restrict__ minmax_all,
+    const uint16_t *__restrict__ row_len_all, const uint32_t *__restrict__ minmax_all,
     uint16_t *__restrict__ row_idx, uint32_t *__restrict__ minmax_sorted,
-    uint16_t *__restrict__ slice_nch, int32_t *__restrict__ counts,
+    uint16_t *__restrict__ slice_len, int32_t *__restrict__ counts,
     int32_t *__restrict__ status, int height, int slices, int kind) {
-  __shared__ int hist[kMaxRowChunks + 2];
-  __shared__ int first_len[1024];   // chunk count of the first row of up to 1024 slices
+  extern __shared__ int order_lds[];
+  int *hist = order_lds;
+  int *first_len = order_lds + kMaxRowEntries + 2;
   const int e = blockIdx.x;
-  const uint16_t *rc = row_chunks_all + static_cast<int64_t>(e) * height;
+  const uint16_t *rl = row_len_all + static_cast<int64_t>(e) * height;
   const uint32_t *mm = minmax_all + static_cast<int64_t>(e) * height;
   const int64_t lane0 = static_cast<int64_t>(e) * slices * 64;
-  for (int i = threadIdx.x; i < kMaxRowChunks + 2; i += blockDim.x) hist[i] = 0;
+  for (int i = threadIdx.x; i < kMaxRowEntries + 2; i += blockDim.x) hist[i] = 0;
   __syncthreads();
   for (int r = threadIdx.x; r < height; r += blockDim.x)
-    atomicAdd(&hist[min(static_cast<int>(rc[r]), kMaxRowChunks)], 1);
+    atomicAdd(&hist[min(static_cast<int>(rl[r]), kMaxRowEntries)], 1);
   __syncthreads();
   if (threadIdx.x == 0) {
     int run = 0;  // rows with a larger count come first
-    for (int len = kMaxRowChunks; len >= 0; len--) {
+    for (int len = kMaxRowEntries; len >= 0; len--) {
       int n = hist[len];
       hist[len] = run;
       run += n;
     }
     for (int r = 0; r < height; r++) {
-      const int len = min(static_cast<int>(rc[r]), kMaxRowChunks);
+      const int len = min(static_cast<int>(rl[r]), kMaxRowEntries);
       int p = hist[len]++;
       row_idx[lane0 + p] = static_cast<uint16_t>(r);
       minmax_sorted[lane0 + p] = mm[r];
@@ -274,13 +284,13 @@ __global__ __launch_bounds__(256) void order_rows_kernel(
   }
   __syncthreads();
   for (int s = threadIdx.x; s < slices; s += blockDim.x) {
-    // a slice is as long as its first row, and at least one chunk
-    int nch = s < 1024 ? first_len[s] : static_cast<int>(rc[row_idx[lane0 + 64 * s]]);
-    nch = max(nch, 1);
+    // a slice is as long as its first row, and at least one entry
+    int len = s < 1024 ? first_len[s] : static_cast<int>(rl[row_idx[lane0 + 64 * s]]);
+    len = max(len, 1);
     int64_t g = static_cast<int64_t>(e) * slices + s;
-    slice_nch[g] = static_cast<uint16_t>(nch);
-    counts[g + 1] = nch;
-    atomicMax(&status[1 + kind], nch);
+    slice_len[g] = static_cast<uint16_t>(len);
+    counts[g + 1] = chunks_of(len);
+    atomicMax(&status[1 + kind], chunks_of(len));
   }
 }
 
@@ -319,12 +329,14 @@ __device__ __forceinline__ int64_t checkpoint_entry(uint32_t slice_base, int64_t
 }
 
 // One thread per lane of every slice: the row's entries into the interleaved
-// stream, nine to a chunk, zero entries up to the slice's chunk count, and the
-// row's position at the start of every group of chunks into the checkpoints.
+// stream, nine to a chunk; a row shorter than its slice then steps onto the
+// next zero column and stays there (steps of 0) to the end of the slice's last
+// chunk; and the row's position at the start of every group of chunks into the
+// checkpoints.
 __global__ __launch_bounds__(256) void emit_entries_kernel(
     const uint16_t *__restrict__ src, const int64_t *__restrict__ code_base,
     const int32_t *__restrict__ row_off_all, const int32_t *__restrict__ dec,
-    const uint32_t *__restrict__ slice_base, const uint16_t *__restrict__ slice_nch,
+    const uint32_t *__restrict__ slice_base, const uint16_t *__restrict__ slice_len,
     const uint16_t *__restrict__ row_idx, uint2 *__restrict__ dst, uint16_t *__restrict__ ckpt,
     int height, int width, int slices, int64_t first_slice, int64_t lanes_total) {
   const int64_t gl = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -334,7 +346,8 @@ __global__ __launch_bounds__(256) void emit_entries_kernel(
   const int e = static_cast<int>(slice / slices);
   const int ridx = row_idx[gl];
   const uint32_t base = slice_base[slice];
-  const int nch = slice_nch[slice];
+  const int len = slice_len[slice];
+  const int nch = chunks_of(len);
   uint2 *d = dst + static_cast<int64_t>(base) * 64 + ln;
   uint16_t *ck = ckpt + checkpoint_entry(base, first_slice + slice) * 64 + ln;
   int c = 0, q = 0;
@@ -355,7 +368,7 @@ __global__ __launch_bounds__(256) void emit_entries_kernel(
     int n;
     const uint16_t *codes = row_codes(src, code_base, row_off_all, e, ridx, height, width, n);
     for_each_nonzero(codes, n, dec, width, [&](int col, int sym) { wr.nonzero(col, sym, emit); });
-    wr.park(emit);
+    if (c * kFields + q < len) wr.park(emit);   // padding follows: it must read zeros
   }
   while (c < nch) emit(0, wr.j);
 }
@@ -364,7 +377,7 @@ __global__ __launch_bounds__(256) void emit_entries_kernel(
 // = 1 or 2 at every entry that stands on an activation; out is zero before.
 __global__ __launch_bounds__(256) void decode_entries_kernel(
     const uint2 *__restrict__ stream, const uint32_t *__restrict__ slice_base,
-    const uint16_t *__restrict__ slice_nch, const uint16_t *__restrict__ row_idx,
+    const uint16_t *__restrict__ slice_len, const uint16_t *__restrict__ row_idx,
     uint8_t *__restrict__ out, int64_t first, int slices, int width) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= slices * 64) return;
@@ -372,12 +385,13 @@ __global__ __launch_bounds__(256) void decode_entries_kernel(
   const int ridx = row_idx[sl * 64 + (t & 63)];
   if (ridx == 0xffff) return;
   const uint2 *p = stream + static_cast<int64_t>(slice_base[sl]) * 64 + (t & 63);
-  const int nch = slice_nch[sl];
+  const int len = slice_len[sl];
+  const int nch = chunks_of(len);
   int j = 0;
   for (int c = 0; c < nch; c++) {
     const uint2 cw = p[c * 64];
     const unsigned long long w = (static_cast<unsigned long long>(cw.y) << 32) | cw.x;
-    for (int q = 0; q < kFields; q++) {
+    for (int q = 0; q < kFields && c * kFields + q < len; q++) {
       j += static_cast<int>(w >> (kFieldBits * q)) & kMaxStep;
       const int pc = j >> 1;   // physical column
       const int col = pc - 1 - pc / kZeroPeriod;
@@ -403,7 +417,7 @@ __global__ void zero_words_kernel(int32_t *p, int n, bool keep_faults = false) {
 
 struct KindArgs {
   const uint32_t *slice_base;
-  const uint16_t *slice_nch;
+  const uint16_t *slice_len;
   const uint16_t *row_idx;
   const uint32_t *minmax;
   int slices, height, width, parts;
@@ -524,6 +538,23 @@ __device__ __forceinline__ uint2 load_chunk(const uint2 *p) {
   return *p;
 }
 
+// The first n entries of a chunk, n the same in every lane: the last chunk of a
+// slice, which is walked only as far as the slice's longest row goes.
+__device__ __forceinline__ void add_entries(uint2 cw, int n, uint32_t &at, float &acc,
+                                            bf16x2 minmax) {
+  if (n == kFields) {
+    add_chunk(cw, at, acc, minmax);
+    return;
+  }
+  unsigned long long w = (static_cast<unsigned long long>(cw.y) << 32) | cw.x;
+  for (int q = 0; q < n; q++) {
+    at += (static_cast<uint32_t>(w) & static_cast<uint32_t>(kMaxStep)) << 2;
+    w >>= kFieldBits;
+    const bf16x2 v = __builtin_bit_cast(bf16x2, *(lds_word *)static_cast<uintptr_t>(at));
+    acc = __builtin_amdgcn_fdot2_f32_bf16(v, minmax, acc, false);
+  }
+}
+
 // This lane's chunk 0 of the slice that starts at chunk `base` of the stream.
 __device__ __forceinline__ const uint2 *chunk_pointer(const uint2 *stream, uint32_t base) {
   return stream + static_cast<int64_t>(base) * 64 + (threadIdx.x & 63);
@@ -535,7 +566,8 @@ __device__ __forceinline__ const uint2 *chunk_pointer(const uint2 *stream, uint3
 template <int R, bool kOnce = false>
 struct Walk {
   uint32_t base;     // the slice's first chunk, in chunks; the same in every lane,
-  int nch;           // like the chunk count (where this wavefront stops)
+  int nch;           // like the chunk count (where this wavefront stops),
+  int last;          // the entries of chunk nch - 1 that are walked (9 unless it ends the slice)
   int c0;            // and the chunk this wavefront starts at (0 unless it shares the slice)
   int j0;            // this lane's position at chunk c0
   int ridx;
@@ -552,8 +584,10 @@ __device__ __forceinline__ Walk<R, kOnce> load_slice(const PreparedArgs &a, cons
                                                      int g_hi = 1 << 20) {
   const int lane = threadIdx.x & 63;
   Walk<R, kOnce> w;
-  const int nch_all = __builtin_amdgcn_readfirstlane(k.slice_nch[sl]);
+  const int len = __builtin_amdgcn_readfirstlane(k.slice_len[sl]);
+  const int nch_all = chunks_of(len);
   w.nch = min(g_hi * kGroupChunks, nch_all);
+  w.last = w.nch == nch_all ? last_entries_of(len) : kFields;
   w.c0 = g_lo * kGroupChunks;
   w.ridx = k.row_idx[sl * 64 + lane];
   w.minmax = k.minmax[sl * 64 + lane];
@@ -568,19 +602,26 @@ __device__ __forceinline__ Walk<R, kOnce> load_slice(const PreparedArgs &a, cons
 }
 
 // R chunks (the depth of the walk's ring) starting at chunk c added onto the
-// partial sum.  kChecked: the wavefront's last chunks, fewer than R.
+// partial sum; all of them whole (c + R <= nch - 1), each replaced in the ring
+// by the chunk R further on.
+// kChecked: the walk's last chunks, fewer than R whole ones and then chunk
+// nch - 1 with its `last` entries; nothing is requested any more.
 template <bool kChecked, int R, bool kOnce>
 __device__ __forceinline__ void run_chunks(Walk<R, kOnce> &w, const uint2 *p, int c, uint32_t &at,
                                            float &part, bf16x2 minmax) {
   const int nch = w.nch;
 #pragma unroll
   for (int i = 0; i < R; i++) {
-    if (!kChecked || c + i < nch) {
+    if (!kChecked) {
       const uint2 cw = w.ring[i];
       // unconditional, clamped to the last chunk: the load can target the ring
       // register itself and the loop needs no wait for it
       w.ring[i] = load_chunk<kOnce>(p + min(c + i + R, nch - 1) * 64);
       add_chunk(cw, at, part, minmax);
+    } else if (c + i < nch - 1) {
+      add_chunk(w.ring[i], at, part, minmax);
+    } else if (c + i == nch - 1) {
+      add_entries(w.ring[i], w.last, at, part, minmax);
     }
   }
 }
@@ -620,6 +661,7 @@ __device__ __forceinline__ float run_slice(Walk<R, kOnce> &w, const uint2 *strea
   // is the same in all lanes back into scalar ones, for scalar loop control
   // and scalar address arithmetic
   w.nch = __builtin_amdgcn_readfirstlane(w.nch);
+  w.last = __builtin_amdgcn_readfirstlane(w.last);
   const uint2 *p = chunk_pointer(stream, __builtin_amdgcn_readfirstlane(w.base));
   const int lane = threadIdx.x & 63;
   const bf16x2 minmax = __builtin_bit_cast(bf16x2, w.minmax);
@@ -636,15 +678,14 @@ __device__ __forceinline__ float run_slice(Walk<R, kOnce> &w, const uint2 *strea
     }
     partial = 0.f;
   };
-  for (; c + R <= w.nch; c += R) {
+  for (; c + R <= w.nch - 1; c += R) {
     run_chunks<false>(w, p, c, at, partial, minmax);
     if ((c + R) % kGroupChunks == 0) group_done();
   }
-  if (c < w.nch) {
-    run_chunks<true>(w, p, c, at, partial, minmax);
-    if ((c + R) % kGroupChunks == 0) group_done();
-    c += R;
-  }
+  // fewer than R whole chunks are left, and the last chunk
+  run_chunks<true>(w, p, c, at, partial, minmax);
+  if ((c + R) % kGroupChunks == 0) group_done();
+  c += R;
   if (part) {
     // the slice's last group, unless the loop has just closed it
     if (c % kGroupChunks) part[(c / kGroupChunks) * 64 + lane] = partial;
@@ -764,6 +805,30 @@ __device__ __forceinline__ void add_chunk_group(uint2 cw, uint32_t &at, GroupSum
   }
 }
 
+// The first n entries of a chunk for four tokens (see add_entries).
+__device__ __forceinline__ void add_entries_group(uint2 cw, int n, uint32_t &at, GroupSums &acc,
+                                                  uint32_t w_min, uint32_t w_max) {
+  if (n == kFields) {
+    add_chunk_group(cw, at, acc, w_min, w_max);
+    return;
+  }
+  unsigned long long w = (static_cast<unsigned long long>(cw.y) << 32) | cw.x;
+  for (int q = 0; q < n; q++) {
+    at += (static_cast<uint32_t>(w) & static_cast<uint32_t>(kMaxStep)) << 2;
+    w >>= kFieldBits;
+    const uint32_t is_max = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int>(at), 2, 1));
+    const uint32_t k_lo = (w_max & is_max) | (w_min & ~is_max);
+    const uint32_t k_hi = k_lo << 16;
+    lds_word *col = (lds_word *)static_cast<uintptr_t>(at & ~7u);
+    const bf16x2 v01 = __builtin_bit_cast(bf16x2, col[0]);
+    const bf16x2 v23 = __builtin_bit_cast(bf16x2, col[1]);
+    acc.v[0] = __builtin_amdgcn_fdot2_f32_bf16(v01, __builtin_bit_cast(bf16x2, k_lo), acc.v[0], false);
+    acc.v[1] = __builtin_amdgcn_fdot2_f32_bf16(v01, __builtin_bit_cast(bf16x2, k_hi), acc.v[1], false);
+    acc.v[2] = __builtin_amdgcn_fdot2_f32_bf16(v23, __builtin_bit_cast(bf16x2, k_lo), acc.v[2], false);
+    acc.v[3] = __builtin_amdgcn_fdot2_f32_bf16(v23, __builtin_bit_cast(bf16x2, k_hi), acc.v[3], false);
+  }
+}
+
 // run_slice for four tokens: the same groups of 72 entries per token.  With
 // `part` the wavefront shares its slice and leaves each group's four partial
 // sums at part[group * 64 + lane].
@@ -771,6 +836,7 @@ __device__ __forceinline__ GroupSums run_slice_group(SliceWalk &w, const uint2 *
                                                      const uint32_t *xa, GroupSums *part,
                                                      int pass, int passes) {
   w.nch = __builtin_amdgcn_readfirstlane(w.nch);
+  w.last = __builtin_amdgcn_readfirstlane(w.last);
   const uint2 *p = chunk_pointer(stream, __builtin_amdgcn_readfirstlane(w.base));
   const int lane = threadIdx.x & 63;
   const uint32_t w_min = w.minmax & 0xffffu, w_max = w.minmax >> 16;
@@ -791,10 +857,12 @@ __device__ __forceinline__ GroupSums run_slice_group(SliceWalk &w, const uint2 *
   for (; c < w.nch; c += kRing) {
 #pragma unroll
     for (int i = 0; i < kRing; i++) {
-      if (c + i < w.nch) {
+      if (c + i < w.nch - 1) {
         const uint2 cw = w.ring[i];
         w.ring[i] = p[min(c + i + kRing, w.nch - 1) * 64];
         add_chunk_group(cw, at, partial, w_min, w_max);
+      } else if (c + i == w.nch - 1) {
+        add_entries_group(w.ring[i], w.last, at, partial, w_min, w_max);   // the walk's last chunk
       }
     }
     if ((c + kRing) % kGroupChunks == 0) {
@@ -841,15 +909,17 @@ __device__ __forceinline__ SplitWalk split_begin(const PreparedArgs &a, const Ki
   r.w.base = 0;
   r.w.j0 = 0;
   r.w.nch = 0;
+  r.w.last = kFields;
   r.w.minmax = 0u;
   r.w.ridx = 0xffff;
   // both words of the slice's description in one round trip (a slice that
   // exists is read also where this wavefront has none)
   const int64_t described = r.mine ? r.sl : static_cast<int64_t>(e) * k.slices + s0;
-  const int nch_word = k.slice_nch[described];
+  const int len_word = k.slice_len[described];
   const uint32_t base_word = k.slice_base[described];
   if (r.mine) {
-    const int nch_all = __builtin_amdgcn_readfirstlane(nch_word);
+    const int len = __builtin_amdgcn_readfirstlane(len_word);
+    const int nch_all = chunks_of(len);
     r.ngroups = (nch_all + kGroupChunks - 1) / kGroupChunks;
     r.g_lo = sub * r.ngroups / k.split;
     r.g_hi = (sub + 1) * r.ngroups / k.split;
@@ -861,6 +931,7 @@ __device__ __forceinline__ SplitWalk split_begin(const PreparedArgs &a, const Ki
       const uint2 *p = chunk_pointer(a.stream, base);
       const int c_lo = r.g_lo * kGroupChunks;
       r.w.nch = min(r.g_hi * kGroupChunks, nch_all);
+      r.w.last = r.w.nch == nch_all ? last_entries_of(len) : kFields;
       if (r.g_lo)
         r.w.j0 = a.ckpt[(checkpoint_entry(base, k.first_slice + r.sl) + r.g_lo) * 64 + lane];
 #pragma unroll
@@ -889,9 +960,9 @@ __device__ __forceinline__ void split_run(const PreparedArgs &a, const KindArgs 
     float partial = 0.f;
     const int c_end = min((g + 1) * kGroupChunks, r.w.nch);
     for (int c = g * kGroupChunks; c < c_end; c += kSplitRing) {
-      if (c + kSplitRing <= c_end)
+      if (c + kSplitRing <= r.w.nch - 1)      // whole chunks only, and more to come
         run_chunks<false>(r.w, p, c, at, partial, minmax);
-      else
+      else                                    // the run that ends with this wavefront's last chunk
         run_chunks<true>(r.w, p, c, at, partial, minmax);
     }
     if (alone) {
@@ -1024,7 +1095,7 @@ __device__ __forceinline__ void walk_tile(const PreparedArgs &a, const KindArgs 
     float *mine = partials + (wave / split) * k.groups_max * 64;
     int groups = 0;
     if (sl < all) {
-      groups = (__builtin_amdgcn_readfirstlane(k.slice_nch[slice]) + kGroupChunks - 1) /
+      groups = (chunks_of(__builtin_amdgcn_readfirstlane(k.slice_len[slice])) + kGroupChunks - 1) /
                kGroupChunks;
       const int g_lo = sub * groups / split, g_hi = (sub + 1) * groups / split;
       if (g_lo < g_hi) {
@@ -1271,8 +1342,8 @@ __device__ __forceinline__ void fused_group_tile(const PreparedArgs &a, uint32_t
     GroupSums *mine = reinterpret_cast<GroupSums *>(xa) + (wave / ko.tail_split) * ko.groups_max * 64;
     int groups = 0;
     if (sl < ko.slices) {
-      groups = (__builtin_amdgcn_readfirstlane(ko.slice_nch[first + sl]) + kGroupChunks - 1) /
-               kGroupChunks;
+      groups = (chunks_of(__builtin_amdgcn_readfirstlane(ko.slice_len[first + sl])) +
+                kGroupChunks - 1) / kGroupChunks;
       const int g_lo = sub * groups / ko.tail_split, g_hi = (sub + 1) * groups / ko.tail_split;
       if (g_lo < g_hi) {
         SliceWalk tail = load_slice(a, ko, first + sl, g_lo, g_hi);
@@ -1405,8 +1476,8 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
       float *mine = reinterpret_cast<float *>(xa) + (wave / ko.tail_split) * ko.groups_max * 64;
       int groups = 0;
       if (sl < ko.slices) {
-        groups = (__builtin_amdgcn_readfirstlane(ko.slice_nch[first + sl]) + kGroupChunks - 1) /
-                 kGroupChunks;
+        groups = (chunks_of(__builtin_amdgcn_readfirstlane(ko.slice_len[first + sl])) +
+                  kGroupChunks - 1) / kGroupChunks;
         const int g_lo = sub * groups / ko.tail_split, g_hi = (sub + 1) * groups / ko.tail_split;
         if (g_lo < g_hi) {
           TokenWalk tail = load_slice<kRing, kOnce>(a, ko, first + sl, g_lo, g_hi);
@@ -1693,18 +1764,21 @@ int prepare_layout(const Source &src, void *meta, int64_t meta_bytes, LayoutResu
   int32_t *status = reinterpret_cast<int32_t *>(base + m.status);
   int32_t *counts = reinterpret_cast<int32_t *>(base + m.counts);
   zero_words_kernel<<<1, 64, 0, s>>>(status, 4);
+  HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(order_rows_kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(kOrderRowsLds)));
   int64_t slice0 = 0;
   for (int i = 0; i < src.kinds; i++) {
     const KindMeta &k = m.k[i];
-    uint16_t *row_chunks = reinterpret_cast<uint16_t *>(base + k.row_chunks);
+    uint16_t *row_len = reinterpret_cast<uint16_t *>(base + k.row_len);
     const int64_t rows = static_cast<int64_t>(src.count) * k.height;
     count_entries_kernel<<<static_cast<unsigned>((rows + 255) / 256), 256, 0, s>>>(
-        src.w_comp, src.code_base[i], src.row_off[i], src.dec, row_chunks, status, k.height,
+        src.w_comp, src.code_base[i], src.row_off[i], src.dec, row_len, status, k.height,
         k.width, rows);
-    order_rows_kernel<<<src.count, 256, 0, s>>>(
-        row_chunks, src.minmax[i], reinterpret_cast<uint16_t *>(base + k.row_idx),
+    order_rows_kernel<<<src.count, 256, kOrderRowsLds, s>>>(
+        row_len, src.minmax[i], reinterpret_cast<uint16_t *>(base + k.row_idx),
         reinterpret_cast<uint32_t *>(base + k.minmax),
-        reinterpret_cast<uint16_t *>(base + k.slice_nch), counts + slice0, status, k.height,
+        reinterpret_cast<uint16_t *>(base + k.slice_len), counts + slice0, status, k.height,
         k.slices, i);
     slice0 += static_cast<int64_t>(src.count) * k.slices;
   }
@@ -1751,7 +1825,7 @@ int prepare_codes(const Source &src, const Prepared &p, hipStream_t s, const cha
     emit_entries_kernel<<<static_cast<unsigned>((lanes + 255) / 256), 256, 0, s>>>(
         src.w_comp, src.code_base[i], src.row_off[i], src.dec,
         reinterpret_cast<const uint32_t *>(base + k.slice_base),
-        reinterpret_cast<const uint16_t *>(base + k.slice_nch),
+        reinterpret_cast<const uint16_t *>(base + k.slice_len),
         reinterpret_cast<const uint16_t *>(base + k.row_idx), stream, ckpt, k.height, k.width,
         k.slices, first_slice, lanes);
     first_slice += kslices;
@@ -1909,7 +1983,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     }
     const KindMeta &k = m.k[i];
     ka.slice_base = reinterpret_cast<const uint32_t *>(base + k.slice_base);
-    ka.slice_nch = reinterpret_cast<const uint16_t *>(base + k.slice_nch);
+    ka.slice_len = reinterpret_cast<const uint16_t *>(base + k.slice_len);
     ka.row_idx = reinterpret_cast<const uint16_t *>(base + k.row_idx);
     ka.minmax = reinterpret_cast<const uint32_t *>(base + k.minmax);
     ka.slices = k.slices;
@@ -2270,7 +2344,7 @@ int decode_prepared(const Prepared &p, int kind, int index, void *tern_out, hipS
   fill_bytes_kernel<<<static_cast<unsigned>((n + 255) / 256), 256, 0, s>>>(out, n, 0);
   decode_entries_kernel<<<(k.slices * 64 + 255) / 256, 256, 0, s>>>(
       static_cast<const uint2 *>(p.codes), reinterpret_cast<const uint32_t *>(base + k.slice_base),
-      reinterpret_cast<const uint16_t *>(base + k.slice_nch),
+      reinterpret_cast<const uint16_t *>(base + k.slice_len),
       reinterpret_cast<const uint16_t *>(base + k.row_idx), out,
       static_cast<int64_t>(index) * k.slices, k.slices, k.width);
   HIP_TRY(hipGetLastError());
