@@ -15,6 +15,9 @@
  *   sub1o_dequant        test.py:110, sub1_cuda_kernel.cu:156-157,170-171
  *   sub1o_matvec_lanes   sub1_cuda_kernel.cu:143-201 (lane order, tree, y +=)
  *   sub1o_matvec_seq     same sums, taken per symbol, in groups of 32 codes
+ *   sub1o_matvec_wave    same sums, codeword i of a row in lane i mod 64, the 64
+ *                        lanes summed by a butterfly (the order of the
+ *                        wavefront-per-row kernel behind sub1_matvec)
  *   sub1o_gap_entries    a row's non-zero weights as the 7-bit gap entries of
  *                        the library's prepared stream (no reference lines:
  *                        the format is the library's own; pinned by decoding
@@ -371,6 +374,40 @@ void sub1o_matvec_seq(const int32_t *dec, const uint16_t *codes,
   }
 }
 
+/* Same product in the order of the library's wavefront-per-row kernel: codeword
+ * i of a row belongs to lane i mod 64; a lane adds, for its codewords in turn
+ * and their non-zero digits left to right, x * (row min | row max) with one
+ * fused multiply-add onto its own fp32 sum; the 64 lane sums are then combined
+ * by a butterfly, lane l taking l + (l ^ m) for m = 1, 2, 4, 8, 16, 32 (both
+ * partners compute the same sum: fp32 addition commutes); bf16; +=.  A third
+ * fp32 ordering of the sum of sub1o_matvec_lanes. */
+void sub1o_matvec_wave(const int32_t *dec, const uint16_t *codes,
+                       const int32_t *row_off, const uint16_t *ter_minmax,
+                       const uint16_t *x, uint16_t *y, int height, int width) {
+  for (int r = 0; r < height; r++) {
+    float deq[3] = {0.f, bf16_to_f32(ter_minmax[2 * r]), bf16_to_f32(ter_minmax[2 * r + 1])};
+    float lane[64], next[64];
+    for (int l = 0; l < 64; l++) lane[l] = 0.f;
+    int idx = 0;
+    for (int c = row_off[r]; c < row_off[r + 1]; c++) {
+      int e = codes[c];
+      int l = (c - row_off[r]) & 63;
+      int n = 2 * (dec[2 * e] & 0xf);
+      for (int d = 0; d < n && idx + d < width; d++) {
+        int t = entry_digit(dec, e, d);
+        if (t) lane[l] = fmaf(bf16_to_f32(x[idx + d]), deq[t], lane[l]);
+      }
+      idx += n;
+    }
+    for (int m = 1; m < 64; m *= 2) {
+      for (int l = 0; l < 64; l++) next[l] = lane[l] + lane[l ^ m];
+      memcpy(lane, next, sizeof lane);
+    }
+    float acc = bf16_to_f32(y[r]) + bf16_to_f32(f32_to_bf16(lane[0]));
+    y[r] = f32_to_bf16(acc);
+  }
+}
+
 /* The prepared stream's view of a row.  Activations are laid out by physical
  * column: real column c is physical column q = c + c/16 + 1, every 17th
  * physical column (0, 17, 34, ...) is a zero column.  A position p = 2q + s - 1
@@ -480,7 +517,8 @@ void sub1o_matvec_f64(const uint8_t *tern, const uint16_t *ter_minmax,
 /* One expert FFN on one token as the model runs it (sub1.py:317 calls
  * wo(relu(wi(x))), each projection through sub1.py:132-143: zeroed bf16
  * output, one matvec).  h is bf16 between the stages.  order: 0 = lane order,
- * 1 = per-symbol stream order, 2 = prepared-stream order.  h_out may be NULL. */
+ * 1 = per-symbol stream order, 2 = prepared-stream order, 3 = wavefront-per-row
+ * order.  h_out may be NULL. */
 void sub1o_expert_ffn(const int32_t *dec,
                       const uint16_t *wi_codes, const int32_t *wi_row_off,
                       const uint16_t *wi_minmax,
@@ -493,6 +531,8 @@ void sub1o_expert_ffn(const int32_t *dec,
     sub1o_matvec_lanes(dec, wi_codes, wi_row_off, wi_minmax, x, h, d_ff, d_model);
   else if (order == 1)
     sub1o_matvec_seq(dec, wi_codes, wi_row_off, wi_minmax, x, h, d_ff, d_model);
+  else if (order == 3)
+    sub1o_matvec_wave(dec, wi_codes, wi_row_off, wi_minmax, x, h, d_ff, d_model);
   else
     sub1o_matvec_gap(dec, wi_codes, wi_row_off, wi_minmax, x, h, d_ff, d_model);
   for (int i = 0; i < d_ff; i++)
@@ -503,6 +543,8 @@ void sub1o_expert_ffn(const int32_t *dec,
     sub1o_matvec_lanes(dec, wo_codes, wo_row_off, wo_minmax, h, y, d_model, d_ff);
   else if (order == 1)
     sub1o_matvec_seq(dec, wo_codes, wo_row_off, wo_minmax, h, y, d_model, d_ff);
+  else if (order == 3)
+    sub1o_matvec_wave(dec, wo_codes, wo_row_off, wo_minmax, h, y, d_model, d_ff);
   else
     sub1o_matvec_gap(dec, wo_codes, wo_row_off, wo_minmax, h, y, d_model, d_ff);
   free(h);

@@ -197,7 +197,7 @@ class COracle:
         L.sub1o_decode.restype = ctypes.c_int
         L.sub1o_dequant.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int, vp]
         L.sub1o_dequant.restype = None
-        for name in ('sub1o_matvec_lanes', 'sub1o_matvec_seq'):
+        for name in ('sub1o_matvec_lanes', 'sub1o_matvec_seq', 'sub1o_matvec_wave'):
             f = getattr(L, name)
             f.argtypes = [vp] * 6 + [ctypes.c_int, ctypes.c_int]
             f.restype = None
@@ -293,6 +293,12 @@ class COracle:
         return self._matvec(self.lib.sub1o_matvec_seq, codes, row_off,
                             ter_minmax, x, y, dec)
 
+    def matvec_wave(self, codes, row_off, ter_minmax, x, y=None, dec=None):
+        """Wavefront-per-row order (codeword i in lane i mod 64, butterfly over
+        the 64 lane sums); returns y."""
+        return self._matvec(self.lib.sub1o_matvec_wave, codes, row_off,
+                            ter_minmax, x, y, dec)
+
     def matvec_gap(self, codes, row_off, ter_minmax, x, y=None, dec=None):
         """Prepared-stream order (groups of 72 gap entries, one fused
         multiply-add per entry); returns y."""
@@ -325,6 +331,8 @@ class COracle:
 
     def expert_ffn(self, wi, wo, x, order=0, dec=None):
         """wo(relu(wi(x))) for one token.  wi/wo = (codes, row_off, ter_minmax).
+        order: 0 lane order, 1 per-symbol stream order, 2 prepared-stream
+        order, 3 wavefront-per-row order.
         Returns (y uint16 [d_model], h uint16 [d_ff])."""
         dec = self.tables()[0] if dec is None else dec
         a = [np.ascontiguousarray(wi[0], dtype=np.uint16),

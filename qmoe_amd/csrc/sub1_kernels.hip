@@ -255,30 +255,128 @@ __device__ __forceinline__ void row_sums(const uint32_t *__restrict__ tab,
 }
 
 // ------------------------------------------------------------- matvec ------
+//
+// One product y += W x on the packed layout, built for the latency of a single
+// call (reference sub1_cuda_kernel.cu:163-201 re-thought for 64-wide
+// wavefronts): a WAVEFRONT per row.  Lane j takes codeword j of each run of 64
+// consecutive codes of the row: one coalesced 128-byte load per run; its
+// dictionary entry straight from the caller's dec (8 bytes per lane, from L2: no
+// derived table and nothing remembered between calls); the column at which the
+// codeword starts from a DPP prefix sum of the entries' lengths across the
+// lanes; the activation under each of the entry's non-zero digits (at most
+// three for the fixed dictionary) from x through the vector cache; products
+// x * (row min | row max) added in fp32 per lane; and at the row's end a
+// butterfly sum over the 64 lanes.  Every load a wavefront needs is requested
+// as early as its address is known: row offsets, (min, max) and y at once, all
+// code loads of the row before the first table read.
+//
+// Order of additions (the oracle's sub1o_matvec_wave): lane j adds its
+// codewords j, j + 64, ... in turn, the digits of a codeword left to right, one
+// fused multiply-add each; then six butterfly steps, lane l adding lane l ^ m
+// for m = 1, 2, 4, 8, 16, 32; bf16; y += in bf16.
 
-template <int kThreads>
-__global__ __launch_bounds__(kThreads) void matvec_kernel(
-    const uint32_t *__restrict__ tab, const uint16_t *__restrict__ w_comp,
+// dpp_ctrl values of the row shifts and row broadcasts (CDNA ISA, DPP)
+constexpr int kDppRowShr1 = 0x111, kDppRowShr2 = 0x112, kDppRowShr4 = 0x114, kDppRowShr8 = 0x118;
+constexpr int kDppBcast15 = 0x142, kDppBcast31 = 0x143;
+constexpr int kDppQuadXor1 = 0xb1, kDppQuadXor2 = 0x4e;      // quad_perm [1,0,3,2], [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141, kDppRowMirror = 0x140;
+
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ int dpp_or_zero(int v) {
+  // lanes outside the row mask and lanes whose source lies outside the row get 0
+  return __builtin_amdgcn_update_dpp(0, v, kCtrl, kRowMask, 0xf, false);
+}
+
+// Inclusive prefix sum over the 64 lanes.
+__device__ __forceinline__ int wave_prefix_sum(int v) {
+  v += dpp_or_zero<kDppRowShr1, 0xf>(v);
+  v += dpp_or_zero<kDppRowShr2, 0xf>(v);
+  v += dpp_or_zero<kDppRowShr4, 0xf>(v);
+  v += dpp_or_zero<kDppRowShr8, 0xf>(v);
+  v += dpp_or_zero<kDppBcast15, 0xa>(v);   // row 0 -> row 1, row 2 -> row 3
+  v += dpp_or_zero<kDppBcast31, 0xc>(v);   // rows 0-1 -> rows 2-3
+  return v;
+}
+
+template <int kCtrl>
+__device__ __forceinline__ float dpp_float(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xf, 0xf, false));
+}
+
+// Lane l receives the sum of the butterfly over all 64 lanes: l + (l ^ 1), then
+// ^ 2, ^ 4, ^ 8, ^ 16, ^ 32.  After the steps 1 and 2 the four lanes of a quad
+// hold the same value, so the mirror within eight lanes pairs a lane with the
+// other quad exactly as ^ 4 does, and the mirror within a row of sixteen as ^ 8.
+__device__ __forceinline__ float wave_butterfly_sum(float v) {
+  v += dpp_float<kDppQuadXor1>(v);
+  v += dpp_float<kDppQuadXor2>(v);
+  v += dpp_float<kDppHalfMirror>(v);
+  v += dpp_float<kDppRowMirror>(v);
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+  return v;
+}
+
+constexpr int kWaveRuns = 4;   // runs of 64 codes whose loads are requested together
+
+template <int kWaves>
+__global__ __launch_bounds__(64 * kWaves) void matvec_wave_kernel(
+    const int32_t *__restrict__ dec, const uint16_t *__restrict__ w_comp,
     const int32_t *__restrict__ row_off, const uint32_t *__restrict__ minmax,
     const uint16_t *__restrict__ x, uint16_t *__restrict__ y, int height, int width,
-    int64_t ldx, int64_t ldy, const int32_t *__restrict__ dec,
-    const int32_t *__restrict__ print, int32_t *sticky) {
-  extern __shared__ float lds[];
-  if (blockIdx.x == 0 && blockIdx.y == 0) compare_print(dec, print, sticky);
+    int64_t ldx, int64_t ldy) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * kWaves + (threadIdx.x >> 6);
+  if (row >= height) return;
   x += static_cast<int64_t>(blockIdx.y) * ldx;
   y += static_cast<int64_t>(blockIdx.y) * ldy;
-  stage_activations<kThreads>(lds, x, width);
-  __syncthreads();
-  const int row = blockIdx.x * kThreads + threadIdx.x;
-  if (row >= height) return;
-  const int off = row_off[row];
-  const int len = row_off[row + 1] - off;
-  float s1, s2;
-  row_sums(tab, w_comp + off, len, lds + 1, s1, s2);
-  float res = row_result(minmax[row], s1, s2);
-  // reference sub1_cuda_kernel.cu:200: y[row] += bf16(res), the sum in bf16
-  float acc = bf16_to_f32(y[row]) + bf16_to_f32(f32_to_bf16(res));
-  y[row] = f32_to_bf16(acc);
+  const int off = __builtin_amdgcn_readfirstlane(row_off[row]);
+  const int len = __builtin_amdgcn_readfirstlane(row_off[row + 1]) - off;
+  const uint32_t mm = minmax[row];
+  const uint16_t y_old = y[row];
+  const float w_min = __uint_as_float(mm << 16), w_max = __uint_as_float(mm & 0xffff0000u);
+  const uint16_t *codes = w_comp + off;
+  const uint2 *table = reinterpret_cast<const uint2 *>(dec);
+  float acc = 0.f;
+  int col = 0;   // the column at which the current run of codes starts
+  for (int c0 = 0; c0 < len; c0 += 64 * kWaveRuns) {
+    // the codes of up to kWaveRuns runs, then their dictionary entries
+    int code[kWaveRuns];
+    uint2 entry[kWaveRuns];
+#pragma unroll
+    for (int u = 0; u < kWaveRuns; u++) {
+      const int i = c0 + 64 * u + lane;
+      code[u] = i < len ? codes[i] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < kWaveRuns; u++)
+      entry[u] = code[u] >= 0 ? table[code[u]] : make_uint2(0u, 0u);   // no code: no digits, length 0
+
+#pragma unroll
+    for (int u = 0; u < kWaveRuns; u++) {
+      if (c0 + 64 * u >= len) break;
+      const int span = 2 * static_cast<int>(entry[u].x & 15u);     // weights the codeword covers
+      const int upto = wave_prefix_sum(span);
+      int at = col + upto - span;                                  // where this lane's codeword starts
+      col += __builtin_amdgcn_readlane(upto, 63);
+      unsigned long long digits = static_cast<unsigned long long>(entry[u].x >> 4) |
+                                  (static_cast<unsigned long long>(entry[u].y >> 4) << 28);
+      while (digits) {
+        const int d = (__ffsll(digits) - 1) >> 1;
+        const int sym = static_cast<int>(digits >> (2 * d)) & 3;
+        digits &= ~(3ull << (2 * d));
+        if (at + d < width) {   // digits past the width are dropped
+          const float xv = bf16_to_f32(x[at + d]);
+          acc = __fmaf_rn(xv, sym == 1 ? w_min : (sym == 2 ? w_max : 0.f), acc);
+        }
+      }
+    }
+  }
+  const float res = wave_butterfly_sum(acc);
+  if (lane == 0) {
+    // reference sub1_cuda_kernel.cu:200: y[row] += bf16(res), the sum in bf16
+    y[row] = f32_to_bf16(bf16_to_f32(y_old) + bf16_to_f32(f32_to_bf16(res)));
+  }
 }
 
 // ------------------------------------------------------------- decode ------
@@ -617,9 +715,8 @@ extern "C" int sub1_matvec_tokens(const int32_t *dec, const int16_t *w_comp,
   if (tokens == 0) return SUB1_OK;
   if (!dec || !row_off || !ter_minmax || !x || !y)
     return fail(SUB1_ERR_NULL, "sub1_matvec: NULL argument");
-  if (height < 1 || width < 1 || width > SUB1_MAX_WIDTH)
-    return fail(SUB1_ERR_SHAPE, "sub1_matvec: height %d width %d unsupported (width 1..%d)",
-                height, width, SUB1_MAX_WIDTH);
+  if (height < 1 || width < 1)
+    return fail(SUB1_ERR_SHAPE, "sub1_matvec: height %d width %d", height, width);
   if (tokens < 0 || tokens > 65535)
     return fail(SUB1_ERR_SHAPE, "sub1_matvec: tokens %d outside 0..65535", tokens);
   if (tokens > 1 && (ldx < width || ldy < height))
@@ -629,20 +726,13 @@ extern "C" int sub1_matvec_tokens(const int32_t *dec, const int16_t *w_comp,
       misaligned(w_comp, 2) || misaligned(x, 2) || misaligned(y, 2))
     return fail(SUB1_ERR_ALIGN, "sub1_matvec: misaligned pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  TableSlot slot;
-  int32_t *sticky = nullptr;
-  int rc = slot_table_for(dec, s, &slot, &sticky);
-  if (rc) return rc;
-  const uint32_t *tab = slot.tab;
-  size_t lds = lds_dwords_for_width(width) * sizeof(float);
-  rc = allow_lds(matvec_kernel<kMatvecThreads>, lds);
-  if (rc) return rc;
-  dim3 grid((height + kMatvecThreads - 1) / kMatvecThreads, tokens);
-  sub1::note_kernel("matvec_kernel<256>");
-  matvec_kernel<kMatvecThreads><<<grid, kMatvecThreads, lds, s>>>(
-      tab, reinterpret_cast<const uint16_t *>(w_comp), row_off,
+  constexpr int kWaves = 4;   // rows per workgroup
+  dim3 grid((height + kWaves - 1) / kWaves, tokens);
+  sub1::note_kernel("matvec_wave_kernel<4>");
+  matvec_wave_kernel<kWaves><<<grid, 64 * kWaves, 0, s>>>(
+      dec, reinterpret_cast<const uint16_t *>(w_comp), row_off,
       static_cast<const uint32_t *>(ter_minmax), static_cast<const uint16_t *>(x),
-      static_cast<uint16_t *>(y), height, width, ldx, ldy, dec, slot.print, sticky);
+      static_cast<uint16_t *>(y), height, width, ldx, ldy);
   HIP_TRY(hipGetLastError());
   return SUB1_OK;
 }

@@ -83,39 +83,53 @@ def test_wait_limit_arguments(lib):
 
 
 def test_an_address_that_holds_another_dictionary(lib, oracle):
-    """sub1matvec caches its compact table by the address of dec.  The same
-    tensor overwritten with another table: the next launch still multiplies by
-    the old one but says so; after clear_faults() the table is derived afresh."""
+    """The grouped launch on the packed layout caches its compact table by the
+    address of dec.  The same tensor overwritten with another table: the next
+    launch still multiplies by the old one but says so; after clear_faults()
+    the table is derived afresh.  The single product reads dec itself and
+    follows the new contents at once."""
     from qmoe_amd import _lib, sub1, sub1_hip
-    height, width = 96, 130
-    t, mm = so.synthetic_ternary(height, width, 0.6, 77)
-    codes, row_off = oracle.encode(t)
-    xv = so.synthetic_activation(width, 78)
-    w_comp = torch.from_numpy(codes.view(np.int16)).cuda()
-    ro, mmd, x = torch.from_numpy(row_off).cuda(), bf16_dev(mm), bf16_dev(xv)
+    d_model, d_ff = 130, 96
+    ti, mi = so.synthetic_ternary(d_ff, d_model, 0.6, 77)
+    to, mo = so.synthetic_ternary(d_model, d_ff, 0.6, 79)
+    wi, wo = oracle.encode(ti) + (mi,), oracle.encode(to) + (mo,)
+    xv = so.synthetic_activation(d_model, 78)
+    dev = lambda l: (torch.from_numpy(l[0].view(np.int16)).cuda(),
+                     torch.from_numpy(l[1]).cuda(), bf16_dev(l[2]))
     mine = sub1.DEC[0].clone()
-    want = oracle.matvec_seq(codes, row_off, mm, xv)
+    stack = sub1_hip.ExpertStack.from_layers(mine, [dev(wi)], [dev(wo)])
+    x = bf16_dev(xv[None, :])
+    te = torch.zeros(1, dtype=torch.int32, device='cuda')
+    want, _ = oracle.expert_ffn(wi, wo, xv, order=1)
+
+    def layer():
+        y = stack.forward(x, te)
+        torch.cuda.synchronize()
+        return bits_host(y)[0]
 
     def product():
-        y = torch.zeros(height, dtype=torch.bfloat16, device='cuda')
-        sub1_hip.sub1matvec(mine, w_comp, ro, mmd, x, y)
+        y = torch.zeros(d_ff, dtype=torch.bfloat16, device='cuda')
+        dwi = dev(wi)
+        sub1_hip.sub1matvec(mine, dwi[0], dwi[1], dwi[2], x[0], y)
         torch.cuda.synchronize()
         return bits_host(y)
 
-    assert np.array_equal(product(), want)
+    assert np.array_equal(layer(), want)
+    assert np.array_equal(product(), oracle.matvec_wave(wi[0], wi[1], mi, xv))
     sub1_hip.check_faults()
     # every entry becomes "one pair of zeros": all products are zero under this table
     mine.fill_(1)
-    assert np.array_equal(product(), want)           # the stale table, and the flag
+    assert not product().any()                       # the single product reads dec itself
+    assert np.array_equal(layer(), want)             # the stale table, and the flag
     with pytest.raises(sub1_hip.Sub1Fault, match='dec'):
         sub1_hip.check_faults()
     sub1_hip.clear_faults()                          # drops the cached tables as well
-    assert not product().any()
+    assert not layer().any()
     sub1_hip.check_faults()
     # and the explicit way: tell the library before the address changes hands
     _lib.check(lib.sub1_unregister_dec(mine.data_ptr()))
     mine.copy_(sub1.DEC[0])
-    assert np.array_equal(product(), want)
+    assert np.array_equal(layer(), want)
     sub1_hip.check_faults()
     _lib.check(lib.sub1_unregister_dec(mine.data_ptr()))
 

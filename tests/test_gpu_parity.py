@@ -4,8 +4,9 @@ binding), against the CPU oracle on the same seeded inputs.
 Bars:
   * decode, pack: bit-exact against the oracle (integer/byte work);
   * products: the output must equal, bit for bit, the oracle's result in the
-    order the kernel adds in (per-symbol stream order for the packed-layout
-    kernels, prepared-stream order for the prepared ones), must lie within
+    order the kernel adds in (wavefront-per-row order for the single product
+    on the packed layout, per-symbol stream order for the grouped launch on
+    it, prepared-stream order for the prepared kernels), must lie within
         2^-8 |exact| + 64 * 2^-24 * sum|w x|
     of the double-precision product, and must agree with the reference kernel's
     lane-order arithmetic to 1e-2 relative (normwise), the tolerance the task
@@ -24,7 +25,7 @@ REL_TOL = 1e-2          # stated tolerance for outputs
 SWITCH_SHAPES = [(3072, 768, 0.90), (768, 3072, 0.90), (4096, 1024, 0.88),
                  (1024, 4096, 0.88), (6144, 2080, 0.90), (2080, 6144, 0.90)]
 ODD_SHAPES = [(77, 333, 0.7), (5, 1, 0.5), (9, 2, 0.5), (33, 29, 0.3), (64, 56, 0.0),
-              (130, 15, 0.9), (1, 4000, 0.95), (300, 12288, 0.99)]
+              (130, 15, 0.9), (1, 4000, 0.95), (300, 12288, 0.99), (2, 13000, 0.97)]
 
 
 @pytest.fixture(scope='module')
@@ -67,7 +68,7 @@ def check_product(oracle, c, y_bits, prepared=False):
     lanes = so.bf16_bits_to_f32(oracle.matvec_lanes(c['codes'], c['row_off'], c['mm'], c['x']))
     denom = max(np.linalg.norm(lanes), 1e-30)
     assert np.linalg.norm(y - lanes) / denom <= REL_TOL
-    fn = oracle.matvec_gap if prepared else oracle.matvec_seq
+    fn = oracle.matvec_gap if prepared else oracle.matvec_wave
     assert np.array_equal(y_bits, fn(c['codes'], c['row_off'], c['mm'], c['x']))
 
 
@@ -126,11 +127,11 @@ def test_matvec_accumulates_into_y(gpu, oracle):
     pre = so.f32_to_bf16_bits(np.random.default_rng(0).standard_normal(200).astype(np.float32))
     y = bf16_dev(pre).clone()
     op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], c['x_d'], y)
-    want = oracle.matvec_seq(c['codes'], c['row_off'], c['mm'], c['x'], y=pre)
+    want = oracle.matvec_wave(c['codes'], c['row_off'], c['mm'], c['x'], y=pre)
     assert np.array_equal(bits_host(y), want)
     # twice more: the reference's benchmark loop keeps adding onto y (test.py:175)
     op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], c['x_d'], y)
-    want = oracle.matvec_seq(c['codes'], c['row_off'], c['mm'], c['x'], y=want)
+    want = oracle.matvec_wave(c['codes'], c['row_off'], c['mm'], c['x'], y=want)
     assert np.array_equal(bits_host(y), want)
 
 
@@ -179,10 +180,10 @@ def test_matvec_rejects_bad_tensors(gpu, oracle):
         op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], c['x_d'].cpu(), y)
     with pytest.raises(ValueError):
         op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'][:-1], c['mm_d'], c['x_d'], y)
-    from qmoe_amd._lib import Sub1Error
-    big = torch.zeros(12289, dtype=torch.bfloat16, device='cuda')
-    with pytest.raises(Sub1Error):
-        op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], big, y)
+    with pytest.raises(ValueError):
+        op.sub1matvec(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'][:-2], c['x_d'], y)
+    with pytest.raises(TypeError):
+        op.sub1matvec(sub1.DEC[0], c['w_comp'].int(), c['row_off_d'], c['mm_d'], c['x_d'], y)
 
 
 def test_matvec_tokens(gpu, oracle):
@@ -192,7 +193,7 @@ def test_matvec_tokens(gpu, oracle):
     y = torch.zeros((5, 300), dtype=torch.bfloat16, device='cuda')
     op.sub1matvec_tokens(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], bf16_dev(xs), y)
     for i in range(5):
-        want = oracle.matvec_seq(c['codes'], c['row_off'], c['mm'], xs[i])
+        want = oracle.matvec_wave(c['codes'], c['row_off'], c['mm'], xs[i])
         assert np.array_equal(bits_host(y[i]), want)
 
 
@@ -403,7 +404,9 @@ def test_routed_batch_equals_per_token_products(gpu):
         h = torch.relu(h)
         out = torch.zeros(d_model, dtype=torch.bfloat16, device='cuda')
         sub1_hip.sub1matvec(dec, wo[0], wo[1], wo[2], h, out)
-        assert torch.equal(out, y_packed[t]), t
+        # (the single product adds a row by lanes of a wavefront, the grouped
+        # launch on the packed layout codeword by codeword: rounding apart)
+        assert close(out, y_packed[t]), t
         # the prepared kernels, one token per launch
         one = prep.forward(x[t:t + 1].contiguous(), route[t:t + 1].contiguous())
         assert torch.equal(one[0], y[t]), t

@@ -57,6 +57,7 @@ def test_fp32_orders_within_bound(oracle):
         assert within_bound(oracle.matvec_lanes(codes, row_off, mm, x), exact, sum_abs)
         assert within_bound(oracle.matvec_seq(codes, row_off, mm, x), exact, sum_abs)
         assert within_bound(oracle.matvec_gap(codes, row_off, mm, x), exact, sum_abs)
+        assert within_bound(oracle.matvec_wave(codes, row_off, mm, x), exact, sum_abs)
 
 
 def test_unit_vector_picks_a_column(oracle):
@@ -66,7 +67,7 @@ def test_unit_vector_picks_a_column(oracle):
     for k in (0, 1, 27, 28, 99, 199):
         x = np.zeros(200, dtype=np.uint16)
         x[k] = one
-        for fn in (oracle.matvec_lanes, oracle.matvec_seq, oracle.matvec_gap):
+        for fn in (oracle.matvec_lanes, oracle.matvec_seq, oracle.matvec_gap, oracle.matvec_wave):
             y = fn(codes, row_off, mm, x)
             assert np.array_equal(so.bf16_bits_to_f32(y), so.bf16_bits_to_f32(w[:, k]))
 
@@ -106,7 +107,8 @@ def test_expert_ffn_is_two_products_with_relu(oracle):
     wi = oracle.encode(ti) + (mi,)
     wo = oracle.encode(to) + (mo,)
     x = so.synthetic_activation(d_model, 23)
-    for order, fn in ((0, oracle.matvec_lanes), (1, oracle.matvec_seq), (2, oracle.matvec_gap)):
+    for order, fn in ((0, oracle.matvec_lanes), (1, oracle.matvec_seq), (2, oracle.matvec_gap),
+                      (3, oracle.matvec_wave)):
         y, h = oracle.expert_ffn(wi, wo, x, order=order)
         h_ref = fn(wi[0], wi[1], mi, x)
         h_ref = np.where(so.bf16_bits_to_f32(h_ref) > 0, h_ref, 0).astype(np.uint16)
@@ -220,3 +222,37 @@ def test_gap_product_sums_in_groups_of_72_entries(oracle):
             total = np.float32(total + part)
         want[r] = so.f32_to_bf16_bits(np.array([total], np.float32))[0]
     assert np.array_equal(oracle.matvec_gap(codes, row_off, mm, x), want)
+
+
+def test_wave_product_lane_sums_and_butterfly(oracle, entries):
+    """The wavefront-per-row order written out in numpy float32 from the
+    symbols and the independent expansion of the codes: codeword i of a row in
+    lane i mod 64, one multiply-add per non-zero (the product of two bf16 is
+    exact in fp32), then lane l takes l + (l ^ m) for m = 1 .. 32.  Rows of
+    fewer than 64 codewords, of several runs of 64, and y +=."""
+    for height, width, p0, seed in ((9, 2080, 0.88, 41), (5, 6144, 0.9, 42), (7, 130, 0.4, 43),
+                                    (3, 4000, 0.0, 44)):
+        t, mm, codes, row_off, x = make_case(oracle, height, width, p0, seed)
+        f = so.bf16_bits_to_f32(mm)
+        xv = so.bf16_bits_to_f32(x)
+        pre = so.f32_to_bf16_bits(np.linspace(-1, 1, height).astype(np.float32))
+        want = np.zeros(height, dtype=np.uint16)
+        for r in range(height):
+            lanes = np.zeros(64, dtype=np.float32)
+            col = 0
+            for i, code in enumerate(codes[row_off[r]:row_off[r + 1]]):
+                for pair in entries[code]:
+                    for sym in (pair % 3, pair // 3):
+                        if sym and col < width:
+                            assert t[r, col] == sym
+                            lanes[i % 64] = np.float32(lanes[i % 64] + np.float32(xv[col] * f[2 * r + sym - 1]))
+                        col += 1
+            m = 1
+            while m < 64:
+                lanes = (lanes + lanes[np.arange(64) ^ m]).astype(np.float32)
+                m *= 2
+            assert len(set(lanes.tolist())) == 1          # every lane ends with the same sum
+            acc = np.float32(so.bf16_bits_to_f32(pre[r:r + 1])[0]
+                             + so.bf16_bits_to_f32(so.f32_to_bf16_bits(lanes[:1]))[0])
+            want[r] = so.f32_to_bf16_bits(np.array([acc], np.float32))[0]
+        assert np.array_equal(oracle.matvec_wave(codes, row_off, mm, x, y=pre), want)
