@@ -57,7 +57,6 @@ def test_bad_arguments_are_refused_on_the_host():
     assert lib.sub1_matvec(None, one, one, one, one, one, 8, 8, None) == -1
     assert b'NULL' in lib.sub1_last_error()
     assert lib.sub1_matvec(one, one, one, one, one, one, 8, 0, None) == -2
-    assert lib.sub1_matvec(one, one, one, one, one, one, 8, _lib.MAX_WIDTH + 1, None) == -2
     assert lib.sub1_matvec(one, one, one, one, one, one, 0, 8, None) == -2
     assert lib.sub1_matvec(one, odd, one, one, one, one, 8, 8, None) == -3
     assert lib.sub1_pack_count(None, one, one, 8, 8, None) == -1
@@ -67,6 +66,9 @@ def test_bad_arguments_are_refused_on_the_host():
     assert lib.sub1_decode(one, one, one, None, None, one, None, 8, 8, None) == -1
     st = _lib.MoeStack()
     assert lib.sub1_moe_grouped(ctypes.byref(st), one, one, one, 4, one, 1 << 20, None) == -1
+    # the grouped launch on the packed layout stages a row of activations in LDS
+    wide = _lib.MoeStack(256, 256, 256, 256, 256, 256, 256, 256, 1, _lib.MAX_WIDTH + 1, 8)
+    assert lib.sub1_moe_grouped(ctypes.byref(wide), one, one, one, 4, one, 1 << 30, None) == -2
     with pytest.raises(_lib.Sub1Error) as err:
         _lib.check(lib.sub1_matvec(one, one, one, one, one, one, 8, 0, None))
     assert err.value.status == -2 and 'width' in str(err.value)
