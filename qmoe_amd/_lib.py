@@ -152,4 +152,8 @@ def check_faults():
 
 
 def clear_faults():
+    """Reset the fault flags.  After a wait fault the workspace of the launch
+    that raised it may hold stale counts: make the stack allocate new ones
+    (`stack._ws.clear()`), or zero the workspace again, before launching from
+    it once more."""
     check(load().sub1_clear_faults())

@@ -74,7 +74,26 @@ __device__ __forceinline__ void raise_fault(int32_t *sticky, int word) {
   __hip_atomic_store(&sticky[word], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
-// Thread 0's bounded wait until *counter reaches `expect`: relaxed looks at
+// Control words at the head of an expert launch's workspace.  The caller zeroes
+// the workspace once; every launch leaves the words it counts with at zero
+// again (the last workgroup out clears the ticket, the last workgroup that
+// waited on a token's word clears that word), so a launch is one kernel and
+// needs no clearing kernel before it.  Words 1 and 2 only ever grow.
+constexpr int kCtrlTicket = 0;     // tiles handed out
+constexpr int kCtrlGaveUp = 1;     // waits that reached their time limit, all launches so far
+constexpr int kCtrlBadIds = 2;     // tokens whose expert id was >= experts, all launches so far
+constexpr int kCtrlTiles = 3;      // tiles of a launch with tokens grouped by expert
+constexpr int kCtrlExits = 4;      // workgroups of a persistent launch that have left
+constexpr int kCtrlHeader = 8;     // then one word per token:
+// low half: workgroups that have written their part of the token's h;
+// high half: workgroups that have waited for it (the last of them clears the word)
+constexpr int kTokenWaited = 1 << 16;
+
+inline int64_t control_bytes(int tokens) {
+  return (static_cast<int64_t>(kCtrlHeader + tokens) * 4 + 255) / 256 * 256;
+}
+
+// Thread 0's bounded wait until the low half of *counter reaches `expect`: relaxed looks at
 // agent scope, the clock read every 16th look, one acquire at the end.  On
 // time-out the wait-fault flag is set, *gave_up (the launch's own count) goes
 // up by one and the caller carries on (its output
@@ -85,7 +104,7 @@ __device__ __forceinline__ void bounded_wait(const int32_t *counter, int expect,
                                              int32_t *gave_up) {
   int looks = 0;
   int64_t t0 = 0;
-  while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < expect) {
+  while ((__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 0xffff) < expect) {
     if ((++looks & 15) == 1) {
       const int64_t now = static_cast<int64_t>(wall_clock64());
       if (looks == 1) t0 = now;
@@ -98,6 +117,26 @@ __device__ __forceinline__ void bounded_wait(const int32_t *counter, int expect,
     __builtin_amdgcn_s_sleep(2);
   }
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+}
+
+// Thread 0 of a workgroup that has waited on a token's word says so; the last
+// of the token's `waiters` puts the word back to zero for the next launch.
+__device__ __forceinline__ void waited_on(int32_t *counter, int waiters) {
+  const int32_t before = __hip_atomic_fetch_add(counter, kTokenWaited, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+  if ((before >> 16) + 1 == waiters)
+    __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Thread 0 of a workgroup that leaves a persistent launch; the last one out
+// puts the ticket back to zero.
+__device__ __forceinline__ void leave_launch(int32_t *ctrl, int workgroups) {
+  const int32_t before = __hip_atomic_fetch_add(&ctrl[kCtrlExits], 1, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+  if (before + 1 == workgroups) {
+    __hip_atomic_store(&ctrl[kCtrlTicket], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&ctrl[kCtrlExits], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 }
 
 }  // namespace sub1

@@ -509,8 +509,7 @@ struct MoeArgs {
   const uint16_t *x;
   uint16_t *y;
   uint16_t *h;
-  int32_t *ctrl;  // [0] ticket, [1] wait-limit hits, [2] tokens with an expert
-                  // id >= experts (treated as dropped), [4+t] wi tiles done for t
+  int32_t *ctrl;  // the control words (sub1_common.h): ticket, fault counts, a word per token
   int tokens, d_model, d_ff, experts;
   int wi_tiles, wo_tiles;  // per token
   int wi_expect;           // wi tiles a wo tile waits for (wi_tiles outside tests)
@@ -520,7 +519,7 @@ struct MoeArgs {
   const int32_t *print;
 };
 
-constexpr int kCtrlHeader = 4;
+using sub1::kCtrlHeader;
 
 template <int kThreads>
 __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
@@ -569,7 +568,7 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
       // back the whole L2)
       sub1::drain_stores();
       __syncthreads();
-      if (threadIdx.x == 0)
+      if (threadIdx.x == 0 && e >= 0)   // a dropped token's word stays untouched
         __hip_atomic_fetch_add(&a.ctrl[kCtrlHeader + t], 1, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
     } else {
@@ -579,7 +578,8 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
       int e = a.token_expert[t];
       if (e >= a.experts) {
         if (blk == 0 && threadIdx.x == 0)
-          __hip_atomic_fetch_add(&a.ctrl[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_fetch_add(&a.ctrl[sub1::kCtrlBadIds], 1, __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
         e = -1;
       }
       const int row = blk * kThreads + threadIdx.x;
@@ -592,7 +592,7 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
       }
       if (threadIdx.x == 0)
         sub1::bounded_wait(&a.ctrl[kCtrlHeader + t], a.wi_expect, a.wait_ticks, a.sticky,
-                           &a.ctrl[1]);
+                           &a.ctrl[sub1::kCtrlGaveUp]);
       __syncthreads();  // thread 0's acquire now covers the whole workgroup
       stage_activations<kThreads>(lds, a.h + static_cast<int64_t>(t) * a.d_ff, a.d_ff);
       __syncthreads();
@@ -606,8 +606,11 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
             a.wo_minmax[static_cast<int64_t>(e) * a.d_model + row], s1, s2);
         a.y[static_cast<int64_t>(t) * a.d_model + row] = f32_to_bf16(res);
       }
+      // said once the tile's work is done: it takes a round trip to memory
+      if (threadIdx.x == 0) sub1::waited_on(&a.ctrl[kCtrlHeader + t], a.wo_tiles);
     }
   }
+  if (threadIdx.x == 0) sub1::leave_launch(a.ctrl, gridDim.x);
 }
 
 __global__ void zero_i32_kernel(int32_t *p, int n) {
@@ -706,7 +709,7 @@ extern "C" const char *sub1_last_error(void) { return sub1::g_err.c_str(); }
 
 extern "C" const char *sub1_last_kernel(void) { return sub1::g_kernel; }
 
-extern "C" int sub1_abi_version(void) { return 3; }
+extern "C" int sub1_abi_version(void) { return 4; }
 
 extern "C" int sub1_matvec_tokens(const int32_t *dec, const int16_t *w_comp,
                                   const int32_t *row_off, const void *ter_minmax,
@@ -798,8 +801,7 @@ extern "C" int sub1_decode(const int32_t *dec, const int16_t *w_comp,
 
 extern "C" int64_t sub1_moe_workspace_bytes(int tokens, int d_ff) {
   if (tokens < 0 || d_ff < 0) return 0;
-  int64_t ctrl = (static_cast<int64_t>(kCtrlHeader + tokens) * 4 + 255) / 256 * 256;
-  return ctrl + static_cast<int64_t>(tokens) * d_ff * 2;
+  return sub1::control_bytes(tokens) + static_cast<int64_t>(tokens) * d_ff * 2;
 }
 
 extern "C" int sub1_moe_grouped(const sub1_moe_stack *st, const int32_t *token_expert,
@@ -850,8 +852,7 @@ extern "C" int sub1_moe_grouped(const sub1_moe_stack *st, const int32_t *token_e
   a.x = static_cast<const uint16_t *>(x);
   a.y = static_cast<uint16_t *>(y);
   a.ctrl = static_cast<int32_t *>(workspace);
-  int64_t ctrl_bytes = (static_cast<int64_t>(kCtrlHeader + tokens) * 4 + 255) / 256 * 256;
-  a.h = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + ctrl_bytes);
+  a.h = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + sub1::control_bytes(tokens));
   a.tokens = tokens;
   a.d_model = st->d_model;
   a.d_ff = st->d_ff;
@@ -877,8 +878,6 @@ extern "C" int sub1_moe_grouped(const sub1_moe_stack *st, const int32_t *token_e
   int64_t grid = static_cast<int64_t>(cus) * per_cu;
   if (grid > tiles) grid = tiles;
 
-  int nctrl = kCtrlHeader + tokens;
-  zero_i32_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl);
   sub1::note_kernel("moe_kernel<256>");
   moe_kernel<kMoeThreads><<<static_cast<unsigned>(grid), kMoeThreads, lds, s>>>(a);
   HIP_TRY(hipGetLastError());

@@ -61,7 +61,11 @@ constexpr int kRing = 4;             // chunks in flight per lane (2 KB per wave
 constexpr int kGroupChunks = 8;      // chunks (72 entries) per partial sum, a multiple of kRing
 constexpr int kSplitRing = 8;        // chunks in flight per lane where wavefronts share a slice
 constexpr int kMaxRowEntries = 16383; // entries per row the row ordering can count (widths to 12288)
-constexpr int kCtrlHeader = 4;       // ctrl[0] ticket, [1] wait-limit hits, [2] bad expert ids
+using sub1::kCtrlBadIds;
+using sub1::kCtrlGaveUp;
+using sub1::kCtrlHeader;
+using sub1::kCtrlTicket;
+using sub1::kCtrlTiles;
 
 // ------------------------------------------------------------- meta layout --
 //
@@ -406,11 +410,9 @@ __global__ void fill_bytes_kernel(uint8_t *p, int64_t n, uint8_t v) {
   if (i < n) p[i] = v;
 }
 
-// keep_faults: leave words 1 and 2 (the fault counts of the control words) as
-// an earlier launch of the same call left them.
-__global__ void zero_words_kernel(int32_t *p, int n, bool keep_faults = false) {
+__global__ void zero_words_kernel(int32_t *p, int n) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n && !(keep_faults && (i == 1 || i == 2))) p[i] = 0;
+  if (i < n) p[i] = 0;
 }
 
 // ------------------------------------------------------------- main kernel --
@@ -981,19 +983,25 @@ __device__ __forceinline__ void split_run(const PreparedArgs &a, const KindArgs 
 
 // A wo tile waits until its token's wi tiles have published h (bounded spin of
 // one lane, then a barrier that extends its acquire to the workgroup); then the
-// tile's activations go into LDS.  Ends with a barrier.
+// tile's activations go into LDS.  Ends with a barrier.  The tile says that it
+// has waited (done_waiting) once its work is done: that takes a round trip to
+// memory, which does not belong between the wait and the walk.
 __device__ __forceinline__ void await_activations(const PreparedArgs &a, const KindArgs &k,
                                                   int kind, int t, uint32_t *xa) {
   if (kind == 1) {
     if (threadIdx.x == 0)
       sub1::bounded_wait(&a.ctrl[kCtrlHeader + t], a.wi_expect, a.wait_ticks, a.sticky,
-                         &a.ctrl[1]);
+                         &a.ctrl[kCtrlGaveUp]);
     __syncthreads();
   }
   const uint16_t *src = kind ? a.h + static_cast<int64_t>(t) * k.width
                              : a.x + static_cast<int64_t>(t) * a.ldx;
   stage_activations(xa, src, k.width);
   __syncthreads();
+}
+
+__device__ __forceinline__ void done_waiting(const PreparedArgs &a, int t) {
+  if (threadIdx.x == 0) sub1::waited_on(&a.ctrl[kCtrlHeader + t], a.k[1].parts);
 }
 
 // What a ticket stands for.  Every field is the same in all lanes.
@@ -1015,7 +1023,7 @@ __device__ __forceinline__ Tile decode_tile(const PreparedArgs &a, int ticket, b
   tile.e = a.token_expert ? __builtin_amdgcn_readfirstlane(a.token_expert[tile.t]) : 0;
   if (tile.e >= a.experts) {
     if (count_faults && tile.kind == a.kinds - 1 && part == 0 && threadIdx.x == 0)
-      __hip_atomic_fetch_add(&a.ctrl[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_fetch_add(&a.ctrl[kCtrlBadIds], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     tile.e = -1;
   }
   return tile;
@@ -1178,8 +1186,10 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
                 [&](int ridx, float res) { write_row(dst, ridx, res, mode); });
     }
     fetch_next();
-    if (a.kinds == 2 && kind == 0) publish_h(a, t);
+    if (a.kinds == 2 && kind == 0 && e >= 0) publish_h(a, t);   // a dropped token's word stays untouched
+    if (a.kinds == 2 && kind == 1 && e >= 0) done_waiting(a, t);
   }
+  if (dynamic && threadIdx.x == 0) sub1::leave_launch(a.ctrl, gridDim.x);
 }
 
 // Tokens by expert, for the fused kernel when experts receive several tokens
@@ -1493,6 +1503,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
       }
     }
   }
+  if (threadIdx.x == 0) sub1::leave_launch(a.ctrl, gridDim.x);
 }
 
 // Between the latency form and a token per workgroup: with fewer tokens than
@@ -1540,6 +1551,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_shared_kernel(Prepar
             (ko.slices - part + parts - 1) / parts, xa, partials,
             [&]() { await_activations(a, ko, 1, t, xa); },
             [&](int ridx, float res) { write_row(y, ridx, res, kStore); });
+  done_waiting(a, t);
 }
 
 // For the batches too small to occupy the GPU with a wavefront per slice: built
@@ -1598,8 +1610,10 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_small_kernel(Prepare
       split_run(a, k, walk, xa, dst, mode);
     }
     fetch_next();
-    if (a.kinds == 2 && kind == 0) publish_h(a, t);
+    if (a.kinds == 2 && kind == 0 && e >= 0) publish_h(a, t);
+    if (a.kinds == 2 && kind == 1 && e >= 0) done_waiting(a, t);
   }
+  if (dynamic && threadIdx.x == 0) sub1::leave_launch(a.ctrl, gridDim.x);
 }
 
 // y[t] += W x[t] for many tokens through ONE matrix (matrix 0 of the prepared
@@ -1943,9 +1957,8 @@ double part_passes(int slices, int waves, int groups_max) {
 
 // Launch of the prepared kernels.  kinds == 2: y = wo(relu(wi x)) per token,
 // workspace required; kinds == 1: y += W x per token, no workspace.
-// `piece`: 0 for a caller's launch; 1 and 2 for the first and the later pieces
-// when a launch is split in two (a piece is not split again, and a later piece
-// keeps the fault counts of the first).
+// `piece`: 0 for a caller's launch; 1 and 2 for the two pieces when a launch is
+// split in two (a piece is not split again).
 int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *x, int64_t ldx,
                     void *y, int64_t ldy, int tokens, void *workspace, int64_t workspace_bytes,
                     hipStream_t s, const char *who, int piece = 0, bool may_allocate = true) {
@@ -2009,8 +2022,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   a.groups = nullptr;
   if (p.kinds == 2) {
     a.ctrl = static_cast<int32_t *>(workspace);
-    int64_t ctrl_bytes = (static_cast<int64_t>(kCtrlHeader + tokens) * 4 + 255) / 256 * 256;
-    a.h = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + ctrl_bytes);
+    a.h = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + sub1::control_bytes(tokens));
   }
   a.tokens = tokens;
   a.experts = p.count;
@@ -2219,8 +2231,6 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     const void *fn = reinterpret_cast<const void *>(moe_prepared_shared_kernel);
     HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(lds_shared)));
-    const int nctrl = kCtrlHeader + tokens;
-    zero_words_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl, piece == 2);
     sub1::note_kernel("moe_prepared_shared_kernel");
     moe_prepared_shared_kernel<<<tokens * shared_parts, 64 * waves, lds_shared, s>>>(a);
     HIP_TRY(hipGetLastError());
@@ -2265,7 +2275,6 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
                              : reinterpret_cast<const void *>(moe_prepared_fused_kernel<false, false>);
     HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(lds_fused)));
-    zero_words_kernel<<<1, 256, 0, s>>>(a.ctrl, kCtrlHeader, piece == 2);
     if (grouped) {
       int32_t *tab = reinterpret_cast<int32_t *>(a.h);
       int32_t *order = tab + table_ints;
@@ -2310,10 +2319,6 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
                          : reinterpret_cast<const void *>(moe_prepared_kernel);
   HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                               static_cast<int>(lds)));
-  if (a.ctrl) {
-    int nctrl = kCtrlHeader + tokens;
-    zero_words_kernel<<<(nctrl + 255) / 256, 256, 0, s>>>(a.ctrl, nctrl, piece == 2);
-  }
   if (small) {
     const int64_t grid = tiles < cus ? tiles : cus;
     sub1::note_kernel("moe_prepared_small_kernel");

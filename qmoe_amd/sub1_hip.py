@@ -150,6 +150,15 @@ def sub1decode(dec, w_comp, row_off, ter_minmax, width, want_tern=True, want_w=T
     return tern, w, int(bad.item())
 
 
+def _fault_delta(stack, tokens):
+    # words 1 and 2 of the workspace count over all launches; report what is new
+    key = _stream().value
+    ctrl = stack.workspace(tokens)[:16].view(torch.int32).tolist()
+    before = stack._seen.get(key, (0, 0))
+    stack._seen[key] = (ctrl[1], ctrl[2])
+    return (ctrl[1] - before[0]) & 0xffffffff, (ctrl[2] - before[1]) & 0xffffffff
+
+
 class ExpertStack:
     """The Sub1Linear buffers of all experts of one MoE layer, back to back in
     one set of tensors, and the one-launch forward over them.
@@ -179,6 +188,7 @@ class ExpertStack:
             _need(wo_minmax, torch.bfloat16, 'wo_minmax', dev, numel=experts * 2 * d_model),
             experts, d_model, d_ff)
         self._ws = {}
+        self._seen = {}      # per workspace: the fault counts launch_faults() last returned from
 
     @classmethod
     def from_layers(cls, dec, wi_layers, wo_layers):
@@ -205,16 +215,19 @@ class ExpertStack:
     def workspace(self, tokens):
         """The launch's scratch memory (control words and h), one buffer per
         stream: launches on different streams may run at once, launches on one
-        stream run in order and share theirs.  A buffer that has to grow is
-        replaced; the old one goes back to torch's allocator, which hands it
-        out again only in the order of the stream it was allocated on."""
+        stream run in order and share theirs.  Zeroed when it is made; the
+        launches leave its control words at zero again.  A buffer that has to
+        grow is replaced; the old one goes back to torch's allocator, which
+        hands it out again only in the order of the stream it was allocated on."""
         need = _lib.load().sub1_moe_workspace_bytes(tokens, self.d_ff)
         key = _stream().value
         ws = self._ws.get(key)
         if ws is None or ws.numel() < need:
             with _on_device(self.device):
-                ws = torch.empty(need, dtype=torch.uint8, device=self.device)
+                # zeroed once: every launch leaves its control words at zero again
+                ws = torch.zeros(need, dtype=torch.uint8, device=self.device)
             self._ws[key] = ws
+            self._seen[key] = (0, 0)
         return ws
 
     def forward(self, x, token_expert, y=None):
@@ -251,13 +264,12 @@ class ExpertStack:
         return PreparedStack(self)
 
     def launch_faults(self, tokens):
-        """(waits inside the last forward on this stream that gave up, tokens
-        whose expert id was >= experts and were passed through); both 0 when
-        all is well.  Reads the control words of the workspace, synchronising.
-        A wait that gave up is also reported, sticky, by check_faults() and by
-        the next forward()."""
-        ctrl = self.workspace(tokens)[:16].view(torch.int32).tolist()
-        return ctrl[1], ctrl[2]
+        """(waits that gave up, tokens whose expert id was >= experts and were
+        passed through) in the forwards on this stream since the last call of
+        this method; both 0 when all is well.  Reads the control words of the
+        workspace, synchronising.  A wait that gave up is also reported,
+        sticky, by check_faults() and by the next forward()."""
+        return _fault_delta(self, tokens)
 
     check_faults = staticmethod(_lib.check_faults)
 
@@ -290,20 +302,24 @@ class PreparedStack:
             _lib.check(lib.sub1_moe_prepare_codes(ctypes.byref(stack._c), ctypes.byref(self._c),
                                                   _stream()))
         self._ws = {}
+        self._seen = {}      # per workspace: the fault counts launch_faults() last returned from
 
     def workspace(self, tokens):
         """The launch's scratch memory (control words and h), one buffer per
         stream: launches on different streams may run at once, launches on one
-        stream run in order and share theirs.  A buffer that has to grow is
-        replaced; the old one goes back to torch's allocator, which hands it
-        out again only in the order of the stream it was allocated on."""
+        stream run in order and share theirs.  Zeroed when it is made; the
+        launches leave its control words at zero again.  A buffer that has to
+        grow is replaced; the old one goes back to torch's allocator, which
+        hands it out again only in the order of the stream it was allocated on."""
         need = _lib.load().sub1_moe_workspace_bytes(tokens, self.d_ff)
         key = _stream().value
         ws = self._ws.get(key)
         if ws is None or ws.numel() < need:
             with _on_device(self.device):
-                ws = torch.empty(need, dtype=torch.uint8, device=self.device)
+                # zeroed once: every launch leaves its control words at zero again
+                ws = torch.zeros(need, dtype=torch.uint8, device=self.device)
             self._ws[key] = ws
+            self._seen[key] = (0, 0)
         return ws
 
     def forward(self, x, token_expert, y=None):
@@ -328,8 +344,7 @@ class PreparedStack:
 
     def launch_faults(self, tokens):
         """As ExpertStack.launch_faults."""
-        ctrl = self.workspace(tokens)[:16].view(torch.int32).tolist()
-        return ctrl[1], ctrl[2]
+        return _fault_delta(self, tokens)
 
     check_faults = staticmethod(_lib.check_faults)
 

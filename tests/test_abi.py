@@ -29,7 +29,7 @@ def test_every_declared_symbol_is_exported_and_bound():
         assert hasattr(lib, name), name
         assert name in _lib.PROTOTYPES, name
     assert set(_lib.PROTOTYPES) == names
-    assert lib.sub1_abi_version() == 3
+    assert lib.sub1_abi_version() == 4
 
 
 def test_header_constants_match_binding():
