@@ -211,7 +211,8 @@ def single_matrix_protocol(seed, stream_ptr):
     packed layout (`sub1matvec`, the drop-in call) and the dense product, and
     the reference's wall-clock protocol (synchronise after every call) for the
     drop-in call and the dense product.  Plus 568 tokens through the same
-    matrix in one launch, against the dense GEMM."""
+    matrix in one launch (walking the prepared stream once per four tokens, and
+    on the matrix cores from the tile form), against the dense GEMM."""
     import torch
     from qmoe_amd import sub1, sub1_hip, synthetic
 
@@ -261,6 +262,12 @@ def single_matrix_protocol(seed, stream_ptr):
         xdt = xt.t().contiguous()
         rows[name]['tokens568_prepared_us'] = round(
             time_launches(lambda: pm.matvec_tokens(xt, yt), 100, 10, stream_ptr)[1], 2)
+        # the same 568 tokens on the matrix cores from the tile form (what
+        # Sub1Linear.forward uses from 64 tokens on): weights decoded once per 64 tokens
+        tm = sub1_hip.TiledMatrix(dec, w_comp, row_off, mm, w)
+        rows[name]['tokens568_tiles_us'] = round(
+            time_launches(lambda: tm.matvec_tokens(xt, yt), 100, 10, stream_ptr)[1], 2)
+        rows[name]['tiles_bytes'] = int(tm.entries.numel() + tm.meta.numel())
         rows[name]['tokens568_dense_bf16_us'] = round(
             time_launches(lambda: torch.matmul(dense, xdt, out=ydt), 100, 10, stream_ptr)[1], 2)
     return rows

@@ -322,6 +322,59 @@ int sub1_matrix_prepared_decode(const sub1_matrix_prepared *prepared, int matrix
                                 void *tern_out, void *stream);
 
 /*
+ * Many tokens through one matrix on the matrix cores (no counterpart in the
+ * reference, whose Sub1Linear.forward launches one product per token,
+ * sub1.py:137-142): y[t, :] += W_m x[t, :] for all tokens in one launch, the
+ * weights decoded once per tile of 64 tokens into a dense bf16 tile in LDS and
+ * multiplied by MFMA.  For that the matrices are copied once into a tile form:
+ * rows in their own order in blocks of 64, columns in windows of 128, per
+ * (block, window) and row the non-zero weights inside the window as one byte
+ * each ((column in the window) * 2 + symbol - 1), eight to an 8-byte chunk
+ * interleaved by lane like the prepared stream (about 1.1 to 1.6 bit per
+ * weight at 10% non-zeros).  Worth it from a few dozen tokens on; below that
+ * sub1_matvec_tokens or sub1_matvec_prepared walk the non-zeros per token.
+ * Products are exact and summed in fp32 in the matrix cores' order: results
+ * agree with the other kernels to rounding (1e-2 bar), not to the bit.
+ *
+ *   meta_bytes = sub1_tiles_meta_bytes(count, height, width);
+ *   sub1_tiles t;
+ *   sub1_tiles_layout(&set, meta, meta_bytes, &t, stream);      // synchronises; sets t.entry_bytes
+ *   t.entries = <device buffer of t.entry_bytes bytes>;
+ *   sub1_tiles_entries(&set, &t, stream);
+ *   sub1_matvec_tiles(&t, matrix, x, ldx, y, ldy, tokens, stream);
+ *
+ * meta and entries are device buffers the caller owns, 256-byte aligned; the
+ * source matrices are not referenced after sub1_tiles_entries has run.  Any
+ * dictionary with symbols 0..2; any height and width.  x rows are read 16 bytes
+ * at a time when x is 16-byte aligned and ldx a multiple of 8 (else element by
+ * element, slower).  sub1_tiles_decode writes one matrix's symbols, read back
+ * from the tile form, to tern_out (uint8 [height, width]): the check that the
+ * copy kept every weight.
+ */
+typedef struct sub1_tiles {
+  const void *meta;
+  const void *entries;
+  int64_t meta_bytes;
+  int64_t entry_bytes;
+  int64_t total_chunks;    /* 512-byte chunk rows of all segments */
+  int32_t count;
+  int32_t height;
+  int32_t width;
+} sub1_tiles;
+
+int64_t sub1_tiles_meta_bytes(int count, int height, int width);
+
+int sub1_tiles_layout(const sub1_matrix_set *set, void *meta, int64_t meta_bytes, sub1_tiles *tiles,
+                      void *stream);
+
+int sub1_tiles_entries(const sub1_matrix_set *set, const sub1_tiles *tiles, void *stream);
+
+int sub1_matvec_tiles(const sub1_tiles *tiles, int matrix, const void *x, int64_t ldx, void *y,
+                      int64_t ldy, int tokens, void *stream);
+
+int sub1_tiles_decode(const sub1_tiles *tiles, int matrix, void *tern_out, void *stream);
+
+/*
  * Average duration in microseconds of the most recent launches, measured with
  * HIP events on the launch stream: call sub1_timing_begin(stream) before and
  * sub1_timing_end(stream, &us) after a run of launches (end synchronises).

@@ -47,6 +47,13 @@ class MatrixPrepared(ctypes.Structure):
                 ('width', ctypes.c_int32), ('max_chunks', ctypes.c_int32)]
 
 
+class Tiles(ctypes.Structure):
+    """struct sub1_tiles"""
+    _fields_ = [('meta', _vp), ('entries', _vp), ('meta_bytes', _i64), ('entry_bytes', _i64),
+                ('total_chunks', _i64), ('count', ctypes.c_int32), ('height', ctypes.c_int32),
+                ('width', ctypes.c_int32)]
+
+
 # every symbol include/sub1_hip.h declares, with its prototype
 PROTOTYPES = {
     'sub1_last_error': (ctypes.c_char_p, []),
@@ -79,6 +86,11 @@ PROTOTYPES = {
     'sub1_matvec_prepared': (_int, [ctypes.POINTER(MatrixPrepared), _vp, _vp, _i64, _vp, _i64,
                                     _int, _vp]),
     'sub1_matrix_prepared_decode': (_int, [ctypes.POINTER(MatrixPrepared), _int, _vp, _vp]),
+    'sub1_tiles_meta_bytes': (_i64, [_int, _int, _int]),
+    'sub1_tiles_layout': (_int, [ctypes.POINTER(MatrixSet), _vp, _i64, ctypes.POINTER(Tiles), _vp]),
+    'sub1_tiles_entries': (_int, [ctypes.POINTER(MatrixSet), ctypes.POINTER(Tiles), _vp]),
+    'sub1_matvec_tiles': (_int, [ctypes.POINTER(Tiles), _int, _vp, _i64, _vp, _i64, _int, _vp]),
+    'sub1_tiles_decode': (_int, [ctypes.POINTER(Tiles), _int, _vp, _vp]),
     'sub1_timing_begin': (_int, [_vp]),
     'sub1_timing_end': (_int, [_vp, ctypes.POINTER(ctypes.c_double)]),
     'sub1_init': (_int, []),

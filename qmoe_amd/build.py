@@ -7,6 +7,7 @@ ROOT = os.path.dirname(HERE)
 LIB_PATH = os.path.join(HERE, 'libsub1_hip.so')
 SOURCES = [os.path.join(HERE, 'csrc', 'sub1_kernels.hip'),
            os.path.join(HERE, 'csrc', 'sub1_prepared.hip'),
+           os.path.join(HERE, 'csrc', 'sub1_tiles.hip'),
            os.path.join(HERE, 'csrc', 'sub1_tables.cpp')]
 
 HIPCC_FLAGS = [

@@ -57,26 +57,34 @@ class Sub1Linear(nn.Module):
         self.register_buffer('ter_minmax', torch.zeros(2 * height, dtype=torch.bfloat16))
         self.register_buffer('weight', torch.zeros(0, dtype=torch.bfloat16))
 
-    # forward() goes through the prepared stream of the non-zero weights, made
-    # from the codes on first use (it costs about as much memory again as w_comp
-    # and is remade when a buffer is replaced or written in place).  Set to
-    # False to run straight from the packed buffers instead (the two add a
-    # row's terms in different orders and agree to rounding, not to the bit).
+    # forward() goes through copies of the weights made from the codes on first
+    # use (each costs about as much memory again as w_comp and is remade when a
+    # buffer is replaced or written in place): for up to `tile_tokens` - 1 tokens
+    # the prepared stream of the non-zero weights, walked per token; from
+    # `tile_tokens` tokens on the tile form that the matrix cores multiply from,
+    # the weights decoded once per 64 tokens.  Set `fast` to False to run
+    # straight from the packed buffers instead.  (The three add a row's terms in
+    # different orders and agree to rounding, not to the bit.)
     fast = True
+    tile_tokens = 64
 
-    def _prepared(self, width):
+    def _copy(self, kind, width):
         live = (self.w_comp, self.row_off, self.ter_minmax)
         key = tuple((t.data_ptr(), t._version, t.numel()) for t in live) + (width,)
-        cached = getattr(self, '_prepared_cache', None)
+        cache = self.__dict__.setdefault('_copies', {})
+        cached = cache.get(kind)
         if cached is None or cached[0] != key:
             table = DEC[self.w_comp.device.index]
+            make = sub1_hip.PreparedMatrix if kind == 'prepared' else sub1_hip.TiledMatrix
             # the entry keeps the source tensors alive: their addresses are part
             # of the key and must not be handed out again while it is cached
-            cached = (key, sub1_hip.PreparedMatrix(table, self.w_comp, self.row_off,
-                                                   self.ter_minmax, width),
+            cached = (key, make(table, self.w_comp, self.row_off, self.ter_minmax, width),
                       [t.detach() for t in live])
-            self._prepared_cache = cached
+            cache[kind] = cached
         return cached[1]
+
+    def _prepared(self, width):
+        return self._copy('prepared', width)
 
     def forward(self, x):
         """x bf16 [T, width] -> bf16 [T, height] (reference sub1.py:132-143)."""
@@ -85,7 +93,9 @@ class Sub1Linear(nn.Module):
         if x.shape[0] == 0:
             return y
         x = x.contiguous()
-        if self.fast and x.shape[1] <= sub1_hip.PREPARED_MAX_WIDTH:
+        if self.fast and x.shape[0] >= self.tile_tokens:
+            self._copy('tiles', x.shape[1]).matvec_tokens(x, y)
+        elif self.fast and x.shape[1] <= sub1_hip.PREPARED_MAX_WIDTH:
             self._prepared(x.shape[1]).matvec_tokens(x, y)
         else:
             table = DEC[self.w_comp.device.index]
@@ -268,7 +278,7 @@ class FasterMLP(nn.Module):
                 for name in ('w_comp', 'row_off', 'ter_minmax'):
                     old = getattr(layer, name)
                     setattr(layer, name, torch.zeros(0, dtype=old.dtype, device=old.device))
-                layer._prepared_cache = None
+                layer.__dict__.pop("_copies", None)
 
     def _forget(self):
         if getattr(self, '_released', False):

@@ -426,3 +426,65 @@ class PreparedMatrix:
             _lib.check(_lib.load().sub1_matrix_prepared_decode(
                 ctypes.byref(self._c), matrix, out.data_ptr(), _stream()))
         return out
+
+
+class TiledMatrix:
+    """Compressed matrices of one shape copied into the tile form that the
+    matrix cores multiply from; `matvec_tokens(x, y)` does y[t] += W x[t] for
+    all tokens of x [T, width] in one launch, the weights decoded once per
+    tile of 64 tokens (made for sequences: from a few dozen tokens on it beats
+    walking the non-zeros per token; results agree with the other paths to
+    rounding, not to the bit).  Arguments as PreparedMatrix."""
+
+    def __init__(self, dec, w_comp, row_off, ter_minmax, width, code_base=None):
+        lib = _lib.load()
+        dev = dec.device
+        if isinstance(w_comp, (list, tuple)):
+            sizes = torch.tensor([0] + [t.numel() for t in w_comp], dtype=torch.int64)
+            code_base = sizes.cumsum(0)[:-1].to(dev)
+            w_comp, row_off, ter_minmax = (torch.cat(list(v)) for v in (w_comp, row_off, ter_minmax))
+        count = 1 if code_base is None else code_base.numel()
+        if row_off.numel() % count:
+            raise ValueError('row_off does not hold %d equal parts' % count)
+        height = row_off.numel() // count - 1
+        self.device, self.count, self.height, self.width = dev, count, height, width
+        src = _lib.MatrixSet(
+            _need(dec, torch.int32, 'dec', numel=_lib.DEC_WORDS),
+            _need(w_comp, torch.int16, 'w_comp', dev),
+            None if code_base is None else _need(code_base, torch.int64, 'code_base', dev),
+            _need(row_off, torch.int32, 'row_off', dev, numel=count * (height + 1)),
+            _need(ter_minmax, torch.bfloat16, 'ter_minmax', dev, numel=count * 2 * height),
+            count, height, width)
+        meta_bytes = lib.sub1_tiles_meta_bytes(count, height, width)
+        if meta_bytes <= 0:
+            raise ValueError('bad matrix dimensions')
+        self.meta = torch.empty(meta_bytes, dtype=torch.uint8, device=dev)
+        self._c = _lib.Tiles()
+        with _on_device(dev):
+            _lib.check(lib.sub1_tiles_layout(ctypes.byref(src), self.meta.data_ptr(), meta_bytes,
+                                             ctypes.byref(self._c), _stream()))
+            self.entries = torch.empty(max(self._c.entry_bytes, 256), dtype=torch.uint8, device=dev)
+            self._c.entries = self.entries.data_ptr()
+            _lib.check(lib.sub1_tiles_entries(ctypes.byref(src), ctypes.byref(self._c), _stream()))
+
+    def matvec_tokens(self, x, y, matrix=0):
+        dev = self.device
+        p_x = _need(x, torch.bfloat16, 'x', dev, dim=2)
+        p_y = _need(y, torch.bfloat16, 'y', dev, dim=2)
+        tokens = x.shape[0]
+        if x.shape[1] != self.width or y.shape != (tokens, self.height):
+            raise ValueError('x must be [T, %d] and y [T, %d]' % (self.width, self.height))
+        if tokens == 0:
+            return
+        with _on_device(dev):
+            _lib.check(_lib.load().sub1_matvec_tiles(
+                ctypes.byref(self._c), matrix, p_x, self.width, p_y, self.height, tokens, _stream()))
+
+    def decode(self, matrix=0):
+        """uint8 [height, width]: the symbols of one matrix read back from the
+        tile form."""
+        out = torch.empty(self.height, self.width, dtype=torch.uint8, device=self.device)
+        with _on_device(self.device):
+            _lib.check(_lib.load().sub1_tiles_decode(ctypes.byref(self._c), matrix, out.data_ptr(),
+                                                     _stream()))
+        return out

@@ -1,0 +1,156 @@
+"""Many tokens through one matrix on the matrix cores (the tile form and
+matvec_tiles_kernel): the tile form must hold every weight (decoded back,
+bit-exact against the oracle's decode of the codes), and the products must lie
+within the fp32 error bound of the double-precision product and within the
+stated 1e-2 of the reference kernel's lane-order arithmetic.  Bit-equality with
+the row-walking kernels is not claimed: the matrix cores add in their own
+order."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import sub1_oracle as so
+from test_gpu_parity import REL_TOL, bf16_dev, bits_host, dev_case
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope='module')
+def gpu():
+    from qmoe_amd import sub1, sub1_hip
+    assert torch.cuda.is_available() and sub1.DEC
+    return sub1, sub1_hip
+
+
+def check_tokens(oracle, c, xs, pre, got, rows):
+    """Tokens `rows` of the launch against the oracle: error bound against the
+    double-precision product, 1e-2 against the lane-order result, on top of
+    what y held before."""
+    for i in rows:
+        exact, sum_abs = oracle.matvec_f64(c['t'].astype(np.uint8), c['mm'], xs[i])
+        # y_new = bf16(y_old + bf16(res)): two bf16 roundings and the fp32 sum's own error
+        y_old = so.bf16_bits_to_f32(pre[i]).astype(np.float64)
+        y = so.bf16_bits_to_f32(got[i]).astype(np.float64)
+        bound = (2.0 ** -8 * np.abs(exact) + 64 * 2.0 ** -24 * sum_abs
+                 + 2.0 ** -8 * np.abs(y_old + exact) + 1e-30)
+        assert np.all(np.abs(y - (y_old + exact)) <= bound), i
+        lanes = so.bf16_bits_to_f32(oracle.matvec_lanes(c['codes'], c['row_off'], c['mm'], xs[i],
+                                                        y=pre[i])).astype(np.float64)
+        assert np.linalg.norm(y - lanes) <= REL_TOL * max(np.linalg.norm(lanes), 1e-30), i
+
+
+@pytest.mark.parametrize('height,width,p0,tokens', [
+    (3072, 768, 0.9, 568), (768, 3072, 0.9, 200), (4096, 1024, 0.88, 64), (1024, 4096, 0.88, 129),
+    (6144, 2080, 0.9, 70), (2080, 6144, 0.9, 65),
+    (77, 333, 0.7, 100),          # ragged rows, columns and tokens; odd width: x rows unaligned
+    (130, 15, 0.3, 64), (1, 4000, 0.95, 3), (200, 129, 0.0, 67), (64, 128, 0.5, 1)])
+def test_tiles_product(gpu, oracle, height, width, p0, tokens):
+    sub1, op = gpu
+    c = dev_case(oracle, height, width, p0, seed=11 * height + width + tokens)
+    tm = op.TiledMatrix(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], width)
+    # the copy holds every weight
+    assert np.array_equal(tm.decode().cpu().numpy(), c['t'].astype(np.uint8))
+    rng = np.random.default_rng(tokens + width)
+    xs = so.f32_to_bf16_bits(rng.standard_normal((tokens, width)).astype(np.float32))
+    pre = so.f32_to_bf16_bits(rng.standard_normal((tokens, height)).astype(np.float32))
+    y = bf16_dev(pre).clone()
+    tm.matvec_tokens(bf16_dev(xs), y)
+    got = bits_host(y)
+    rows = sorted(set(list(range(0, tokens, 41)) + [tokens - 1, min(63, tokens - 1),
+                                                    min(64, tokens - 1)]))
+    check_tokens(oracle, c, xs, pre, got, rows)
+    # the same launch again gives the same bits, and so does any split of the
+    # tokens into launches (a token's result does not depend on its tile mates)
+    y2 = bf16_dev(pre).clone()
+    tm.matvec_tokens(bf16_dev(xs), y2)
+    assert torch.equal(y, y2)
+    y3 = bf16_dev(pre).clone()
+    xd = bf16_dev(xs)
+    for lo in range(0, tokens, 50):
+        tm.matvec_tokens(xd[lo:lo + 50].contiguous(), y3[lo:lo + 50])
+    assert torch.equal(y, y3)
+    # agreement with the row-walking kernel on the prepared stream, to rounding
+    if width <= op.PREPARED_MAX_WIDTH:
+        pm = op.PreparedMatrix(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], width)
+        y4 = bf16_dev(pre).clone()
+        pm.matvec_tokens(xd, y4)
+        a, b = y.float().double(), y4.float().double()
+        assert torch.linalg.norm(a - b) <= REL_TOL * torch.linalg.norm(b)
+
+
+def test_tiles_closed_forms(gpu, oracle):
+    """Unit vectors pick a column exactly; zero activations leave y as it was;
+    doubling the activations doubles the product exactly (y zero before)."""
+    sub1, op = gpu
+    height, width, tokens = 96, 300, 70
+    c = dev_case(oracle, height, width, 0.6, seed=4321)
+    tm = op.TiledMatrix(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], width)
+    w = so.bf16_bits_to_f32(oracle.dequant(c['t'].astype(np.uint8), c['mm']))
+    one = so.f32_to_bf16_bits(np.array([1.0], np.float32))[0]
+    xs = np.zeros((tokens, width), dtype=np.uint16)
+    cols = [(7 * i) % width for i in range(tokens)]
+    for i, k in enumerate(cols):
+        xs[i, k] = one
+    y = torch.zeros((tokens, height), dtype=torch.bfloat16, device='cuda')
+    tm.matvec_tokens(bf16_dev(xs), y)
+    got = so.bf16_bits_to_f32(bits_host(y))
+    for i, k in enumerate(cols):
+        assert np.array_equal(got[i], w[:, k]), (i, k)
+    pre = so.f32_to_bf16_bits(np.random.default_rng(1).standard_normal((tokens, height)).astype(np.float32))
+    y = bf16_dev(pre).clone()
+    tm.matvec_tokens(torch.zeros((tokens, width), dtype=torch.bfloat16, device='cuda'), y)
+    assert np.array_equal(bits_host(y), pre)
+    x = torch.randn((tokens, width), generator=torch.Generator().manual_seed(2)).bfloat16().cuda()
+    y1 = torch.zeros((tokens, height), dtype=torch.bfloat16, device='cuda')
+    y2 = torch.zeros_like(y1)
+    tm.matvec_tokens(x, y1)
+    tm.matvec_tokens(x * 2, y2)
+    assert torch.equal(y2, y1 * 2)
+
+
+def test_tiles_matrix_set_and_arguments(gpu, oracle):
+    """Several matrices in one tile buffer; arguments are checked."""
+    sub1, op = gpu
+    from qmoe_amd._lib import Sub1Error
+    height, width, count, tokens = 130, 200, 3, 80
+    cases = [dev_case(oracle, height, width, 0.8, seed=650 + i) for i in range(count)]
+    tm = op.TiledMatrix(sub1.DEC[0], [c['w_comp'] for c in cases], [c['row_off_d'] for c in cases],
+                        [c['mm_d'] for c in cases], width)
+    rng = np.random.default_rng(9)
+    xs = so.f32_to_bf16_bits(rng.standard_normal((tokens, width)).astype(np.float32))
+    pre = np.zeros((tokens, height), dtype=np.uint16)
+    for m, c in enumerate(cases):
+        assert np.array_equal(tm.decode(m).cpu().numpy(), c['t'].astype(np.uint8))
+        y = torch.zeros((tokens, height), dtype=torch.bfloat16, device='cuda')
+        tm.matvec_tokens(bf16_dev(xs), y, matrix=m)
+        check_tokens(oracle, c, xs, pre, bits_host(y), [0, 63, 64, 79])
+    y = torch.zeros((tokens, height), dtype=torch.bfloat16, device='cuda')
+    with pytest.raises(Sub1Error):
+        tm.matvec_tokens(bf16_dev(xs), y, matrix=3)
+    with pytest.raises(ValueError):
+        tm.matvec_tokens(bf16_dev(xs)[:, :-1].contiguous(), y)
+    bad = cases[0]['row_off_d'].clone()
+    bad[40] -= 1
+    with pytest.raises(Sub1Error):
+        op.TiledMatrix(sub1.DEC[0], cases[0]['w_comp'], bad, cases[0]['mm_d'], width)
+
+
+def test_sub1linear_takes_the_tiles_from_64_tokens_on(gpu, oracle):
+    """Sub1Linear.forward on a sequence: the tile form from `tile_tokens` tokens
+    on, the prepared stream below; both within the tolerance of the dense
+    product, and the tile copy follows the buffers like the prepared one."""
+    sub1, op = gpu
+    from qmoe_amd import _lib
+    t, mm = so.synthetic_ternary(320, 512, 0.85, seed=77)
+    w = bf16_dev(oracle.dequant(t.astype(np.uint8), mm))
+    lin = sub1.Sub1Linear.make(w)
+    x = torch.randn((100, 512), generator=torch.Generator().manual_seed(3)).bfloat16().cuda()
+    ref = x.float() @ w.float().t()
+    y = lin(x)
+    assert _lib.load().sub1_last_kernel() == b'matvec_tiles_kernel'
+    assert torch.linalg.norm(y.float() - ref) <= REL_TOL * torch.linalg.norm(ref)
+    y_few = lin(x[:10])
+    assert _lib.load().sub1_last_kernel() != b'matvec_tiles_kernel'
+    assert torch.linalg.norm(y_few.float() - ref[:10]) <= REL_TOL * torch.linalg.norm(ref[:10])
+    lin.ter_minmax = (lin.ter_minmax.float() * 2).bfloat16()
+    assert torch.equal(lin(x).float(), 2 * y.float())
