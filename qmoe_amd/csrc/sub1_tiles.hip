@@ -1,37 +1,44 @@
 // Many tokens through one compressed matrix on the matrix cores.
 //
 // Sub1Linear.forward on a sequence (reference sub1.py:132-143 launches one
-// product per token and calls that "naive") is a skinny GEMM Y += X W^T: the
-// weights are decoded ONCE per tile of 64 tokens into a dense bf16 tile in LDS
-// and multiplied with the tokens' activations by v_mfma_f32_32x32x16_bf16,
-// instead of walking the non-zeros once per token (or per four tokens) as the
-// row-walking kernels do; the work no longer grows with tokens x non-zeros.
+// product per token and calls that "naive") is a skinny GEMM Y += X W^T, and
+// the matrix cores do it (v_mfma_f32_32x32x16_bf16) once the ternary weights
+// are bf16 values again.  Nothing is walked per token and nothing is scattered:
+// the work no longer grows with tokens x non-zeros.
 //
 // The tile form of a matrix (sub1_tiles_*) is made for that, once, from the
-// packed codes:
-//   * rows stay in their own order, in blocks of 64 (a lane per row), so a
-//     tile's outputs are 64 consecutive rows of y: coalesced read-modify-writes;
-//   * columns are cut into windows of 128; a (block, window) segment lists, per
-//     lane, the row's non-zero weights inside the window as one byte each,
-//     (column in the window) * 2 + (symbol - 1), eight to a chunk of 8 bytes,
-//     chunk c of lane l at ((segment base + c) * 64 + l) * 8 bytes as in the
-//     prepared stream; a segment is as long as its fullest lane, each lane's
-//     own count says where its bytes end;
-//   * (min, max) per row, copied.
-// Segments are independent, so a wavefront decodes a window with no state
-// carried over from the windows before it.
+// packed codes: 2 bits per weight, whatever the density, cut into units of
+// 32 rows x 128 columns of 64 x 16 bytes.  In unit (u, w) lane l = 32 h + r
+// holds the weights of row 32 u + r that it feeds the matrix core as its share
+// of the B operand: in step s (0..7) of the window the eight columns
+// 128 w + 16 s + 8 h + q.  Word s / 2 of its 16 bytes holds steps s and s + 1;
+// the weight of step s = 2 m + e and q = 2 k + o sits in bits
+// 16 o + 8 e + 2 k (+1) of word m, as 0 (the row's min), 1 (its max) or 2
+// (zero).  A wavefront fetches a unit with one coalesced 16-byte load per
+// lane.  Rows are padded to a multiple of 64 and columns to a multiple of 128
+// with zeros; (min, max) per row are copied.
 //
-// Kernel: a workgroup of four wavefronts owns 64 rows x 64 tokens.  Wavefront v
-// takes the windows v, v + 4, ...: it zeroes its weight tile, writes the window's
-// weights into it (bf16 values of the row's min or max), copies the tokens'
-// activations of the same 128 columns next to it, and multiplies the two
-// 64 x 128 tiles into its own 64 x 64 fp32 accumulators (2 x 2 MFMA blocks, one
-// LDS read per MFMA).  The wavefronts never wait for each other inside the
-// loop; at the end the four partial tiles are added through LDS in wavefront
+// From the codes to bf16 pairs without a table: (word >> 2 k) & 0x00030003
+// times 0x0202 plus 0x01000100 is a byte selector that picks, out of the row's
+// (min, max) word and a zero word, the two weights of pair k (v_perm_b32):
+// four plain instructions per pair of weights.
+//
+// Kernel: a workgroup owns 64 rows x 64 tokens; its wavefronts split the
+// windows of 128 columns among themselves (wavefront v takes v, v + n, ...).  Per
+// window a wavefront copies the tokens' activations, 64 x 128, through
+// registers into its own 16 KB of LDS (coalesced 16-byte loads, four tokens an
+// instruction; the 16-byte pieces of a token are XOR-swizzled with the token's
+// number so that neither the stores nor the operand reads meet in a bank), and
+// per step of 16 columns reads its A operands from there, builds its B
+// operands from the codes and adds into a 64 x 64 fp32 accumulator (2 x 2 MFMA
+// blocks).  The loads of the next window are issued as soon as the registers
+// are free, a whole window ahead.  All of them are buffer loads: what lies past
+// the last token, past the width or past a wavefront's last window is given an
+// offset outside the buffer and comes back as zeros, without a branch or a
+// mask.  At the end the partial tiles are added through LDS in wavefront
 // order, rounded to bf16 and added onto y in bf16 (reference
-// sub1_cuda_kernel.cu:199-200).  The loads of a wavefront's next window (its
-// chunks, its counts, the activations) are requested before it works on the
-// current one.
+// sub1_cuda_kernel.cu:199-200).  The number of wavefronts depends on the matrix
+// alone, so a token's result does not depend on the launch it is part of.
 //
 // Results: each product x * w is exact in fp32 and the sums are fp32, but in
 // the matrix cores' own order; they agree with the row-walking kernels and the
@@ -50,29 +57,26 @@ using sub1::f32_to_bf16;
 using sub1::fail;
 using sub1::misaligned;
 
-constexpr int kRows = 64;                 // rows per block, a lane each
+constexpr int kUnitRows = 32;             // rows per unit
+constexpr int kRows = 64;                 // rows per workgroup: two units
 constexpr int kCols = 128;                // columns per window
-constexpr int kPerChunk = 8;              // entries (bytes) per chunk
 constexpr int kTokens = 64;               // tokens per workgroup
-constexpr int kWaves = 4;                 // wavefronts per workgroup
-// bf16 elements per LDS row of a tile: 272 bytes, so that the 16-byte operand
-// reads of 32 consecutive rows fall into all banks evenly
-constexpr int kStride = kCols + 8;
-constexpr int kTileElems = kRows * kStride;
-constexpr size_t kTilesLds = static_cast<size_t>(kWaves) * 2 * kTileElems * sizeof(uint16_t);
-constexpr int kAhead = 4;                 // chunks of the next window requested ahead
+constexpr int kSteps = kCols / 16;        // MFMA steps per window
+constexpr int kMaxWaves = 8;              // wavefronts per workgroup, at most
+constexpr uint32_t kAllZero = 0xaaaaaaaau; // a word of codes of zero weights
+constexpr int kPartialBytes = kTokens * kRows * 4;   // one wavefront's scaled tile
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 
-// One block of device memory, arrays back to back, each 256-byte aligned.
+// The meta block: arrays back to back, each 256-byte aligned.
 struct TileLayout {
-  int blocks, windows;
-  int64_t segments;
-  int64_t seg_base;   // i32 [segments + 1]: chunk counts, scanned in place
-  int64_t cnt;        // u8  [segments * 64]: entries of every lane
+  int units_down;     // units of 32 rows per matrix, even
+  int windows;
+  int64_t units;      // of all matrices
   int64_t minmax;     // u32 [count * height]
   int64_t status;     // i32 [4]: [0] rows whose codes do not cover the width
   int64_t bytes;
@@ -80,17 +84,15 @@ struct TileLayout {
 
 TileLayout tile_layout(int count, int height, int width) {
   TileLayout t;
-  t.blocks = (height + kRows - 1) / kRows;
+  t.units_down = (height + kRows - 1) / kRows * (kRows / kUnitRows);
   t.windows = (width + kCols - 1) / kCols;
-  t.segments = static_cast<int64_t>(count) * t.blocks * t.windows;
+  t.units = static_cast<int64_t>(count) * t.units_down * t.windows;
   int64_t off = 0;
   auto take = [&](int64_t bytes) {
     int64_t o = off;
     off += align256(bytes);
     return o;
   };
-  t.seg_base = take((t.segments + 1) * 4);
-  t.cnt = take(t.segments * kRows);
   t.minmax = take(static_cast<int64_t>(count) * height * 4);
   t.status = take(16);
   t.bytes = off;
@@ -136,135 +138,87 @@ __device__ __forceinline__ const uint16_t *codes_of(const RowSource &s, int m, i
   return s.w_comp + (s.code_base ? s.code_base[m] : 0) + ro[r];
 }
 
-// One thread per lane of every block: the entries of its row in every window.
-__global__ __launch_bounds__(256) void tile_count_kernel(RowSource s, int blocks, int windows,
-                                                         uint8_t *__restrict__ cnt,
-                                                         int32_t *__restrict__ status,
-                                                         int64_t lanes_total) {
+// Where the weight of column c of a window sits in its lane's 16 bytes.
+__device__ __forceinline__ void code_place(int c, int &half, int &word, int &shift) {
+  const int step = c >> 4, q = c & 7;
+  half = (c >> 3) & 1;
+  word = step >> 1;
+  shift = 16 * (q & 1) + 8 * (step & 1) + 2 * (q >> 1);
+}
+
+// One thread per row of every matrix: its codes into the units (all zero
+// weights before).
+__global__ __launch_bounds__(256) void code_emit_kernel(RowSource s, int units_down, int windows,
+                                                        u32x4 *__restrict__ units,
+                                                        int32_t *__restrict__ status,
+                                                        int64_t rows_total) {
   const int64_t gl = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (gl >= lanes_total) return;
-  const int lane = static_cast<int>(gl & 63);
-  const int64_t mb = gl >> 6;                 // matrix * blocks + block
-  const int m = static_cast<int>(mb / blocks);
-  const int r = static_cast<int>(mb % blocks) * kRows + lane;
-  uint8_t *mine = cnt + mb * windows * kRows + lane;   // [window * 64]
-  int w_cur = 0, n_cur = 0;
-  auto flush_to = [&](int w) {
-    while (w_cur < w) {
-      mine[static_cast<int64_t>(w_cur) * kRows] = static_cast<uint8_t>(n_cur);
-      n_cur = 0;
-      w_cur++;
-    }
+  if (gl >= rows_total) return;
+  const int m = static_cast<int>(gl / s.height);
+  const int r = static_cast<int>(gl % s.height);
+  u32x4 *mine = units + (static_cast<int64_t>(m) * units_down + r / kUnitRows) * windows * 64 +
+                r % kUnitRows;
+  uint32_t held[2][4];   // [half][word] of the window at hand
+  int w_cur = 0;
+  bool dirty = false;
+  auto clear = [&]() {
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+      for (int d = 0; d < 4; d++) held[h][d] = kAllZero;
+    dirty = false;
   };
-  if (r < s.height) {
-    int n;
-    const uint16_t *codes = codes_of(s, m, r, n);
-    const int covered = each_nonzero(codes, n, s.dec, s.width, [&](int col, int) {
-      flush_to(col / kCols);
-      n_cur++;
-    });
-    if (covered != ((s.width + 1) & ~1)) atomicAdd(&status[0], 1);
-  }
-  flush_to(windows);
-}
-
-// One thread per segment: its chunks are those of its fullest lane.
-__global__ __launch_bounds__(256) void tile_segments_kernel(const uint8_t *__restrict__ cnt,
-                                                            int32_t *__restrict__ counts,
-                                                            int64_t segments) {
-  const int64_t g = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (g >= segments) return;
-  const uint4 *p = reinterpret_cast<const uint4 *>(cnt + g * kRows);
-  uint32_t most = 0;
-  for (int i = 0; i < kRows / 16; i++) {
-    const uint4 v = p[i];
-    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-    for (int j = 0; j < 4; j++)
-      for (int k = 0; k < 4; k++) most = max(most, (w[j] >> (8 * k)) & 255u);
-  }
-  counts[g + 1] = static_cast<int32_t>((most + kPerChunk - 1) / kPerChunk);
-}
-
-// In-place inclusive prefix sum over v[1..n], v[0] = 0; one workgroup.
-__global__ __launch_bounds__(1024) void tile_scan_kernel(int32_t *__restrict__ v, int64_t n) {
-  __shared__ int32_t part[1024];
-  const int tid = threadIdx.x;
-  const int64_t seg = (n + 1023) / 1024;
-  const int64_t lo = 1 + tid * seg;
-  const int64_t hi = min(n + 1, lo + seg);
-  int32_t s = 0;
-  for (int64_t i = lo; i < hi; i++) s += v[i];
-  part[tid] = s;
-  __syncthreads();
-  for (int d = 1; d < 1024; d *= 2) {
-    int32_t t = tid >= d ? part[tid - d] : 0;
-    __syncthreads();
-    part[tid] += t;
-    __syncthreads();
-  }
-  int32_t run = tid ? part[tid - 1] : 0;
-  if (tid == 0) v[0] = 0;
-  for (int64_t i = lo; i < hi; i++) {
-    run += v[i];
-    v[i] = run;
-  }
-}
-
-// One thread per lane of every block: its entries into the segments.
-__global__ __launch_bounds__(256) void tile_emit_kernel(RowSource s, int blocks, int windows,
-                                                        const int32_t *__restrict__ seg_base,
-                                                        uint8_t *__restrict__ dst,
-                                                        int64_t lanes_total) {
-  const int64_t gl = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (gl >= lanes_total) return;
-  const int lane = static_cast<int>(gl & 63);
-  const int64_t mb = gl >> 6;
-  const int m = static_cast<int>(mb / blocks);
-  const int r = static_cast<int>(mb % blocks) * kRows + lane;
-  if (r >= s.height) return;
+  auto flush = [&]() {
+    if (dirty) {
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        u32x4 v = {held[h][0], held[h][1], held[h][2], held[h][3]};
+        mine[static_cast<int64_t>(w_cur) * 64 + h * kUnitRows] = v;
+      }
+    }
+    clear();
+  };
+  clear();
   int n;
   const uint16_t *codes = codes_of(s, m, r, n);
-  int w_cur = -1, i = 0;
-  int64_t base = 0;
-  each_nonzero(codes, n, s.dec, s.width, [&](int col, int sym) {
+  const int covered = each_nonzero(codes, n, s.dec, s.width, [&](int col, int sym) {
     const int w = col / kCols;
     if (w != w_cur) {
+      flush();
       w_cur = w;
-      i = 0;
-      base = seg_base[mb * windows + w];
     }
-    dst[((base + i / kPerChunk) * kRows + lane) * 8 + i % kPerChunk] =
-        static_cast<uint8_t>(((col - w * kCols) << 1) | (sym - 1));
-    i++;
+    int half, word, shift;
+    code_place(col % kCols, half, word, shift);
+    // symbol 1 (min) is code 0, symbol 2 (max) code 1; the place holds 2 (zero)
+    const uint32_t flip = (sym == 2 ? 3u : 2u) << shift;
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+      for (int d = 0; d < 4; d++)
+        if (h == half && d == word) held[h][d] ^= flip;
+    dirty = true;
   });
+  flush();
+  if (covered != ((s.width + 1) & ~1)) atomicAdd(&status[0], 1);
 }
 
-// The symbols of one matrix back out of its tile form: out[row, column] = 1 or
-// 2 at every entry; out is zero before.
-__global__ __launch_bounds__(256) void tile_decode_kernel(const uint8_t *__restrict__ entries,
-                                                          const int32_t *__restrict__ seg_base,
-                                                          const uint8_t *__restrict__ cnt,
+// The symbols of one matrix back out of its units, a thread per weight.
+__global__ __launch_bounds__(256) void code_decode_kernel(const u32x4 *__restrict__ units,
                                                           uint8_t *__restrict__ out, int matrix,
-                                                          int blocks, int windows, int height,
+                                                          int units_down, int windows, int height,
                                                           int width) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= blocks * kRows) return;
-  const int lane = t & 63, r = t;
-  if (r >= height) return;
-  const int64_t mb = static_cast<int64_t>(matrix) * blocks + (t >> 6);
-  for (int w = 0; w < windows; w++) {
-    const int64_t g = mb * windows + w;
-    const int n = cnt[g * kRows + lane];
-    const int64_t base = seg_base[g];
-    for (int i = 0; i < n; i++) {
-      const uint8_t e = entries[((base + i / kPerChunk) * kRows + lane) * 8 + i % kPerChunk];
-      const int col = w * kCols + (e >> 1);
-      if (col < width) out[static_cast<int64_t>(r) * width + col] = static_cast<uint8_t>((e & 1) + 1);
-    }
-  }
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= static_cast<int64_t>(height) * width) return;
+  const int r = static_cast<int>(i / width), col = static_cast<int>(i % width);
+  int half, word, shift;
+  code_place(col % kCols, half, word, shift);
+  const u32x4 v = units[((static_cast<int64_t>(matrix) * units_down + r / kUnitRows) * windows +
+                         col / kCols) * 64 + half * kUnitRows + r % kUnitRows];
+  const uint32_t code = (v[word] >> shift) & 3u;
+  out[i] = static_cast<uint8_t>(code == 2 ? 0 : code + 1);
 }
 
-__global__ void tile_fill_kernel(uint8_t *p, int64_t n, uint8_t v) {
+__global__ void tile_fill_kernel(uint32_t *p, int64_t n, uint32_t v) {
   int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i < n) p[i] = v;
 }
@@ -277,76 +231,95 @@ __global__ void tile_copy_words_kernel(const uint32_t *src, uint32_t *dst, int64
 // --------------------------------------------------------------- product ---
 
 struct TileArgs {
-  const uint2 *entries;
-  const int32_t *seg_base;
-  const uint8_t *cnt;
+  const u32x4 *units;
   const uint32_t *minmax;
   const uint16_t *x;
   uint16_t *y;
   int64_t ldx, ldy;
   int height, width, tokens;
-  int blocks, windows, matrix;
-  int x_wide;   // x rows can be read 16 bytes at a time
+  int units_down, windows, matrix;
 };
 
-// What a wavefront has requested for a window before it works on it.
-struct WindowLoads {
-  int32_t base, nch;          // the same in every lane
-  int cnt;                    // this lane's entries
-  uint2 chunk[kAhead];        // the segment's first chunks of this lane
-  uint4 xv[kTokens * kCols / 8 / 64];   // this lane's 16-byte pieces of the activations
-};
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ WindowLoads request_window(const TileArgs &a, int64_t seg0, int w,
-                                                      int t0) {
-  const int lane = threadIdx.x & 63;
-  WindowLoads l;
-  const int64_t g = seg0 + w;
-  l.base = a.seg_base[g];
-  l.nch = a.seg_base[g + 1];
-  l.cnt = a.cnt[g * kRows + lane];
-  l.base = __builtin_amdgcn_readfirstlane(l.base);
-  l.nch = __builtin_amdgcn_readfirstlane(l.nch) - l.base;
-  const uint2 *p = a.entries + static_cast<int64_t>(l.base) * kRows + lane;
+// A buffer over `bytes` bytes from base on: loads at offsets from `bytes` on
+// return zeros and touch no memory.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_over(const void *base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, static_cast<int>(bytes),
+                                           0x00020000);
+}
+constexpr uint32_t kOutside = 0x80000000u;   // an offset past every buffer here
+
+// Eight activations of one token from byte offset `at` of the buffer on, of
+// which the first `inside` lie inside the width (8 or more: all; 0 or less:
+// none).  kWide: x rows are 16-byte aligned and the width is a multiple of 8,
+// so a piece lies inside or outside as a whole; otherwise element by element.
+template <bool kWide>
+__device__ __forceinline__ u32x4 load_piece(__amdgpu_buffer_rsrc_t x, uint32_t at, int inside) {
+  if (kWide) return __builtin_amdgcn_raw_buffer_load_b128(x, inside > 0 ? at : kOutside, 0, 0);
+  uint32_t e[8];
 #pragma unroll
-  for (int c = 0; c < kAhead; c++)
-    l.chunk[c] = c < l.nch ? p[c * kRows] : make_uint2(0u, 0u);
-  // 64 tokens x 128 columns = 1024 pieces of 8 elements; lane takes piece
-  // i = lane + 64 * u: token i / 16, columns (i % 16) * 8 ...
-  const int k0 = w * kCols;
-#pragma unroll
-  for (int u = 0; u < kTokens * kCols / 8 / 64; u++) {
-    const int i = lane + 64 * u;
-    const int t = t0 + (i >> 4), col = k0 + (i & 15) * 8;
-    uint4 v = make_uint4(0u, 0u, 0u, 0u);
-    if (t < a.tokens && col < a.width) {
-      const uint16_t *src = a.x + static_cast<int64_t>(t) * a.ldx + col;
-      if (a.x_wide && col + 8 <= a.width) {
-        v = *reinterpret_cast<const uint4 *>(src);
-      } else {
-        uint16_t e[8];
-#pragma unroll
-        for (int q = 0; q < 8; q++) e[q] = col + q < a.width ? src[q] : static_cast<uint16_t>(0);
-        v = make_uint4(e[0] | (static_cast<uint32_t>(e[1]) << 16), e[2] | (static_cast<uint32_t>(e[3]) << 16),
-                       e[4] | (static_cast<uint32_t>(e[5]) << 16), e[6] | (static_cast<uint32_t>(e[7]) << 16));
-      }
-    }
-    l.xv[u] = v;
-  }
-  return l;
+  for (int q = 0; q < 8; q++)
+    e[q] = __builtin_amdgcn_raw_buffer_load_b16(x, (q < inside ? at : kOutside) + 2 * q, 0, 0);
+  u32x4 v = {e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+  return v;
 }
 
-__global__ __launch_bounds__(64 * kWaves) void matvec_tiles_kernel(TileArgs a) {
-  extern __shared__ __align__(16) uint16_t lds[];
+// The bf16 pair of weights of pair k (0..7) of a word of codes: `min_max` is
+// the row's (min, max) word.
+__device__ __forceinline__ uint32_t weight_pair(uint32_t codes, int k, uint32_t min_max) {
+  const uint32_t two = (codes >> (2 * k)) & 0x00030003u;
+  const uint32_t pick = two * 0x0202u + 0x01000100u;
+  return __builtin_amdgcn_perm(0u, min_max, pick);
+}
+
+template <bool kWide>
+__global__ __launch_bounds__(64 * kMaxWaves, 1) void matvec_tiles_kernel(TileArgs a) {
+  extern __shared__ __align__(16) unsigned char lds[];
+  float *partial = reinterpret_cast<float *>(lds);
+  const int waves = blockDim.x >> 6;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
-  uint16_t *wt = lds + wave * (2 * kTileElems);   // [64 rows][kStride]: the window's weights
-  uint16_t *xt = wt + kTileElems;                 // [64 tokens][kStride]: its activations
+  const int half = lane >> 5;
   const int block = blockIdx.x, t0 = blockIdx.y * kTokens;
-  const int row = block * kRows + lane;
-  const uint32_t mm = row < a.height ? a.minmax[static_cast<int64_t>(a.matrix) * a.height + row] : 0u;
-  const uint16_t w_min = static_cast<uint16_t>(mm & 0xffffu), w_max = static_cast<uint16_t>(mm >> 16);
-  const int64_t seg0 = (static_cast<int64_t>(a.matrix) * a.blocks + block) * a.windows;
+  // the lane's two rows as the B operand (and as the outputs' column): 32 j + lane % 32
+  uint32_t min_max[2];
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    const int row = block * kRows + j * kUnitRows + (lane & 31);
+    min_max[j] = row < a.height ? a.minmax[static_cast<int64_t>(a.matrix) * a.height + row] : 0u;
+  }
+  // The activations of this workgroup's tokens.  Load u of a window brings
+  // tokens 4 u + lane / 16; the lane's piece of its token is the one that
+  // belongs at its place in LDS, piece (lane % 16) ^ (token % 16), and
+  // token % 16 = 4 (u % 4) + lane / 16 takes four values.
+  const int rows_here = min(kTokens, a.tokens - t0);
+  const __amdgpu_buffer_rsrc_t xb = buffer_over(
+      a.x + static_cast<int64_t>(t0) * a.ldx,
+      static_cast<uint32_t>((static_cast<int64_t>(rows_here - 1) * a.ldx + a.width) * 2));
+  uint32_t x_at[4];      // byte offset of the lane's piece in window 0, loads u = 0..3
+  int x_col[4];          // and its first column
+#pragma unroll
+  for (int u = 0; u < 4; u++) {
+    const int token = 4 * u + (lane >> 4);
+    x_col[u] = 8 * ((lane & 15) ^ token);
+    x_at[u] = static_cast<uint32_t>((token * a.ldx + x_col[u]) * 2);
+  }
+  const uint32_t x_step = static_cast<uint32_t>(16 * a.ldx * 2);   // sixteen tokens on
+  unsigned char *xt = lds + wave * kPartialBytes;                   // [64 tokens][16 pieces]
+  unsigned char *xt_put = xt + lane * 16;
+  // as the A operand the lane has tokens 32 i + lane % 32 and in step s their
+  // piece 2 s + half, kept at place (2 s + half) ^ (token % 16)
+  const unsigned char *xt_get = xt + (lane & 31) * 256;
+  const uint32_t get_z = static_cast<uint32_t>((half ^ (lane & 15)) << 4);
+  // the two units of this workgroup's rows, window after window
+  const __amdgpu_buffer_rsrc_t ub = buffer_over(
+      a.units + (static_cast<int64_t>(a.matrix) * a.units_down + block * 2) * a.windows * 64,
+      static_cast<uint32_t>(2 * a.windows * 1024));
+  uint32_t unit_at[2];
+#pragma unroll
+  for (int j = 0; j < 2; j++) unit_at[j] = static_cast<uint32_t>(j * a.windows * 1024 + lane * 16);
+
   f32x16 acc[2][2];   // [32 tokens][32 rows] blocks
 #pragma unroll
   for (int i = 0; i < 2; i++)
@@ -355,90 +328,132 @@ __global__ __launch_bounds__(64 * kWaves) void matvec_tiles_kernel(TileArgs a) {
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
-  WindowLoads cur;
-  if (wave < a.windows) cur = request_window(a, seg0, wave, t0);
-  for (int w = wave; w < a.windows; w += kWaves) {
-    WindowLoads nxt;
-    const bool more = w + kWaves < a.windows;
-    if (more) nxt = request_window(a, seg0, w + kWaves, t0);
-    // a clean tile; the LDS serves a wavefront's operations in order, so these
-    // stores come before the decoded weights and after the last window's reads
-    uint4 *wz = reinterpret_cast<uint4 *>(wt);
-    for (int i = lane; i < kTileElems / 8; i += 64) wz[i] = make_uint4(0u, 0u, 0u, 0u);
-    // the window's weights
-    uint16_t *my_row = wt + lane * kStride;
-    const int nch = __builtin_amdgcn_readfirstlane(cur.nch);   // uniform: scalar loop control
-    const uint2 *p = a.entries +
-                     static_cast<int64_t>(__builtin_amdgcn_readfirstlane(cur.base)) * kRows + lane;
-    for (int c = 0; c < nch; c += kAhead) {
-      uint2 cw[kAhead];
+  if (wave < a.windows) {
+    int w = wave;
+    u32x4 xv[16], codes[2];
+    // The first window's loads, in the order in which the loop renews them: the
+    // waits in the loop count the loads issued since, and are only as long as
+    // they need to be when the way in and the way round agree.
 #pragma unroll
-      for (int u = 0; u < kAhead; u++)
-        cw[u] = c == 0 ? cur.chunk[u] : (c + u < nch ? p[(c + u) * kRows] : make_uint2(0u, 0u));
+    for (int u = 0; u < 16; u++)
+      xv[u] = load_piece<kWide>(xb, x_at[u & 3] + (u >> 2) * x_step + w * (kCols * 2),
+                                a.width - w * kCols - x_col[u & 3]);
 #pragma unroll
-      for (int u = 0; u < kAhead; u++) {
-        if (c + u < nch) {
+    for (int j = 0; j < 2; j++) codes[j] = __builtin_amdgcn_raw_buffer_load_b128(ub, unit_at[j], w * 1024, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    for (;;) {
+      // this window's activations into LDS (after the last window's reads: the
+      // LDS serves a wavefront's operations in order)
 #pragma unroll
-          for (int j = 0; j < kPerChunk; j++) {
-            const uint32_t word = j < 4 ? cw[u].x : cw[u].y;
-            const uint32_t e = (word >> (8 * (j & 3))) & 255u;
-            if ((c + u) * kPerChunk + j < cur.cnt) my_row[e >> 1] = (e & 1u) ? w_max : w_min;
-          }
+      for (int u = 0; u < 16; u++) *reinterpret_cast<u32x4 *>(xt_put + u * 1024) = xv[u];
+      // what this wavefront takes next; after its last window nothing: every
+      // offset outside, zeros that are not used
+      const bool more = w + waves < a.windows;
+      const int wn = w + waves;
+      const int width_next = more ? a.width - wn * kCols : 0;
+#pragma unroll
+      for (int u = 0; u < 16; u++)
+        xv[u] = load_piece<kWide>(xb, x_at[u & 3] + (u >> 2) * x_step + wn * (kCols * 2),
+                                  width_next - x_col[u & 3]);
+      u32x4 codes_next[2];
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+        codes_next[j] = __builtin_amdgcn_raw_buffer_load_b128(ub, more ? unit_at[j] : kOutside,
+                                                              wn * 1024, 0);
+      __builtin_amdgcn_sched_barrier(0);   // the loads stay up here, a window ahead
+#pragma unroll
+      for (int s = 0; s < kSteps; s++) {
+        bf16x8 xa[2], wb[2];
+        const uint32_t get = get_z ^ (32 * s);
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+          xa[i] = *reinterpret_cast<const bf16x8 *>(xt_get + i * (32 * 256) + get);
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+          const uint32_t word = codes[j][s >> 1];
+          u32x4 v;
+#pragma unroll
+          for (int k = 0; k < 4; k++) v[k] = weight_pair(word, 4 * (s & 1) + k, min_max[j]);
+          wb[j] = __builtin_bit_cast(bf16x8, v);
         }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+          for (int j = 0; j < 2; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[i], wb[j], acc[i][j], 0, 0, 0);
       }
+      if (!more) break;
+      w = wn;
+      codes[0] = codes_next[0];
+      codes[1] = codes_next[1];
     }
-    // the tokens' activations of the same columns
-#pragma unroll
-    for (int u = 0; u < kTokens * kCols / 8 / 64; u++) {
-      const int i = lane + 64 * u;
-      *reinterpret_cast<uint4 *>(xt + (i >> 4) * kStride + (i & 15) * 8) = cur.xv[u];
-    }
-    // 64 tokens x 64 rows += activations x weights^T over the 128 columns
-#pragma unroll
-    for (int kk = 0; kk < kCols; kk += 16) {
-      const int at = (lane & 31) * kStride + kk + 8 * (lane >> 5);
-      bf16x8 xa[2], wb[2];
-#pragma unroll
-      for (int i = 0; i < 2; i++) {
-        xa[i] = *reinterpret_cast<const bf16x8 *>(xt + i * 32 * kStride + at);
-        wb[i] = *reinterpret_cast<const bf16x8 *>(wt + i * 32 * kStride + at);
-      }
-#pragma unroll
-      for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[i], wb[j], acc[i][j], 0, 0, 0);
-    }
-    if (more) cur = nxt;
   }
+  __syncthreads();   // the partial tiles take the place of the activations
 
-  // The four wavefronts' partial tiles, added in wavefront order.  Element
-  // (token i, row j) of an accumulator block sits in lane j + 32 * ((i / 4) % 2),
-  // register 4 * (i / 8) + i % 4.
-  __syncthreads();   // every wavefront is done with its tiles
-  float *red = reinterpret_cast<float *>(lds) + wave * (kTokens * kRows);
+  // Each wavefront's tile into LDS; then added in wavefront order.  Element
+  // (token i, row j) of an accumulator block sits in lane
+  // j + 32 * ((i / 4) % 2), register 4 * (i / 8) + i % 4.
+  float *mine = partial + wave * (kTokens * kRows);
 #pragma unroll
   for (int i = 0; i < 2; i++)
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int v = 0; v < 16; v++) {
-        const int token = i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        const int token = i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
         const int r = j * 32 + (lane & 31);
-        red[token * kRows + r] = acc[i][j][v];
+        mine[token * kRows + r] = acc[i][j][v];
       }
   __syncthreads();
+  // The wavefronts share the tokens; a lane has row `lane` of the block.  Eight
+  // tokens at a time: their y are all requested before the first is needed
+  // (tokens past the last: loads that return zero, stores that are dropped).
+  const int row = block * kRows + lane;
   if (row < a.height) {
-    const float *all = reinterpret_cast<const float *>(lds);
-    for (int t = wave; t < kTokens && t0 + t < a.tokens; t += kWaves) {
-      const int at = t * kRows + lane;
-      const float sum = ((all[at] + all[kTokens * kRows + at]) + all[2 * kTokens * kRows + at]) +
-                        all[3 * kTokens * kRows + at];
-      uint16_t *dst = a.y + static_cast<int64_t>(t0 + t) * a.ldy + row;
-      // reference sub1_cuda_kernel.cu:200: y[row] += bf16(res), the sum in bf16
-      *dst = f32_to_bf16(bf16_to_f32(*dst) + bf16_to_f32(f32_to_bf16(sum)));
+    const __amdgpu_buffer_rsrc_t yb = buffer_over(
+        a.y + static_cast<int64_t>(t0) * a.ldy,
+        static_cast<uint32_t>((static_cast<int64_t>(rows_here - 1) * a.ldy + a.height) * 2));
+    const uint32_t y_at = static_cast<uint32_t>(row * 2), y_step = static_cast<uint32_t>(a.ldy * 2);
+    for (int first = wave; first < rows_here; first += 8 * waves) {
+      uint16_t before[8];
+#pragma unroll
+      for (int k = 0; k < 8; k++)
+        before[k] = __builtin_amdgcn_raw_buffer_load_b16(yb, y_at + (first + k * waves) * y_step, 0, 0);
+#pragma unroll
+      for (int k = 0; k < 8; k++) {
+        const int t = first + k * waves;
+        const int at = (t & (kTokens - 1)) * kRows + lane;
+        float sum = partial[at];
+        for (int v = 1; v < waves; v++) sum += partial[v * (kTokens * kRows) + at];
+        // reference sub1_cuda_kernel.cu:200: y[row] += bf16(res), the sum in bf16
+        __builtin_amdgcn_raw_buffer_store_b16(
+            f32_to_bf16(bf16_to_f32(before[k]) + bf16_to_f32(f32_to_bf16(sum))), yb,
+            t < kTokens ? y_at + t * y_step : kOutside, 0, 0);
+      }
     }
   }
+}
+
+// Wavefronts per workgroup for a matrix of `blocks` blocks of 64 rows and
+// `windows` windows: 1, 2, 4 or 8, whichever gives the fewest rounds of
+// workgroups over the chip times the windows a wavefront walks in a row
+// (counting what a workgroup costs besides its windows) at eight tiles of
+// tokens.  It depends on the matrix alone, never on the tokens of a launch, so
+// a token's result is the same whatever launch it is part of.  A CU holds
+// eight of these wavefronts (registers).
+int pick_waves(int blocks, int windows) {
+  int best = 1;
+  double best_cost = 0;
+  for (int n = 1; n <= kMaxWaves; n *= 2) {
+    const int64_t slots = 256 * (8 / n);
+    const int64_t rounds = (8ll * blocks + slots - 1) / slots;
+    const double cost = rounds * (2.0 + 0.9 * ((windows + n - 1) / n));
+    if (n == 1 || cost < best_cost - 1e-9) {
+      best = n;
+      best_cost = cost;
+    }
+  }
+  return best;
 }
 
 int check_set(const sub1_matrix_set *ms, const char *who) {
@@ -475,8 +490,10 @@ int check_tiles(const sub1_tiles *t, const char *who) {
     return fail(SUB1_ERR_SHAPE, "%s: %d matrices of %d x %d", who, t->count, t->height, t->width);
   if (misaligned(t->meta, 256) || misaligned(t->entries, 256))
     return fail(SUB1_ERR_ALIGN, "%s: buffers must be 256-byte aligned", who);
-  if (t->meta_bytes < tile_layout(t->count, t->height, t->width).bytes)
-    return fail(SUB1_ERR_SHAPE, "%s: meta smaller than its layout", who);
+  const TileLayout l = tile_layout(t->count, t->height, t->width);
+  if (t->meta_bytes < l.bytes) return fail(SUB1_ERR_SHAPE, "%s: meta smaller than its layout", who);
+  if (t->total_chunks != l.units || t->entry_bytes < l.units * 1024)
+    return fail(SUB1_ERR_SHAPE, "%s: entries buffer smaller than the layout needs", who);
   return SUB1_OK;
 }
 
@@ -492,6 +509,7 @@ extern "C" int64_t sub1_tiles_meta_bytes(int count, int height, int width) {
 extern "C" int sub1_tiles_layout(const sub1_matrix_set *ms, void *meta, int64_t meta_bytes,
                                  sub1_tiles *out, void *stream) {
   const char *who = "sub1_tiles_layout";
+  (void)stream;
   int rc = check_set(ms, who);
   if (rc) return rc;
   if (!meta || !out) return fail(SUB1_ERR_NULL, "%s: NULL argument", who);
@@ -499,34 +517,11 @@ extern "C" int sub1_tiles_layout(const sub1_matrix_set *ms, void *meta, int64_t 
   const TileLayout t = tile_layout(ms->count, ms->height, ms->width);
   if (meta_bytes < t.bytes)
     return fail(SUB1_ERR_SHAPE, "%s: meta needs %lld bytes", who, static_cast<long long>(t.bytes));
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  char *base = static_cast<char *>(meta);
-  int32_t *counts = reinterpret_cast<int32_t *>(base + t.seg_base);
-  uint8_t *cnt = reinterpret_cast<uint8_t *>(base + t.cnt);
-  int32_t *status = reinterpret_cast<int32_t *>(base + t.status);
-  tile_fill_kernel<<<1, 64, 0, s>>>(reinterpret_cast<uint8_t *>(status), 16, 0);
-  const int64_t lanes = static_cast<int64_t>(ms->count) * t.blocks * kRows;
-  tile_count_kernel<<<static_cast<unsigned>((lanes + 255) / 256), 256, 0, s>>>(
-      source_of(ms), t.blocks, t.windows, cnt, status, lanes);
-  tile_segments_kernel<<<static_cast<unsigned>((t.segments + 255) / 256), 256, 0, s>>>(cnt, counts,
-                                                                                        t.segments);
-  tile_scan_kernel<<<1, 1024, 0, s>>>(counts, t.segments);
-  const int64_t words = static_cast<int64_t>(ms->count) * ms->height;
-  tile_copy_words_kernel<<<static_cast<unsigned>((words + 255) / 256), 256, 0, s>>>(
-      static_cast<const uint32_t *>(ms->ter_minmax), reinterpret_cast<uint32_t *>(base + t.minmax),
-      words);
-  HIP_TRY(hipGetLastError());
-  int32_t bad = 0, total = 0;
-  HIP_TRY(hipMemcpyAsync(&bad, status, 4, hipMemcpyDeviceToHost, s));
-  HIP_TRY(hipMemcpyAsync(&total, counts + t.segments, 4, hipMemcpyDeviceToHost, s));
-  HIP_TRY(hipStreamSynchronize(s));
-  if (bad) return fail(SUB1_ERR_SHAPE, "%s: the codes of %d rows do not cover the width", who, bad);
-  if (total < 0) return fail(SUB1_ERR_SHAPE, "%s: too many entries", who);
   out->meta = meta;
   out->entries = nullptr;
   out->meta_bytes = t.bytes;
-  out->total_chunks = total;
-  out->entry_bytes = align256(static_cast<int64_t>(total) * kRows * 8 + 256);
+  out->total_chunks = t.units;
+  out->entry_bytes = t.units * 1024;
   out->count = ms->count;
   out->height = ms->height;
   out->width = ms->width;
@@ -541,16 +536,26 @@ extern "C" int sub1_tiles_entries(const sub1_matrix_set *ms, const sub1_tiles *t
   if (rc) return rc;
   if (t->count != ms->count || t->height != ms->height || t->width != ms->width)
     return fail(SUB1_ERR_SHAPE, "%s: the layout belongs to other matrices", who);
-  if (t->total_chunks < 0 || t->entry_bytes < t->total_chunks * kRows * 8)
-    return fail(SUB1_ERR_SHAPE, "%s: entries buffer smaller than the layout needs", who);
   const TileLayout l = tile_layout(t->count, t->height, t->width);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const char *base = static_cast<const char *>(t->meta);
-  const int64_t lanes = static_cast<int64_t>(ms->count) * l.blocks * kRows;
-  tile_emit_kernel<<<static_cast<unsigned>((lanes + 255) / 256), 256, 0, s>>>(
-      source_of(ms), l.blocks, l.windows, reinterpret_cast<const int32_t *>(base + l.seg_base),
-      static_cast<uint8_t *>(const_cast<void *>(t->entries)), lanes);
+  char *base = static_cast<char *>(const_cast<void *>(t->meta));
+  int32_t *status = reinterpret_cast<int32_t *>(base + l.status);
+  u32x4 *units = static_cast<u32x4 *>(const_cast<void *>(t->entries));
+  tile_fill_kernel<<<1, 64, 0, s>>>(reinterpret_cast<uint32_t *>(status), 4, 0u);
+  const int64_t unit_words = l.units * 256;
+  tile_fill_kernel<<<static_cast<unsigned>((unit_words + 255) / 256), 256, 0, s>>>(
+      reinterpret_cast<uint32_t *>(units), unit_words, kAllZero);
+  const int64_t rows = static_cast<int64_t>(ms->count) * ms->height;
+  code_emit_kernel<<<static_cast<unsigned>((rows + 255) / 256), 256, 0, s>>>(
+      source_of(ms), l.units_down, l.windows, units, status, rows);
+  tile_copy_words_kernel<<<static_cast<unsigned>((rows + 255) / 256), 256, 0, s>>>(
+      static_cast<const uint32_t *>(ms->ter_minmax), reinterpret_cast<uint32_t *>(base + l.minmax),
+      rows);
   HIP_TRY(hipGetLastError());
+  int32_t bad = 0;
+  HIP_TRY(hipMemcpyAsync(&bad, status, 4, hipMemcpyDeviceToHost, s));
+  HIP_TRY(hipStreamSynchronize(s));
+  if (bad) return fail(SUB1_ERR_SHAPE, "%s: the codes of %d rows do not cover the width", who, bad);
   return SUB1_OK;
 }
 
@@ -570,9 +575,7 @@ extern "C" int sub1_matvec_tiles(const sub1_tiles *t, int matrix, const void *x,
   const TileLayout l = tile_layout(t->count, t->height, t->width);
   const char *base = static_cast<const char *>(t->meta);
   TileArgs a;
-  a.entries = static_cast<const uint2 *>(t->entries);
-  a.seg_base = reinterpret_cast<const int32_t *>(base + l.seg_base);
-  a.cnt = reinterpret_cast<const uint8_t *>(base + l.cnt);
+  a.units = static_cast<const u32x4 *>(t->entries);
   a.minmax = reinterpret_cast<const uint32_t *>(base + l.minmax);
   a.x = static_cast<const uint16_t *>(x);
   a.y = static_cast<uint16_t *>(y);
@@ -581,16 +584,21 @@ extern "C" int sub1_matvec_tiles(const sub1_tiles *t, int matrix, const void *x,
   a.height = t->height;
   a.width = t->width;
   a.tokens = tokens;
-  a.blocks = l.blocks;
+  a.units_down = l.units_down;
   a.windows = l.windows;
   a.matrix = matrix;
-  a.x_wide = !misaligned(x, 16) && ldx % 8 == 0;
-  HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_tiles_kernel),
+  const bool wide = !misaligned(x, 16) && ldx % 8 == 0 && t->width % 8 == 0;
+  if (ldx >= (1 << 24) || ldy >= (1 << 24))
+    return fail(SUB1_ERR_SHAPE, "%s: token strides of 2^24 elements or more", who);
+  const dim3 grid(l.units_down / 2, (tokens + kTokens - 1) / kTokens);
+  const int waves = pick_waves(l.units_down / 2, l.windows);
+  const size_t lds_bytes = static_cast<size_t>(waves) * kPartialBytes;
+  auto kernel = wide ? matvec_tiles_kernel<true> : matvec_tiles_kernel<false>;
+  HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                               hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(kTilesLds)));
-  const dim3 grid(l.blocks, (tokens + kTokens - 1) / kTokens);
-  sub1::note_kernel("matvec_tiles_kernel");
-  matvec_tiles_kernel<<<grid, 64 * kWaves, kTilesLds, static_cast<hipStream_t>(stream)>>>(a);
+                              static_cast<int>(kMaxWaves * kPartialBytes)));
+  sub1::note_kernel(wide ? "matvec_tiles_kernel<true>" : "matvec_tiles_kernel<false>");
+  kernel<<<grid, 64 * waves, lds_bytes, static_cast<hipStream_t>(stream)>>>(a);
   HIP_TRY(hipGetLastError());
   return SUB1_OK;
 }
@@ -602,15 +610,11 @@ extern "C" int sub1_tiles_decode(const sub1_tiles *t, int matrix, void *tern_out
   if (!tern_out) return fail(SUB1_ERR_NULL, "%s: NULL argument", who);
   if (matrix < 0 || matrix >= t->count) return fail(SUB1_ERR_SHAPE, "%s: no matrix %d", who, matrix);
   const TileLayout l = tile_layout(t->count, t->height, t->width);
-  const char *base = static_cast<const char *>(t->meta);
-  hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t n = static_cast<int64_t>(t->height) * t->width;
-  tile_fill_kernel<<<static_cast<unsigned>((n + 255) / 256), 256, 0, s>>>(
-      static_cast<uint8_t *>(tern_out), n, 0);
-  tile_decode_kernel<<<(l.blocks * kRows + 255) / 256, 256, 0, s>>>(
-      static_cast<const uint8_t *>(t->entries), reinterpret_cast<const int32_t *>(base + l.seg_base),
-      reinterpret_cast<const uint8_t *>(base + l.cnt), static_cast<uint8_t *>(tern_out), matrix,
-      l.blocks, l.windows, t->height, t->width);
+  code_decode_kernel<<<static_cast<unsigned>((n + 255) / 256), 256, 0,
+                        static_cast<hipStream_t>(stream)>>>(
+      static_cast<const u32x4 *>(t->entries), static_cast<uint8_t *>(tern_out), matrix,
+      l.units_down, l.windows, t->height, t->width);
   HIP_TRY(hipGetLastError());
   return SUB1_OK;
 }

@@ -147,7 +147,7 @@ def test_sub1linear_takes_the_tiles_from_64_tokens_on(gpu, oracle):
     x = torch.randn((100, 512), generator=torch.Generator().manual_seed(3)).bfloat16().cuda()
     ref = x.float() @ w.float().t()
     y = lin(x)
-    assert _lib.load().sub1_last_kernel() == b'matvec_tiles_kernel'
+    assert _lib.load().sub1_last_kernel() .startswith(b'matvec_tiles_kernel')
     assert torch.linalg.norm(y.float() - ref) <= REL_TOL * torch.linalg.norm(ref)
     y_few = lin(x[:10])
     assert _lib.load().sub1_last_kernel() != b'matvec_tiles_kernel'
