@@ -25,20 +25,27 @@
 //
 // Kernel: a workgroup owns 64 rows x 64 tokens; its wavefronts split the
 // windows of 128 columns among themselves (wavefront v takes v, v + n, ...).  Per
-// window a wavefront copies the tokens' activations, 64 x 128, through
-// registers into its own 16 KB of LDS (coalesced 16-byte loads, four tokens an
-// instruction; the 16-byte pieces of a token are XOR-swizzled with the token's
-// number so that neither the stores nor the operand reads meet in a bank), and
-// per step of 16 columns reads its A operands from there, builds its B
-// operands from the codes and adds into a 64 x 64 fp32 accumulator (2 x 2 MFMA
-// blocks).  The loads of the next window are issued as soon as the registers
-// are free, a whole window ahead.  All of them are buffer loads: what lies past
-// the last token, past the width or past a wavefront's last window is given an
-// offset outside the buffer and comes back as zeros, without a branch or a
-// mask.  At the end the partial tiles are added through LDS in wavefront
-// order, rounded to bf16 and added onto y in bf16 (reference
-// sub1_cuda_kernel.cu:199-200).  The number of wavefronts depends on the matrix
-// alone, so a token's result does not depend on the launch it is part of.
+// window a wavefront brings the tokens' activations, 64 x 128, into its own
+// 16 KB of LDS (16-byte pieces, four tokens an instruction; the pieces of a
+// token are XOR-swizzled with the token's number so that neither the arrivals
+// nor the operand reads meet in a bank), and per step of 16 columns reads its
+// A operands from there, builds its B operands from the codes and adds into a
+// 64 x 64 fp32 accumulator (2 x 2 MFMA blocks).  Where x rows are 16-byte
+// aligned the loads go straight into LDS, into a second buffer, a whole window
+// ahead of the arithmetic (matvec_tiles_kernel); otherwise through registers,
+// element by element (matvec_tiles_ragged_kernel).  All of them are buffer
+// loads: what lies past the last token, past the width or past a wavefront's
+// last window is given an offset outside the buffer (or an empty buffer) and
+// reads nothing, without a branch or a mask.  At the end the partial tiles are
+// added through LDS in wavefront order, rounded to bf16 and added onto y in
+// bf16 (reference sub1_cuda_kernel.cu:199-200).  The number of wavefronts
+// depends on the matrix alone, so a token's result does not depend on the
+// launch it is part of.
+//
+// Bound: building the B operands, four plain instructions per pair of weights
+// and 64 per step of four MFMAs, takes a wavefront twice as long to issue as
+// the matrix core needs for the four; with the one wavefront per SIMD that the
+// LDS leaves room for, a window takes 1.25 us where its MFMAs alone take 0.43.
 //
 // Results: each product x * w is exact in fp32 and the sums are fp32, but in
 // the matrix cores' own order; they agree with the row-walking kernels and the
@@ -62,7 +69,7 @@ constexpr int kRows = 64;                 // rows per workgroup: two units
 constexpr int kCols = 128;                // columns per window
 constexpr int kTokens = 64;               // tokens per workgroup
 constexpr int kSteps = kCols / 16;        // MFMA steps per window
-constexpr int kMaxWaves = 8;              // wavefronts per workgroup, at most
+constexpr int kMaxWaves = 4;              // wavefronts per workgroup, at most
 constexpr uint32_t kAllZero = 0xaaaaaaaau; // a word of codes of zero weights
 constexpr int kPartialBytes = kTokens * kRows * 4;   // one wavefront's scaled tile
 
@@ -250,21 +257,6 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_over(const void *base, 
 }
 constexpr uint32_t kOutside = 0x80000000u;   // an offset past every buffer here
 
-// Eight activations of one token from byte offset `at` of the buffer on, of
-// which the first `inside` lie inside the width (8 or more: all; 0 or less:
-// none).  kWide: x rows are 16-byte aligned and the width is a multiple of 8,
-// so a piece lies inside or outside as a whole; otherwise element by element.
-template <bool kWide>
-__device__ __forceinline__ u32x4 load_piece(__amdgpu_buffer_rsrc_t x, uint32_t at, int inside) {
-  if (kWide) return __builtin_amdgcn_raw_buffer_load_b128(x, inside > 0 ? at : kOutside, 0, 0);
-  uint32_t e[8];
-#pragma unroll
-  for (int q = 0; q < 8; q++)
-    e[q] = __builtin_amdgcn_raw_buffer_load_b16(x, (q < inside ? at : kOutside) + 2 * q, 0, 0);
-  u32x4 v = {e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
-  return v;
-}
-
 // The bf16 pair of weights of pair k (0..7) of a word of codes: `min_max` is
 // the row's (min, max) word.
 __device__ __forceinline__ uint32_t weight_pair(uint32_t codes, int k, uint32_t min_max) {
@@ -273,52 +265,305 @@ __device__ __forceinline__ uint32_t weight_pair(uint32_t codes, int k, uint32_t 
   return __builtin_amdgcn_perm(0u, min_max, pick);
 }
 
-template <bool kWide>
-__global__ __launch_bounds__(64 * kMaxWaves, 1) void matvec_tiles_kernel(TileArgs a) {
-  extern __shared__ __align__(16) unsigned char lds[];
-  float *partial = reinterpret_cast<float *>(lds);
-  const int waves = blockDim.x >> 6;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  const int half = lane >> 5;
-  const int block = blockIdx.x, t0 = blockIdx.y * kTokens;
-  // the lane's two rows as the B operand (and as the outputs' column): 32 j + lane % 32
+// What the kernels share.  A workgroup owns rows 64 block .. +64 and tokens
+// t0 .. +64; as the B operand (and as an output column) a lane has the rows
+// 32 j + lane % 32, as the A operand the tokens 32 i + lane % 32 and in step s
+// their piece 2 s + half.  In LDS piece p of token t of a window sits at
+// 256 t + 16 (p ^ (t % 16)) of the wavefront's 16 KB.
+struct TileLane {
+  int lane, half, block, t0, rows_here;
   uint32_t min_max[2];
+  uint32_t unit_at[2];   // byte offset of the lane's codes in window 0, per unit
+  uint32_t get_at;       // of its A operand of step 0 in the wavefront's tile
+};
+
+__device__ __forceinline__ TileLane tile_lane(const TileArgs &a) {
+  TileLane l;
+  l.lane = threadIdx.x & 63;
+  l.half = l.lane >> 5;
+  l.block = blockIdx.x;
+  l.t0 = blockIdx.y * kTokens;
+  l.rows_here = min(kTokens, a.tokens - l.t0);
 #pragma unroll
   for (int j = 0; j < 2; j++) {
-    const int row = block * kRows + j * kUnitRows + (lane & 31);
-    min_max[j] = row < a.height ? a.minmax[static_cast<int64_t>(a.matrix) * a.height + row] : 0u;
+    const int row = l.block * kRows + j * kUnitRows + (l.lane & 31);
+    l.min_max[j] = row < a.height ? a.minmax[static_cast<int64_t>(a.matrix) * a.height + row] : 0u;
+    l.unit_at[j] = static_cast<uint32_t>(j * a.windows * 1024 + l.lane * 16);
   }
-  // The activations of this workgroup's tokens.  Load u of a window brings
-  // tokens 4 u + lane / 16; the lane's piece of its token is the one that
-  // belongs at its place in LDS, piece (lane % 16) ^ (token % 16), and
-  // token % 16 = 4 (u % 4) + lane / 16 takes four values.
-  const int rows_here = min(kTokens, a.tokens - t0);
-  const __amdgpu_buffer_rsrc_t xb = buffer_over(
-      a.x + static_cast<int64_t>(t0) * a.ldx,
-      static_cast<uint32_t>((static_cast<int64_t>(rows_here - 1) * a.ldx + a.width) * 2));
-  uint32_t x_at[4];      // byte offset of the lane's piece in window 0, loads u = 0..3
-  int x_col[4];          // and its first column
+  l.get_at = static_cast<uint32_t>((l.lane & 31) * 256 + ((l.half ^ (l.lane & 15)) << 4));
+  return l;
+}
+
+// The codes of this workgroup's two units, window after window.
+// (`any` false: an empty buffer, every load from it returns zeros.)
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t units_of(const TileArgs &a, int block,
+                                                           bool any = true) {
+  return buffer_over(
+      a.units + (static_cast<int64_t>(a.matrix) * a.units_down + block * 2) * a.windows * 64,
+      any ? static_cast<uint32_t>(2 * a.windows * 1024) : 0u);
+}
+
+// The activations of this workgroup's tokens.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tokens_of(const TileArgs &a, const TileLane &l,
+                                                            bool any = true) {
+  return buffer_over(
+      a.x + static_cast<int64_t>(l.t0) * a.ldx,
+      any ? static_cast<uint32_t>((static_cast<int64_t>(l.rows_here - 1) * a.ldx + a.width) * 2)
+          : 0u);
+}
+
+// One window: eight steps of four MFMAs on the activations in `tile` (this
+// wavefront's 16 KB) and the weights in `codes`.  Each MFMA keeps the matrix
+// core busy for as long as eight plain instructions take to issue, so the next
+// step's B operands are built a quarter at a time behind the MFMAs of this one
+// and its A operands are requested at its start.
+__device__ __forceinline__ void window_steps(const unsigned char *tile, const TileLane &l,
+                                             const u32x4 (&codes)[2], f32x16 (&acc)[2][2]) {
+  const unsigned char *get = tile + l.get_at;
+  bf16x8 xa[2];
+  u32x4 wv[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) xa[i] = *reinterpret_cast<const bf16x8 *>(get + i * (32 * 256));
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+#pragma unroll
+    for (int k = 0; k < 4; k++) wv[j][k] = weight_pair(codes[j][0], k, l.min_max[j]);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int s = 0; s < kSteps; s++) {
+    bf16x8 xa_next[2];
+    u32x4 wv_next[2];
+    const int sn = s + 1 < kSteps ? s + 1 : s;   // after the last step nothing new
+    if (s + 1 < kSteps) {
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+        xa_next[i] = *reinterpret_cast<const bf16x8 *>(
+            tile + (l.get_at ^ static_cast<uint32_t>(32 * sn)) + i * (32 * 256));
+    }
+    const bf16x8 wb0 = __builtin_bit_cast(bf16x8, wv[0]), wb1 = __builtin_bit_cast(bf16x8, wv[1]);
+#pragma unroll
+    for (int quarter = 0; quarter < 4; quarter++) {
+      const int i = quarter >> 1, j = quarter & 1;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[i], j ? wb1 : wb0, acc[i][j], 0, 0, 0);
+      if (s + 1 < kSteps) {
+        const int jn = quarter >> 1, k0 = 2 * (quarter & 1);
+#pragma unroll
+        for (int k = k0; k < k0 + 2; k++)
+          wv_next[jn][k] = weight_pair(codes[jn][sn >> 1], 4 * (sn & 1) + k, l.min_max[jn]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (s + 1 < kSteps) {
+      xa[0] = xa_next[0];
+      xa[1] = xa_next[1];
+      wv[0] = wv_next[0];
+      wv[1] = wv_next[1];
+    }
+  }
+}
+
+// The end of a workgroup: its wavefronts' tiles added in wavefront order,
+// rounded to bf16 and added onto y in bf16 (reference sub1_cuda_kernel.cu:199-
+// 200).  The wavefronts share the tokens, a lane has row `lane` of the block;
+// the y of a lane's tokens are all requested before anything else (tokens past
+// the last: loads that return zero, stores that are dropped).  `partial` is
+// LDS that no wavefront reads any more.  kPer = 64 / waves.
+template <int kPer>
+__device__ __forceinline__ void finish_tile(const TileArgs &a, const TileLane &l, int wave,
+                                            int waves, float *partial, const f32x16 (&acc)[2][2]) {
+  const int row = l.block * kRows + l.lane;
+  const __amdgpu_buffer_rsrc_t yb = buffer_over(
+      a.y + static_cast<int64_t>(l.t0) * a.ldy,
+      static_cast<uint32_t>((static_cast<int64_t>(l.rows_here - 1) * a.ldy + a.height) * 2));
+  // rows past the height: outside the buffer
+  const uint32_t y_at = row < a.height ? static_cast<uint32_t>(row * 2) : kOutside;
+  const uint32_t y_step = static_cast<uint32_t>(a.ldy * 2);
+  uint16_t before[kPer];
+#pragma unroll
+  for (int k = 0; k < kPer; k++)
+    before[k] = __builtin_amdgcn_raw_buffer_load_b16(yb, y_at + (wave + k * waves) * y_step, 0, 0);
+  // Element (token i, row j) of an accumulator block sits in lane
+  // j + 32 * ((i / 4) % 2), register 4 * (i / 8) + i % 4.
+  float *mine = partial + wave * (kTokens * kRows);
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int token = i * 32 + 8 * (v >> 2) + 4 * l.half + (v & 3);
+        mine[token * kRows + j * 32 + (l.lane & 31)] = acc[i][j][v];
+      }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kPer; k++) {
+    const int t = wave + k * waves;
+    const int at = t * kRows + l.lane;
+    float sum = partial[at];
+    for (int v = 1; v < waves; v++) sum += partial[v * (kTokens * kRows) + at];
+    __builtin_amdgcn_raw_buffer_store_b16(
+        f32_to_bf16(bf16_to_f32(before[k]) + bf16_to_f32(f32_to_bf16(sum))), yb, y_at + t * y_step, 0,
+        0);
+  }
+}
+
+// ---- x rows 16-byte aligned, the width a multiple of 8 ----------------------
+//
+// Activations and codes go from global memory straight into LDS (buffer loads
+// with the lds bit, 16 bytes a lane: four tokens of activations, or one unit
+// of codes, an instruction).  A wavefront has two buffers (a tile of
+// activations of 16 KB and a block of codes of 2 KB each) and asks for the next
+// window before it starts on the current one.
+//
+// Waiting is done by hand.  Left to the compiler, an LDS read behind such
+// loads waits for all of them (it cannot tell the two buffers apart), which
+// puts the memory latency of every window back in front of its arithmetic.  So
+// the loop reads LDS through ds_read_b128 written as inline assembly, which
+// the compiler does not see as LDS reads, and counts the loads itself: every
+// turn issues exactly kLoadsPerWindow of them (after a wavefront's last window
+// from empty buffers: nothing is read, nothing lands), loads complete in the
+// order issued, and "all but the newest kLoadsPerWindow have landed" is the
+// wait before a window is read.  The LDS reads are waited for with lgkmcnt(0)
+// in statements that take the read registers as operands, so nothing uses them
+// earlier.
+
+constexpr int kLoadsPerWindow = 18;   // 16 of activations, 2 of codes
+constexpr int kTileBytes = 16384;     // a tile of activations
+constexpr int kBlockBytes = 2048;     // a window's codes (two units)
+
+// Load u (0..15) of a window brings tokens 4 u + lane / 16, the lane its piece
+// (lane % 16) ^ (token % 16): the one that belongs at its place in LDS.  `at`
+// holds the lane's byte offsets for u = 0..3 (token % 16 takes four values per
+// lane), `col` the first column of each.
+struct Fetch {
+  uint32_t at[4];
+  int col[4];
+  uint32_t step;   // sixteen tokens on
+};
+
+__device__ __forceinline__ Fetch fetch_of(const TileArgs &a, int lane) {
+  Fetch f;
 #pragma unroll
   for (int u = 0; u < 4; u++) {
     const int token = 4 * u + (lane >> 4);
-    x_col[u] = 8 * ((lane & 15) ^ token);
-    x_at[u] = static_cast<uint32_t>((token * a.ldx + x_col[u]) * 2);
+    f.col[u] = 8 * ((lane & 15) ^ token);
+    f.at[u] = static_cast<uint32_t>((token * a.ldx + f.col[u]) * 2);
   }
-  const uint32_t x_step = static_cast<uint32_t>(16 * a.ldx * 2);   // sixteen tokens on
-  unsigned char *xt = lds + wave * kPartialBytes;                   // [64 tokens][16 pieces]
-  unsigned char *xt_put = xt + lane * 16;
-  // as the A operand the lane has tokens 32 i + lane % 32 and in step s their
-  // piece 2 s + half, kept at place (2 s + half) ^ (token % 16)
-  const unsigned char *xt_get = xt + (lane & 31) * 256;
-  const uint32_t get_z = static_cast<uint32_t>((half ^ (lane & 15)) << 4);
-  // the two units of this workgroup's rows, window after window
-  const __amdgpu_buffer_rsrc_t ub = buffer_over(
-      a.units + (static_cast<int64_t>(a.matrix) * a.units_down + block * 2) * a.windows * 64,
-      static_cast<uint32_t>(2 * a.windows * 1024));
-  uint32_t unit_at[2];
+  f.step = static_cast<uint32_t>(16 * a.ldx * 2);
+  return f;
+}
+
+typedef __attribute__((address_space(3))) unsigned char *lds_bytes;
+
+// Window w on its way: the activations into the tile at `tile`, the codes into
+// the block at `block`.  Pieces from the width on are not fetched (`edge`: this
+// window reaches past the width; their places hold zeros or older activations,
+// and the weights there are zeros).
+__device__ __forceinline__ void fetch_window(__amdgpu_buffer_rsrc_t xb, __amdgpu_buffer_rsrc_t ub,
+                                             const Fetch &f, const TileArgs &a, const TileLane &l,
+                                             int w, bool edge, lds_bytes tile, lds_bytes block) {
+  if (edge) {
+    const int inside = a.width - w * kCols;
 #pragma unroll
-  for (int j = 0; j < 2; j++) unit_at[j] = static_cast<uint32_t>(j * a.windows * 1024 + lane * 16);
+    for (int u = 0; u < 16; u++)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          xb, tile + u * 1024, 16,
+          f.col[u & 3] < inside ? f.at[u & 3] + (u >> 2) * f.step : kOutside, w * (kCols * 2), 0, 0);
+  } else {
+#pragma unroll
+    for (int u = 0; u < 16; u++)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(xb, tile + u * 1024, 16,
+                                               f.at[u & 3] + (u >> 2) * f.step, w * (kCols * 2), 0, 0);
+  }
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ub, block + j * 1024, 16, l.unit_at[j], w * 1024, 0, 0);
+}
+
+// 16 bytes from LDS address `at` and from `at` + kFar, requested only.
+template <int kFar>
+__device__ __forceinline__ void lds_request(uint32_t at, u32x4 &near, u32x4 &far) {
+  asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:%3"
+               : "=&v"(near), "=&v"(far)
+               : "v"(at), "n"(kFar)
+               : "memory");
+}
+// What was requested has arrived.
+__device__ __forceinline__ void lds_arrived(u32x4 &p, u32x4 &q) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(p), "+v"(q)::"memory");
+}
+
+// window_steps with the operands read by hand: the tile at LDS address `tile`,
+// the codes at `block`.
+__device__ __forceinline__ void window_steps_counted(uint32_t tile, uint32_t block,
+                                                     const TileLane &l, f32x16 (&acc)[2][2]) {
+  const uint32_t get = tile + l.get_at;
+  u32x4 xa[2], codes[2], wv[2];
+  lds_request<1024>(block + l.lane * 16, codes[0], codes[1]);
+  lds_request<32 * 256>(get, xa[0], xa[1]);
+  lds_arrived(codes[0], codes[1]);
+  lds_arrived(xa[0], xa[1]);
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+#pragma unroll
+    for (int k = 0; k < 4; k++) wv[j][k] = weight_pair(codes[j][0], k, l.min_max[j]);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int s = 0; s < kSteps; s++) {
+    u32x4 xa_next[2], wv_next[2];
+    const int sn = s + 1 < kSteps ? s + 1 : s;   // after the last step nothing new
+    if (s + 1 < kSteps) lds_request<32 * 256>(get ^ static_cast<uint32_t>(32 * sn), xa_next[0], xa_next[1]);
+    const bf16x8 wb0 = __builtin_bit_cast(bf16x8, wv[0]), wb1 = __builtin_bit_cast(bf16x8, wv[1]);
+    const bf16x8 xa0 = __builtin_bit_cast(bf16x8, xa[0]), xa1 = __builtin_bit_cast(bf16x8, xa[1]);
+#pragma unroll
+    for (int quarter = 0; quarter < 4; quarter++) {
+      const int i = quarter >> 1, j = quarter & 1;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(i ? xa1 : xa0, j ? wb1 : wb0, acc[i][j], 0, 0, 0);
+      if (s + 1 < kSteps) {
+        const int jn = quarter >> 1, k0 = 2 * (quarter & 1);
+#pragma unroll
+        for (int k = k0; k < k0 + 2; k++)
+          wv_next[jn][k] = weight_pair(codes[jn][sn >> 1], 4 * (sn & 1) + k, l.min_max[jn]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (s + 1 < kSteps) {
+      lds_arrived(xa_next[0], xa_next[1]);
+      xa[0] = xa_next[0];
+      xa[1] = xa_next[1];
+      wv[0] = wv_next[0];
+      wv[1] = wv_next[1];
+    }
+  }
+}
+
+template <int kWaves>
+__global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(1, 2)))
+void matvec_tiles_kernel(TileArgs a) {
+  __shared__ __align__(16384) unsigned char tiles[2 * kWaves * kTileBytes];   // [buffer][wavefront]
+  __shared__ __align__(1024) unsigned char blocks[2 * kWaves * kBlockBytes];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const TileLane l = tile_lane(a);
+  const Fetch f = fetch_of(a, l.lane);
+  // (the rows' min and max are waited for here, while nothing else is on its way)
+  asm volatile("" ::"v"(l.min_max[0]), "v"(l.min_max[1]));
+  const lds_bytes my_tiles = (lds_bytes)tiles + wave * kTileBytes;
+  const lds_bytes my_blocks = (lds_bytes)blocks + wave * kBlockBytes;
+  const int last = a.windows - 1;
+  const bool ragged_edge = (a.width & (kCols - 1)) != 0;
+  if (ragged_edge) {
+    // places that no fetch writes must not hold what LDS happened to hold
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+      for (int u = 0; u < 16; u++)
+        *reinterpret_cast<u32x4 *>(tiles + (b * kWaves + wave) * kTileBytes + (u * 64 + l.lane) * 16) =
+            zero;
+    // these stores and the fetches below go to LDS by different ways: the
+    // zeros must have arrived before the first fetch is asked for
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
 
   f32x16 acc[2][2];   // [32 tokens][32 rows] blocks
 #pragma unroll
@@ -330,130 +575,113 @@ __global__ __launch_bounds__(64 * kMaxWaves, 1) void matvec_tiles_kernel(TileArg
 
   if (wave < a.windows) {
     int w = wave;
-    u32x4 xv[16], codes[2];
-    // The first window's loads, in the order in which the loop renews them: the
-    // waits in the loop count the loads issued since, and are only as long as
-    // they need to be when the way in and the way round agree.
-#pragma unroll
-    for (int u = 0; u < 16; u++)
-      xv[u] = load_piece<kWide>(xb, x_at[u & 3] + (u >> 2) * x_step + w * (kCols * 2),
-                                a.width - w * kCols - x_col[u & 3]);
-#pragma unroll
-    for (int j = 0; j < 2; j++) codes[j] = __builtin_amdgcn_raw_buffer_load_b128(ub, unit_at[j], w * 1024, 0);
-    __builtin_amdgcn_sched_barrier(0);
+    int cur = 0;   // the buffer that holds, or is about to hold, window w
+    fetch_window(tokens_of(a, l), units_of(a, l.block), f, a, l, w, ragged_edge && w == last,
+                 my_tiles, my_blocks);
     for (;;) {
-      // this window's activations into LDS (after the last window's reads: the
-      // LDS serves a wavefront's operations in order)
-#pragma unroll
-      for (int u = 0; u < 16; u++) *reinterpret_cast<u32x4 *>(xt_put + u * 1024) = xv[u];
-      // what this wavefront takes next; after its last window nothing: every
-      // offset outside, zeros that are not used
-      const bool more = w + waves < a.windows;
-      const int wn = w + waves;
-      const int width_next = more ? a.width - wn * kCols : 0;
-#pragma unroll
-      for (int u = 0; u < 16; u++)
-        xv[u] = load_piece<kWide>(xb, x_at[u & 3] + (u >> 2) * x_step + wn * (kCols * 2),
-                                  width_next - x_col[u & 3]);
-      u32x4 codes_next[2];
-#pragma unroll
-      for (int j = 0; j < 2; j++)
-        codes_next[j] = __builtin_amdgcn_raw_buffer_load_b128(ub, more ? unit_at[j] : kOutside,
-                                                              wn * 1024, 0);
-      __builtin_amdgcn_sched_barrier(0);   // the loads stay up here, a window ahead
-#pragma unroll
-      for (int s = 0; s < kSteps; s++) {
-        bf16x8 xa[2], wb[2];
-        const uint32_t get = get_z ^ (32 * s);
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-          xa[i] = *reinterpret_cast<const bf16x8 *>(xt_get + i * (32 * 256) + get);
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-          const uint32_t word = codes[j][s >> 1];
-          u32x4 v;
-#pragma unroll
-          for (int k = 0; k < 4; k++) v[k] = weight_pair(word, 4 * (s & 1) + k, min_max[j]);
-          wb[j] = __builtin_bit_cast(bf16x8, v);
-        }
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-          for (int j = 0; j < 2; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[i], wb[j], acc[i][j], 0, 0, 0);
-      }
+      const int wn = __builtin_amdgcn_readfirstlane(w + kWaves);
+      const bool more = wn < a.windows;
+      const int next = __builtin_amdgcn_readfirstlane(cur ^ 1);
+      // that buffer was read a turn ago, and those reads have been waited for
+      fetch_window(tokens_of(a, l, more), units_of(a, l.block, more), f, a, l, wn,
+                   ragged_edge && wn == last, my_tiles + next * (kWaves * kTileBytes),
+                   my_blocks + next * (kWaves * kBlockBytes));
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerWindow) : "memory");
+      window_steps_counted(
+          static_cast<uint32_t>(reinterpret_cast<uintptr_t>(my_tiles + cur * (kWaves * kTileBytes))),
+          static_cast<uint32_t>(reinterpret_cast<uintptr_t>(my_blocks + cur * (kWaves * kBlockBytes))),
+          l, acc);
       if (!more) break;
       w = wn;
-      codes[0] = codes_next[0];
-      codes[1] = codes_next[1];
+      cur = next;
     }
   }
-  __syncthreads();   // the partial tiles take the place of the activations
+  // nothing is on its way into LDS any more; then the partial tiles take the
+  // place of the activations
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  finish_tile<kTokens / kWaves>(a, l, wave, kWaves, reinterpret_cast<float *>(tiles), acc);
+}
 
-  // Each wavefront's tile into LDS; then added in wavefront order.  Element
-  // (token i, row j) of an accumulator block sits in lane
-  // j + 32 * ((i / 4) % 2), register 4 * (i / 8) + i % 4.
-  float *mine = partial + wave * (kTokens * kRows);
+// ---- any x ------------------------------------------------------------------
+//
+// The same, the activations read element by element into registers and stored
+// into LDS from there (one tile per wavefront, the next window's loads issued
+// as soon as the registers are free): for x rows that are not 16-byte aligned
+// or a width that is not a multiple of 8.  The same sums in the same order.
+
+// Eight activations of one token from byte offset `at` of the buffer on, of
+// which the first `inside` lie inside the width (0 or less: none).
+__device__ __forceinline__ u32x4 load_piece(__amdgpu_buffer_rsrc_t x, uint32_t at, int inside) {
+  uint32_t e[8];
+#pragma unroll
+  for (int q = 0; q < 8; q++)
+    e[q] = __builtin_amdgcn_raw_buffer_load_b16(x, (q < inside ? at : kOutside) + 2 * q, 0, 0);
+  u32x4 v = {e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+  return v;
+}
+
+template <int kWaves>
+__global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void matvec_tiles_ragged_kernel(TileArgs a) {
+  __shared__ u32x4 tile[kWaves * 1024];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const TileLane l = tile_lane(a);
+  const __amdgpu_buffer_rsrc_t xb = tokens_of(a, l), ub = units_of(a, l.block);
+  const Fetch f = fetch_of(a, l.lane);
+  u32x4 *mine = tile + wave * 1024;
+
+  f32x16 acc[2][2];
 #pragma unroll
   for (int i = 0; i < 2; i++)
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
-      for (int v = 0; v < 16; v++) {
-        const int token = i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
-        const int r = j * 32 + (lane & 31);
-        mine[token * kRows + r] = acc[i][j][v];
-      }
-  __syncthreads();
-  // The wavefronts share the tokens; a lane has row `lane` of the block.  Eight
-  // tokens at a time: their y are all requested before the first is needed
-  // (tokens past the last: loads that return zero, stores that are dropped).
-  const int row = block * kRows + lane;
-  if (row < a.height) {
-    const __amdgpu_buffer_rsrc_t yb = buffer_over(
-        a.y + static_cast<int64_t>(t0) * a.ldy,
-        static_cast<uint32_t>((static_cast<int64_t>(rows_here - 1) * a.ldy + a.height) * 2));
-    const uint32_t y_at = static_cast<uint32_t>(row * 2), y_step = static_cast<uint32_t>(a.ldy * 2);
-    for (int first = wave; first < rows_here; first += 8 * waves) {
-      uint16_t before[8];
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+  for (int w = wave; w < a.windows; w += kWaves) {
+    u32x4 codes[2];
 #pragma unroll
-      for (int k = 0; k < 8; k++)
-        before[k] = __builtin_amdgcn_raw_buffer_load_b16(yb, y_at + (first + k * waves) * y_step, 0, 0);
+    for (int j = 0; j < 2; j++) codes[j] = __builtin_amdgcn_raw_buffer_load_b128(ub, l.unit_at[j], w * 1024, 0);
 #pragma unroll
-      for (int k = 0; k < 8; k++) {
-        const int t = first + k * waves;
-        const int at = (t & (kTokens - 1)) * kRows + lane;
-        float sum = partial[at];
-        for (int v = 1; v < waves; v++) sum += partial[v * (kTokens * kRows) + at];
-        // reference sub1_cuda_kernel.cu:200: y[row] += bf16(res), the sum in bf16
-        __builtin_amdgcn_raw_buffer_store_b16(
-            f32_to_bf16(bf16_to_f32(before[k]) + bf16_to_f32(f32_to_bf16(sum))), yb,
-            t < kTokens ? y_at + t * y_step : kOutside, 0, 0);
-      }
-    }
+    for (int u = 0; u < 16; u++)
+      mine[u * 64 + l.lane] = load_piece(xb, f.at[u & 3] + (u >> 2) * f.step + w * (kCols * 2),
+                                         a.width - w * kCols - f.col[u & 3]);
+    window_steps(reinterpret_cast<const unsigned char *>(mine), l, codes, acc);
   }
+  __syncthreads();
+  finish_tile<kTokens / kWaves>(a, l, wave, kWaves, reinterpret_cast<float *>(tile), acc);
 }
 
 // Wavefronts per workgroup for a matrix of `blocks` blocks of 64 rows and
-// `windows` windows: 1, 2, 4 or 8, whichever gives the fewest rounds of
-// workgroups over the chip times the windows a wavefront walks in a row
-// (counting what a workgroup costs besides its windows) at eight tiles of
-// tokens.  It depends on the matrix alone, never on the tokens of a launch, so
-// a token's result is the same whatever launch it is part of.  A CU holds
-// eight of these wavefronts (registers).
+// `windows` windows: 1, 2 or 4, whichever is estimated fastest at nine tiles of
+// tokens (568, the longest sequence of the Switch encoders): rounds of
+// workgroups over the chip, each taking 4 us plus 1.25 us per window that a
+// wavefront walks (measured on the six Switch shapes).  A wavefront has 36 KB
+// of a compute unit's 160 KB of LDS, so a unit holds four.  The choice depends
+// on the matrix alone, never on the tokens of a launch, so a token's result is
+// the same whatever launch it is part of.
 int pick_waves(int blocks, int windows) {
   int best = 1;
   double best_cost = 0;
   for (int n = 1; n <= kMaxWaves; n *= 2) {
-    const int64_t slots = 256 * (8 / n);
-    const int64_t rounds = (8ll * blocks + slots - 1) / slots;
-    const double cost = rounds * (2.0 + 0.9 * ((windows + n - 1) / n));
+    const int64_t slots = 256 * (4 / n);
+    const int64_t rounds = (9ll * blocks + slots - 1) / slots;
+    const double cost = rounds * (4.0 + 1.25 * ((windows + n - 1) / n));
     if (n == 1 || cost < best_cost - 1e-9) {
       best = n;
       best_cost = cost;
     }
   }
   return best;
+}
+
+template <int kWaves>
+void launch_tiles(const TileArgs &a, bool wide, dim3 grid, hipStream_t stream) {
+  if (wide)
+    matvec_tiles_kernel<kWaves><<<grid, 64 * kWaves, 0, stream>>>(a);
+  else
+    matvec_tiles_ragged_kernel<kWaves><<<grid, 64 * kWaves, 0, stream>>>(a);
 }
 
 int check_set(const sub1_matrix_set *ms, const char *who) {
@@ -592,13 +820,11 @@ extern "C" int sub1_matvec_tiles(const sub1_tiles *t, int matrix, const void *x,
     return fail(SUB1_ERR_SHAPE, "%s: token strides of 2^24 elements or more", who);
   const dim3 grid(l.units_down / 2, (tokens + kTokens - 1) / kTokens);
   const int waves = pick_waves(l.units_down / 2, l.windows);
-  const size_t lds_bytes = static_cast<size_t>(waves) * kPartialBytes;
-  auto kernel = wide ? matvec_tiles_kernel<true> : matvec_tiles_kernel<false>;
-  HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(kMaxWaves * kPartialBytes)));
-  sub1::note_kernel(wide ? "matvec_tiles_kernel<true>" : "matvec_tiles_kernel<false>");
-  kernel<<<grid, 64 * waves, lds_bytes, static_cast<hipStream_t>(stream)>>>(a);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  sub1::note_kernel(wide ? "matvec_tiles_kernel" : "matvec_tiles_ragged_kernel");
+  if (waves == 1) launch_tiles<1>(a, wide, grid, s);
+  else if (waves == 2) launch_tiles<2>(a, wide, grid, s);
+  else launch_tiles<4>(a, wide, grid, s);
   HIP_TRY(hipGetLastError());
   return SUB1_OK;
 }
