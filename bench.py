@@ -25,8 +25,9 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel.  A recorded figure, not measured by this run:
 # it comes from rocprofv3 counter runs of this same command (FETCH_SIZE x 2.0 + WRITE_SIZE x
 # 1.0, the factors a 1 GiB device copy reads on those counters), summarised in the file
-# named beside it.  None where no such run was made.
-MEASURED_TRAFFIC = {'c2048-sweep': (4.905e9 + 0.057e9,
+# named beside it (the copy of known size is part of `--sweep-only`).  None where no such
+# run was made.
+MEASURED_TRAFFIC = {'c2048-sweep': (4.884e9 + 0.009e9,
                                     'profiles/moe_prepared_fused_kernel_c2048_sweep.txt')}
 
 WORKLOADS = {
@@ -347,6 +348,15 @@ def main():
     route = torch.arange(experts, dtype=torch.int32, device='cuda')
     y = torch.empty_like(x)
     stream_ptr = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    if args.sweep_only:
+        # One plain elementwise kernel of known size ahead of the timed region (1 GiB read,
+        # 1 GiB written): what a counter run of this command scales FETCH_SIZE and
+        # WRITE_SIZE by.
+        cal = torch.zeros(2, 1 << 28, dtype=torch.int32, device='cuda')
+        torch.add(cal[0], 1, out=cal[1])
+        torch.cuda.synchronize()
+        del cal
 
     wall, us_launch = time_launches(lambda: prep.forward(x, route, y), args.steps,
                                     args.warmup, stream_ptr)
