@@ -40,7 +40,7 @@ extern "C" {
 #define SUB1_DEC_WORDS (2 * SUB1_DICT_ENTRIES)
 #define SUB1_TRIE_ROWS (SUB1_DICT_ENTRIES + 1)
 #define SUB1_TRIE_WORDS (9 * SUB1_TRIE_ROWS)
-#define SUB1_MAX_WIDTH 12288                 /* x is staged in LDS */
+#define SUB1_MAX_WIDTH 12288                 /* sub1_moe_grouped: x is staged in LDS */
 
 /* Message of the last failure on this thread ("" if none). */
 const char *sub1_last_error(void);
@@ -65,13 +65,11 @@ int sub1_build_tables(int32_t *dec_host, int32_t *trie_host);
 
 /*
  * y[r] += bf16( sum_k deq(w[r,k]) * x[k] ),  fp32 accumulation, for any
- * height >= 1 and 1 <= width <= SUB1_MAX_WIDTH.  Replaces `sub1matvec`
- * (reference sub1_cuda.cpp:35-45, sub1_cuda_kernel.cu:70-88,129-202), which
- * handled six hard-coded shapes and silently did nothing for others.
- * The first call with a given `dec` pointer derives a compact device table
- * from it (one allocation, two small kernels and a synchronisation, so not
- * inside a stream capture; cached by the address of dec, see
- * sub1_unregister_dec).
+ * height >= 1 and width >= 1.  Replaces `sub1matvec` (reference
+ * sub1_cuda.cpp:35-45, sub1_cuda_kernel.cu:70-88,129-202), which handled six
+ * hard-coded shapes and silently did nothing for others.  A wavefront per row;
+ * the dictionary entries are read straight from `dec`: nothing is derived,
+ * cached or allocated, so the call may be captured in a stream from the first.
  */
 int sub1_matvec(const int32_t *dec, const int16_t *w_comp, const int32_t *row_off,
                 const void *ter_minmax, const void *x, void *y, int height,
@@ -421,8 +419,9 @@ int sub1_set_wait_limit_us(int64_t microseconds);
 int sub1_test_overstate_wait(int extra);
 
 /*
- * sub1_matvec and sub1_moe_grouped keep the compact table they derive from
- * `dec` by the ADDRESS of dec (per device).  Call this before freeing a dec
+ * sub1_moe_grouped keeps the compact table it derives from `dec` by the
+ * ADDRESS of dec (per device), and the prepare calls remember that they have
+ * compared a dec at that address with the fixed dictionary.  Call this before freeing a dec
  * buffer whose address may be handed out again for other contents; NULL drops
  * every cached table.  Synchronises the device.  (A launch that finds other
  * contents at a cached address sets the flag above and the next call derives
