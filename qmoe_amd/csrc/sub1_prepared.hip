@@ -447,6 +447,7 @@ struct PreparedArgs {
   int hdwords;                   // fused kernel: LDS dwords of h (wo's activations)
   int tail_room;                 // persistent kernel: partial sums (groups x 64 lanes) LDS has room for
   int wi_expect;                 // workgroups of a token's wi a wait expects (k[0].parts outside tests)
+  int by_ticket;                 // shared-token kernel: a workgroup's place comes from the ticket
   int64_t wait_ticks;            // longest wait between workgroups, ticks of wall_clock64
   int32_t *sticky;               // fault flags in pinned host memory
 };
@@ -1514,22 +1515,34 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
 // slice of wo.  Unlike tiles of one projection handed out by ticket, every
 // workgroup works in both phases, the token's activations are staged once per
 // phase and workgroup, and h crosses memory once.
-// The workgroups of a token wait for each other.  The launch keeps the grid
-// (tokens x parts) within one workgroup per compute unit, so that all of them
-// run at once.  Where they cannot (other work on the GPU), the waits still end:
-// the workgroups of a token have consecutive indices and workgroups start in
-// index order, so at most one token of a launch is ever partly on the GPU; all
-// others run to completion and make room.  The wait is bounded like the other
-// kernels' in any case.
+// The workgroups of a token wait for each other.  A grid (tokens x parts) of at
+// most one workgroup per compute unit runs all at once on a GPU that does
+// nothing else, and a workgroup's place in it is its index (no round trip
+// before the work starts; where other work holds compute units, the missing
+// workgroups start when that work ends, and the waits are bounded in any case).
+// A larger grid cannot be on the GPU at once, and there a workgroup takes its
+// place by ticket when it starts (by_ticket): the workgroups that are running
+// then hold the lowest places, the places of a token are consecutive, so at
+// most one token is partly on the GPU whatever order the hardware starts
+// workgroups in; all others run to completion and make room.
 __global__ __launch_bounds__(kMaxThreads) void moe_prepared_shared_kernel(PreparedArgs a) {
   extern __shared__ __align__(16) uint32_t lds[];
+  __shared__ int s_place;
   uint32_t *xa = lds;
   float *partials = reinterpret_cast<float *>(xa + a.xdwords);
   const KindArgs &ki = a.k[0];
   const KindArgs &ko = a.k[1];
   const int parts = ki.parts;
-  const int t = blockIdx.x / parts;
-  const int part = blockIdx.x - t * parts;
+  int place = blockIdx.x;
+  if (a.by_ticket) {
+    if (threadIdx.x == 0)
+      s_place = __hip_atomic_fetch_add(&a.ctrl[kCtrlTicket], 1, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    place = __builtin_amdgcn_readfirstlane(s_place);
+  }
+  const int t = place / parts;
+  const int part = place - t * parts;
   int e = __builtin_amdgcn_readfirstlane(a.token_expert[t]);
   if (e >= a.experts) {
     if (part == 0 && threadIdx.x == 0)
@@ -1538,6 +1551,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_shared_kernel(Prepar
   }
   if (e < 0) {
     if (part == 0) pass_through(a, ko, t, 0, ko.slices);
+    if (a.by_ticket && threadIdx.x == 0) sub1::leave_launch(a.ctrl, gridDim.x);
     return;
   }
   uint16_t *h = a.h + static_cast<int64_t>(t) * ki.height;
@@ -1552,6 +1566,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_shared_kernel(Prepar
             [&]() { await_activations(a, ko, 1, t, xa); },
             [&](int ridx, float res) { write_row(y, ridx, res, kStore); });
   done_waiting(a, t);
+  if (a.by_ticket && threadIdx.x == 0) sub1::leave_launch(a.ctrl, gridDim.x);
 }
 
 // For the batches too small to occupy the GPU with a wavefront per slice: built
@@ -1983,6 +1998,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   const char *base = static_cast<const char *>(p.meta);
 
   PreparedArgs a;
+  a.by_ticket = 0;
   a.stream = static_cast<const uint2 *>(p.codes);
   a.ckpt = reinterpret_cast<const uint16_t *>(a.stream + p.total_chunks * 64);
   a.kinds = p.kinds;
@@ -2227,6 +2243,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     }
     a.tail_room = (waves / 2) * std::max(a.k[0].groups_max, a.k[1].groups_max);
     a.wi_expect = a.k[0].parts + sub1::expect_extra();
+    a.by_ticket = static_cast<int64_t>(tokens) * shared_parts > cus;
     const size_t lds_shared = lds_base + static_cast<size_t>(a.tail_room) * 256;
     const void *fn = reinterpret_cast<const void *>(moe_prepared_shared_kernel);
     HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
