@@ -460,8 +460,49 @@ __host__ __device__ constexpr int activation_dwords(int width) {
 }
 
 // Every load of a thread is in flight before its first LDS store, so a tile
-// pays one memory round trip for its activations, not one per pass.
-__device__ __forceinline__ void stage_activations(uint32_t *xa, const uint16_t *x, int width) {
+// pays one memory round trip for its activations, not one per pass.  In two
+// steps, so that a kernel can ask for the activations long before it needs
+// them: stage_request issues a thread's first four loads (all of them up to a
+// width of eight times the workgroup), stage_finish stores them and does the
+// rest.
+struct StagedPairs {
+  uint32_t v[4];
+};
+
+__device__ __forceinline__ uint32_t load_pair(const uint16_t *x, int m, int width, bool aligned) {
+  uint32_t v = 0u;
+  if (aligned && 2 * m + 1 < width) {
+    v = *reinterpret_cast<const uint32_t *>(x + 2 * m);
+  } else {
+    if (2 * m < width) v = x[2 * m];
+    if (2 * m + 1 < width) v |= static_cast<uint32_t>(x[2 * m + 1]) << 16;
+  }
+  return v;
+}
+
+__device__ __forceinline__ void store_pair(uint32_t *xa, int m, int width, uint32_t v) {
+  if (2 * m >= width) return;
+  // columns 2m and 2m+1 are neighbours among the physical columns too
+  uint32_t *p = xa + 2 * physical_column(2 * m);
+  p[0] = v & 0xffffu;
+  p[1] = v << 16;
+  if (2 * m + 1 < width) {
+    p[2] = v >> 16;
+    p[3] = v & 0xffff0000u;
+  }
+}
+
+__device__ __forceinline__ StagedPairs stage_request(const uint16_t *x, int width) {
+  const bool aligned = (reinterpret_cast<uintptr_t>(x) & 3u) == 0;
+  StagedPairs s;
+#pragma unroll
+  for (int u = 0; u < 4; u++)
+    s.v[u] = load_pair(x, threadIdx.x + u * blockDim.x, width, aligned);
+  return s;
+}
+
+__device__ __forceinline__ void stage_finish(uint32_t *xa, const uint16_t *x, int width,
+                                             const StagedPairs &s) {
   const int npairs = (width + 1) / 2;
   const int step = blockDim.x;
   const bool aligned = (reinterpret_cast<uintptr_t>(x) & 3u) == 0;
@@ -469,34 +510,20 @@ __device__ __forceinline__ void stage_activations(uint32_t *xa, const uint16_t *
     xa[2 * z] = 0u;
     xa[2 * z + 1] = 0u;
   }
-  for (int m0 = threadIdx.x; m0 < npairs; m0 += 4 * step) {
+#pragma unroll
+  for (int u = 0; u < 4; u++) store_pair(xa, threadIdx.x + u * step, width, s.v[u]);
+  for (int m0 = threadIdx.x + 4 * step; m0 < npairs; m0 += 4 * step) {
     uint32_t v[4];
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
-      const int m = m0 + u * step;
-      v[u] = 0u;
-      if (aligned && 2 * m + 1 < width) {
-        v[u] = *reinterpret_cast<const uint32_t *>(x + 2 * m);
-      } else {
-        if (2 * m < width) v[u] = x[2 * m];
-        if (2 * m + 1 < width) v[u] |= static_cast<uint32_t>(x[2 * m + 1]) << 16;
-      }
-    }
+    for (int u = 0; u < 4; u++) v[u] = load_pair(x, m0 + u * step, width, aligned);
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
-      const int m = m0 + u * step;
-      if (m < npairs) {
-        // columns 2m and 2m+1 are neighbours among the physical columns too
-        uint32_t *p = xa + 2 * physical_column(2 * m);
-        p[0] = v[u] & 0xffffu;
-        p[1] = v[u] << 16;
-        if (2 * m + 1 < width) {
-          p[2] = v[u] >> 16;
-          p[3] = v[u] & 0xffff0000u;
-        }
-      }
-    }
+    for (int u = 0; u < 4; u++) store_pair(xa, m0 + u * step, width, v[u]);
   }
+}
+
+__device__ __forceinline__ void stage_activations(uint32_t *xa, const uint16_t *x, int width) {
+  const StagedPairs s = stage_request(x, width);
+  stage_finish(xa, x, width, s);
 }
 
 typedef __attribute__((address_space(3))) const uint32_t lds_word;
@@ -525,6 +552,34 @@ __device__ __forceinline__ void add_chunk(uint2 cw, uint32_t &at, float &acc, bf
     const bf16x2 v = __builtin_bit_cast(bf16x2, *(lds_word *)static_cast<uintptr_t>(at));
     acc = __builtin_amdgcn_fdot2_f32_bf16(v, minmax, acc, false);
   }
+}
+
+// The same sums in the same order with all nine LDS reads of the chunk asked
+// for before the first is used: where a compute unit has few wavefronts at work
+// (a handful of tokens), a walk is a chain of LDS round trips, and this makes it
+// one per chunk instead of one per entry.  (With sixteen wavefronts at it the
+// LDS is busy either way, and the registers are better spent elsewhere.)
+__device__ __forceinline__ void add_chunk_ahead(uint2 cw, uint32_t &at, float &acc,
+                                                bf16x2 minmax) {
+  const uint32_t mid = __builtin_amdgcn_alignbit(cw.y, cw.x, 28);
+  uint32_t f[kFields], where[kFields];
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    asm("v_bfe_u32 %0, %1, %2, 7" : "=v"(f[q]) : "v"(cw.x), "n"(kFieldBits * q));
+    asm("v_bfe_u32 %0, %1, %2, 7" : "=v"(f[4 + q]) : "v"(mid), "n"(kFieldBits * q));
+  }
+  asm("v_bfe_u32 %0, %1, 24, 7" : "=v"(f[8]) : "v"(cw.y));
+#pragma unroll
+  for (int q = 0; q < kFields; q++) {
+    asm("v_lshl_add_u32 %0, %1, 2, %2" : "=v"(where[q]) : "v"(f[q]), "v"(q ? where[q - 1] : at));
+  }
+  at = where[kFields - 1];
+  bf16x2 v[kFields];
+#pragma unroll
+  for (int q = 0; q < kFields; q++)
+    v[q] = __builtin_bit_cast(bf16x2, *(lds_word *)static_cast<uintptr_t>(where[q]));
+#pragma unroll
+  for (int q = 0; q < kFields; q++) acc = __builtin_amdgcn_fdot2_f32_bf16(v[q], minmax, acc, false);
 }
 
 // A chunk of the stream.  kOnce: the launch reads more of the stream than the
@@ -558,6 +613,36 @@ __device__ __forceinline__ void add_entries(uint2 cw, int n, uint32_t &at, float
   }
 }
 
+// The same with the reads asked for together (see add_chunk_ahead).
+__device__ __forceinline__ void add_entries_ahead(uint2 cw, int n, uint32_t &at, float &acc,
+                                                  bf16x2 minmax) {
+  if (n == kFields) {
+    add_chunk_ahead(cw, at, acc, minmax);
+    return;
+  }
+  unsigned long long w = (static_cast<unsigned long long>(cw.y) << 32) | cw.x;
+  uint32_t where[kFields - 1];
+  bf16x2 v[kFields - 1];
+#pragma unroll
+  for (int q = 0; q < kFields - 1; q++) {
+    where[q] = (q ? where[q - 1] : at) + ((static_cast<uint32_t>(w) & static_cast<uint32_t>(kMaxStep)) << 2);
+    w >>= kFieldBits;
+  }
+#pragma unroll
+  for (int q = 0; q < kFields - 1; q++)
+    if (q < n) v[q] = __builtin_bit_cast(bf16x2, *(lds_word *)static_cast<uintptr_t>(where[q]));
+#pragma unroll
+  for (int q = 0; q < kFields - 1; q++)
+    if (q < n) acc = __builtin_amdgcn_fdot2_f32_bf16(v[q], minmax, acc, false);
+  if (n > 0) {
+    uint32_t last = where[0];
+#pragma unroll
+    for (int q = 1; q < kFields - 1; q++)
+      if (q < n) last = where[q];
+    at = last;
+  }
+}
+
 // This lane's chunk 0 of the slice that starts at chunk `base` of the stream.
 __device__ __forceinline__ const uint2 *chunk_pointer(const uint2 *stream, uint32_t base) {
   return stream + static_cast<int64_t>(base) * 64 + (threadIdx.x & 63);
@@ -581,20 +666,21 @@ typedef Walk<kRing> SliceWalk;
 
 // g_lo, g_hi: the run of chunk groups to walk, for a wavefront that shares the
 // slice with others (it then starts from the position checkpoint of group g_lo).
+// (len, base: the slice's description, where the caller has read it already.)
 template <int R = kRing, bool kOnce = false>
-__device__ __forceinline__ Walk<R, kOnce> load_slice(const PreparedArgs &a, const KindArgs &k,
-                                                     int64_t sl, int g_lo = 0,
-                                                     int g_hi = 1 << 20) {
+__device__ __forceinline__ Walk<R, kOnce> load_slice_described(const PreparedArgs &a,
+                                                               const KindArgs &k, int64_t sl,
+                                                               int len, uint32_t base, int g_lo,
+                                                               int g_hi) {
   const int lane = threadIdx.x & 63;
   Walk<R, kOnce> w;
-  const int len = __builtin_amdgcn_readfirstlane(k.slice_len[sl]);
   const int nch_all = chunks_of(len);
   w.nch = min(g_hi * kGroupChunks, nch_all);
   w.last = w.nch == nch_all ? last_entries_of(len) : kFields;
   w.c0 = g_lo * kGroupChunks;
   w.ridx = k.row_idx[sl * 64 + lane];
   w.minmax = k.minmax[sl * 64 + lane];
-  w.base = __builtin_amdgcn_readfirstlane(k.slice_base[sl]);
+  w.base = base;
   w.j0 = 0;
   if (g_lo)
     w.j0 = a.ckpt[(checkpoint_entry(w.base, k.first_slice + sl) + g_lo) * 64 + lane];
@@ -602,6 +688,16 @@ __device__ __forceinline__ Walk<R, kOnce> load_slice(const PreparedArgs &a, cons
 #pragma unroll
   for (int i = 0; i < R; i++) w.ring[i] = load_chunk<kOnce>(p + min(w.c0 + i, w.nch - 1) * 64);
   return w;
+}
+
+template <int R = kRing, bool kOnce = false>
+__device__ __forceinline__ Walk<R, kOnce> load_slice(const PreparedArgs &a, const KindArgs &k,
+                                                     int64_t sl, int g_lo = 0,
+                                                     int g_hi = 1 << 20) {
+  const int len_word = k.slice_len[sl];
+  const uint32_t base_word = k.slice_base[sl];
+  return load_slice_described<R, kOnce>(a, k, sl, __builtin_amdgcn_readfirstlane(len_word),
+                                        __builtin_amdgcn_readfirstlane(base_word), g_lo, g_hi);
 }
 
 // R chunks (the depth of the walk's ring) starting at chunk c added onto the
@@ -613,6 +709,8 @@ template <bool kChecked, int R, bool kOnce>
 __device__ __forceinline__ void run_chunks(Walk<R, kOnce> &w, const uint2 *p, int c, uint32_t &at,
                                            float &part, bf16x2 minmax) {
   const int nch = w.nch;
+  // the deep ring is the one of the walks built for latency
+  constexpr bool kAhead = R == kSplitRing;
 #pragma unroll
   for (int i = 0; i < R; i++) {
     if (!kChecked) {
@@ -620,11 +718,14 @@ __device__ __forceinline__ void run_chunks(Walk<R, kOnce> &w, const uint2 *p, in
       // unconditional, clamped to the last chunk: the load can target the ring
       // register itself and the loop needs no wait for it
       w.ring[i] = load_chunk<kOnce>(p + min(c + i + R, nch - 1) * 64);
-      add_chunk(cw, at, part, minmax);
+      if (kAhead) add_chunk_ahead(cw, at, part, minmax);
+      else add_chunk(cw, at, part, minmax);
     } else if (c + i < nch - 1) {
-      add_chunk(w.ring[i], at, part, minmax);
+      if (kAhead) add_chunk_ahead(w.ring[i], at, part, minmax);
+      else add_chunk(w.ring[i], at, part, minmax);
     } else if (c + i == nch - 1) {
-      add_entries(w.ring[i], w.last, at, part, minmax);
+      if (kAhead) add_entries_ahead(w.ring[i], w.last, at, part, minmax);
+      else add_entries(w.ring[i], w.last, at, part, minmax);
     }
   }
 }
@@ -1081,6 +1182,38 @@ __device__ __forceinline__ void walk_tile(const PreparedArgs &a, const KindArgs 
     split = min(waves / rest, k.groups_max);
   const int count = split > 1 ? all - rest : all;
   const int passes = (count + waves - 1) / waves + (split > 1);
+  // the shared last pass: slice `tail_sl` of the tile, this wavefront its
+  // groups g_lo .. g_hi - 1 of `groups`
+  const int tail_sl = count + wave / split;
+  const int sub = wave % split;
+  const int64_t tail_slice = first + static_cast<int64_t>(tail_sl) * stride;
+  // With a few tokens that pass is the whole walk, and the walk a chain of
+  // memory round trips: its loads (the slice's description, then a whole group
+  // of chunks) go out before the wait and the staging like the first loads of
+  // any other walk.
+  const bool tail_only = split > 1 && count == 0;
+  int groups = 0, g_lo = 0, g_hi = 0, tail_len = 0;
+  uint32_t tail_base = 0;
+  auto tail_groups = [&]() {
+    if (tail_sl < all) {
+      // both words of the slice's description in one round trip
+      const int len_word = k.slice_len[tail_slice];
+      const uint32_t base_word = k.slice_base[tail_slice];
+      tail_len = __builtin_amdgcn_readfirstlane(len_word);
+      tail_base = __builtin_amdgcn_readfirstlane(base_word);
+      groups = (chunks_of(tail_len) + kGroupChunks - 1) / kGroupChunks;
+      g_lo = sub * groups / split;
+      g_hi = (sub + 1) * groups / split;
+    }
+  };
+  Walk<kSplitRing> tail_ahead;
+  int tail_ridx = 0xffff;   // the rows of the shared slice, in the wavefront that adds them up
+  if (tail_only) {
+    if (sub == 0 && tail_sl < all) tail_ridx = k.row_idx[tail_slice * 64 + (threadIdx.x & 63)];
+    tail_groups();
+    if (g_lo < g_hi)
+      tail_ahead = load_slice_described<kSplitRing>(a, k, tail_slice, tail_len, tail_base, g_lo, g_hi);
+  }
   int s = slice_of_pass(0, wave, waves, count);
   SliceWalk cur;
   // the first loads of the stream go out before the wait and the staging
@@ -1098,32 +1231,22 @@ __device__ __forceinline__ void walk_tile(const PreparedArgs &a, const KindArgs 
   if (split > 1) {
     __builtin_amdgcn_s_setprio(0);
     const int lane = threadIdx.x & 63;
-    const int sl = count + wave / split;
-    const int sub = wave % split;
-    const int64_t slice = first + static_cast<int64_t>(sl) * stride;
     float *mine = partials + (wave / split) * k.groups_max * 64;
-    int groups = 0;
-    if (sl < all) {
-      groups = (chunks_of(__builtin_amdgcn_readfirstlane(k.slice_len[slice])) + kGroupChunks - 1) /
-               kGroupChunks;
-      const int g_lo = sub * groups / split, g_hi = (sub + 1) * groups / split;
+    if (tail_only) {
+      if (g_lo < g_hi) run_slice(tail_ahead, a.stream, act, mine);
+    } else {
+      if (sub == 0 && tail_sl < all) tail_ridx = k.row_idx[tail_slice * 64 + lane];
+      tail_groups();
       if (g_lo < g_hi) {
-        if (count == 0) {
-          // this pass is all there is (a few tokens): the walk is a chain of
-          // memory round trips, so a whole group of chunks is kept in flight
-          Walk<kSplitRing> tail = load_slice<kSplitRing>(a, k, slice, g_lo, g_hi);
-          run_slice(tail, a.stream, act, mine);
-        } else {
-          SliceWalk tail = load_slice(a, k, slice, g_lo, g_hi);
-          run_slice(tail, a.stream, act, mine);
-        }
+        SliceWalk tail = load_slice_described(a, k, tail_slice, tail_len, tail_base, g_lo, g_hi);
+        run_slice(tail, a.stream, act, mine);
       }
     }
     __syncthreads();
-    if (sub == 0 && sl < all) {
+    if (sub == 0 && tail_sl < all) {
       float sum = 0.f;
       for (int g = 0; g < groups; g++) sum += mine[g * 64 + lane];
-      out(k.row_idx[slice * 64 + lane], sum);
+      out(tail_ridx, sum);
     }
   }
 }
@@ -1543,6 +1666,9 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_shared_kernel(Prepar
   }
   const int t = place / parts;
   const int part = place - t * parts;
+  // the token's activations are asked for before anything else is known
+  const uint16_t *x = a.x + static_cast<int64_t>(t) * a.ldx;
+  const StagedPairs x_ahead = stage_request(x, ki.width);
   int e = __builtin_amdgcn_readfirstlane(a.token_expert[t]);
   if (e >= a.experts) {
     if (part == 0 && threadIdx.x == 0)
@@ -1557,7 +1683,10 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_shared_kernel(Prepar
   uint16_t *h = a.h + static_cast<int64_t>(t) * ki.height;
   walk_tile(a, ki, static_cast<int64_t>(e) * ki.slices + part, parts,
             (ki.slices - part + parts - 1) / parts, xa, partials,
-            [&]() { await_activations(a, ki, 0, t, xa); },
+            [&]() {
+              stage_finish(xa, x, ki.width, x_ahead);
+              __syncthreads();
+            },
             [&](int ridx, float res) { write_row(h, ridx, res, kStoreRelu); });
   publish_h(a, t);
   uint16_t *y = a.y + static_cast<int64_t>(t) * a.ldy;
