@@ -818,9 +818,9 @@ extern "C" int sub1_matvec_tiles(const sub1_tiles *t, int matrix, const void *x,
   const bool wide = !misaligned(x, 16) && ldx % 8 == 0 && t->width % 8 == 0;
   if (ldx >= (1 << 24) || ldy >= (1 << 24))
     return fail(SUB1_ERR_SHAPE, "%s: token strides of 2^24 elements or more", who);
+  hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid(l.units_down / 2, (tokens + kTokens - 1) / kTokens);
   const int waves = pick_waves(l.units_down / 2, l.windows);
-  hipStream_t s = static_cast<hipStream_t>(stream);
   sub1::note_kernel(wide ? "matvec_tiles_kernel" : "matvec_tiles_ragged_kernel");
   if (waves == 1) launch_tiles<1>(a, wide, grid, s);
   else if (waves == 2) launch_tiles<2>(a, wide, grid, s);

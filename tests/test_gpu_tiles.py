@@ -41,7 +41,7 @@ def check_tokens(oracle, c, xs, pre, got, rows):
 
 @pytest.mark.parametrize('height,width,p0,tokens', [
     (3072, 768, 0.9, 568), (768, 3072, 0.9, 200), (4096, 1024, 0.88, 64), (1024, 4096, 0.88, 129),
-    (6144, 2080, 0.9, 70), (2080, 6144, 0.9, 65),
+    (6144, 2080, 0.9, 70), (2080, 6144, 0.9, 65), (2080, 6144, 0.9, 300),
     (77, 333, 0.7, 100),          # ragged rows, columns and tokens; odd width: x rows unaligned
     (130, 15, 0.3, 64), (1, 4000, 0.95, 3), (200, 129, 0.0, 67), (64, 128, 0.5, 1)])
 def test_tiles_product(gpu, oracle, height, width, p0, tokens):
