@@ -57,15 +57,19 @@ class Sub1Linear(nn.Module):
         self.register_buffer('ter_minmax', torch.zeros(2 * height, dtype=torch.bfloat16))
         self.register_buffer('weight', torch.zeros(0, dtype=torch.bfloat16))
 
-    # forward() goes through copies of the weights made from the codes on first
-    # use (each costs about as much memory again as w_comp and is remade when a
-    # buffer is replaced or written in place): for up to `tile_tokens` - 1 tokens
-    # the prepared stream of the non-zero weights, walked per token; from
-    # `tile_tokens` tokens on the tile form that the matrix cores multiply from,
-    # the weights decoded once per 64 tokens.  Set `fast` to False to run
-    # straight from the packed buffers instead.  (The three add a row's terms in
-    # different orders and agree to rounding, not to the bit.)
+    # forward() on one or two tokens runs straight from the packed buffers, a
+    # wavefront per row (nothing is faster for a single product: 3.8 to 7.8 us
+    # of kernel time on the Switch shapes).  More tokens go through copies of
+    # the weights made from the codes on first use (each costs about as much
+    # memory again as w_comp and is remade when a buffer is replaced or written
+    # in place): up to `tile_tokens` - 1 tokens the prepared stream of the
+    # non-zero weights, walked per token; from `tile_tokens` tokens on the tile
+    # form that the matrix cores multiply from, the weights decoded once per 64
+    # tokens.  Set `fast` to False to run straight from the packed buffers
+    # whatever the number of tokens.  (The three add a row's terms in different
+    # orders and agree to rounding, not to the bit.)
     fast = True
+    packed_tokens = 2
     tile_tokens = 64
 
     def _copy(self, kind, width):
@@ -95,7 +99,8 @@ class Sub1Linear(nn.Module):
         x = x.contiguous()
         if self.fast and x.shape[0] >= self.tile_tokens:
             self._copy('tiles', x.shape[1]).matvec_tokens(x, y)
-        elif self.fast and x.shape[1] <= sub1_hip.PREPARED_MAX_WIDTH:
+        elif (self.fast and x.shape[0] > self.packed_tokens
+              and x.shape[1] <= sub1_hip.PREPARED_MAX_WIDTH):
             self._prepared(x.shape[1]).matvec_tokens(x, y)
         else:
             table = DEC[self.w_comp.device.index]

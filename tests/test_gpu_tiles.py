@@ -137,8 +137,9 @@ def test_tiles_matrix_set_and_arguments(gpu, oracle):
 
 def test_sub1linear_takes_the_tiles_from_64_tokens_on(gpu, oracle):
     """Sub1Linear.forward on a sequence: the tile form from `tile_tokens` tokens
-    on, the prepared stream below; both within the tolerance of the dense
-    product, and the tile copy follows the buffers like the prepared one."""
+    on, the prepared stream below, the packed buffers for one or two tokens; all
+    within the tolerance of the dense product, and the tile copy follows the
+    buffers like the prepared one."""
     sub1, op = gpu
     from qmoe_amd import _lib
     t, mm = so.synthetic_ternary(320, 512, 0.85, seed=77)
@@ -152,5 +153,9 @@ def test_sub1linear_takes_the_tiles_from_64_tokens_on(gpu, oracle):
     y_few = lin(x[:10])
     assert _lib.load().sub1_last_kernel() != b'matvec_tiles_kernel'
     assert torch.linalg.norm(y_few.float() - ref[:10]) <= REL_TOL * torch.linalg.norm(ref[:10])
+    # one or two tokens: straight from the packed buffers, a wavefront per row
+    y_two = lin(x[:2])
+    assert _lib.load().sub1_last_kernel() == b'matvec_wave_kernel<4>'
+    assert torch.linalg.norm(y_two.float() - ref[:2]) <= REL_TOL * torch.linalg.norm(ref[:2])
     lin.ter_minmax = (lin.ter_minmax.float() * 2).bfloat16()
     assert torch.equal(lin(x).float(), 2 * y.float())
