@@ -274,6 +274,68 @@ def single_matrix_protocol(seed, stream_ptr):
     return rows
 
 
+def faster_mlp_protocol(stack, seed, stream_ptr, tokens=64):
+    """The sparse-MLP module around the experts (reference sub1.py:299-321) on
+    `tokens` tokens: router, one launch over the experts, probability scaling,
+    beside the reference's own way through the same modules, a Python loop over
+    the experts that received tokens with two products per token.  The router
+    is transformers' SwitchTransformersTop1Router built from a config where
+    transformers can be imported."""
+    import types
+    import torch
+    import torch.nn as nn
+    from qmoe_amd import sub1, synthetic
+    experts, d_model, d_ff = stack.experts, stack.d_model, stack.d_ff
+
+    class Expert(nn.Module):
+        def __init__(self, wi, wo):
+            super().__init__()
+            self.wi, self.wo = wi, wo
+
+        def forward(self, x):
+            return self.wo(torch.relu(self.wi(x)))
+
+    def layer(triple, height):
+        lin = sub1.Sub1Linear(height, triple[0].numel())
+        lin.w_comp.data, lin.row_off.data, lin.ter_minmax.data = triple
+        return lin
+
+    modules = nn.ModuleDict()
+    for e in range(experts):
+        wi, wo = synthetic.expert_layers(stack, e)
+        modules['expert_%d' % e] = Expert(layer(wi, d_ff), layer(wo, d_model))
+    try:
+        from transformers import SwitchTransformersConfig
+        from transformers.models.switch_transformers.modeling_switch_transformers import (
+            SwitchTransformersTop1Router)
+        cfg = SwitchTransformersConfig(d_model=d_model, d_ff=d_ff, num_experts=experts,
+                                       expert_capacity=tokens, router_jitter_noise=0.0)
+        router, which = SwitchTransformersTop1Router(cfg).cuda().eval(), 'transformers'
+    except Exception as exc:                                   # absent or another layout
+        return {'skipped': 'no transformers router: %s' % type(exc).__name__}
+    fast = sub1.FasterMLP(types.SimpleNamespace(router=router, experts=modules),
+                          router_outputs=False)
+    hidden = synthetic.activations(tokens, d_model, seed).view(1, tokens, d_model)
+
+    def loop():                      # reference sub1.py:306-321 on the same modules
+        mask, probs, _ = sub1._router_outputs(router(hidden), experts)
+        next_states = hidden.clone()
+        for e in torch.nonzero(mask.sum(dim=(0, 1)), as_tuple=True)[0]:
+            sel = mask[:, :, e].bool()
+            next_states[sel] = modules['expert_%d' % int(e)](hidden[sel])
+        return probs * next_states
+
+    with torch.no_grad():
+        a, b = fast(hidden), loop()
+        diff = rel_diff(a, b)
+        _, us_fast = time_launches(lambda: fast(hidden), 50, 5, stream_ptr)
+        _, us_router = time_launches(lambda: router(hidden), 50, 5, stream_ptr)
+        _, us_loop = time_launches(loop, 5, 1, stream_ptr, preheat_s=0.0)
+    return {'tokens': tokens, 'router': which, 'module_us': round(us_fast, 1),
+            'router_alone_us': round(us_router, 1), 'expert_loop_us': round(us_loop, 1),
+            'vs_expert_loop_rel_diff': diff}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -473,6 +535,7 @@ def main():
                 yb = torch.empty_like(xb)
                 _, us_b = time_launches(lambda: pr.forward(xb, rb, yb), 30, 5, stream_ptr)
                 entry['tokens4096_us_per_layer'] = round(us_b, 1)
+                entry['faster_mlp'] = faster_mlp_protocol(st, args.seed + 14, stream_ptr)
             also[name] = entry
             del st, pr
     if not args.no_dense:
