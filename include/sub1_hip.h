@@ -133,12 +133,16 @@ int sub1_decode(const int32_t *dec, const int16_t *w_comp, const int32_t *row_of
  *   wo_row_off        int32 [E, d_model+1]
  *   wi_minmax         bf16  [E, 2*d_ff]
  *   wo_minmax         bf16  [E, 2*d_model]
- * workspace: sub1_moe_workspace_bytes(tokens, d_ff) bytes of device memory,
- * 256-byte aligned, ZEROED ONCE by the caller before its first use (its first
- * 32 + 4 * tokens bytes are control words; the rest, h, may hold anything).
- * Every launch leaves the control words it counts with at zero again, so a
- * launch is one kernel and the same workspace serves any number of launches of
- * any batch size that fits it; launches that share a workspace must not overlap
+ * workspace: at least sub1_moe_workspace_bytes(tokens, d_ff) bytes of device
+ * memory, 256-byte aligned, ZEROED ONCE by the caller before its first use.
+ * Its head holds the control words (a fixed part of 192 KB, then 64 bytes per
+ * token); h, which may hold anything, is kept in the LAST tokens * d_ff * 2
+ * bytes of the workspace_bytes given.  Every launch leaves the control words it
+ * counts with at zero again, so a launch is one kernel and the same workspace
+ * serves any number of launches of any batch size that fits it, in any order:
+ * give every launch the size of the whole buffer as workspace_bytes, not the
+ * size that launch needs, so that a small launch's h stays clear of the words
+ * a larger one counts with.  Launches that share a workspace must not overlap
  * in time.  Words 1 and 2 (int32) count, over all launches, the waits that gave
  * up and the tokens whose expert id was >= experts (those tokens are passed
  * through like dropped ones).  After a wait fault (sub1_fault_flags) zero the

@@ -11,6 +11,7 @@ DEC_WORDS = 2 * DICT_ENTRIES
 TRIE_ROWS = DICT_ENTRIES + 1
 MAX_WIDTH = 12288
 PREPARED_MAX_WIDTH = 12288
+STATIC_SCRATCH_BYTES = 1 << 20   # SUB1_STATIC_SCRATCH_BYTES
 
 _vp = ctypes.c_void_p
 _int = ctypes.c_int

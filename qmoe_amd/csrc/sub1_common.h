@@ -84,13 +84,44 @@ constexpr int kCtrlGaveUp = 1;     // waits that reached their time limit, all l
 constexpr int kCtrlBadIds = 2;     // tokens whose expert id was >= experts, all launches so far
 constexpr int kCtrlTiles = 3;      // tiles of a launch with tokens grouped by expert
 constexpr int kCtrlExits = 4;      // workgroups of a persistent launch that have left
-constexpr int kCtrlHeader = 8;     // then one word per token:
+constexpr int kCtrlLaunch = 6;     // and 7, one 64-bit count: launches that handed h over by tag
+// Words 64 on: the tagged copy of h, for launches of a token or two whose
+// workgroups hand h over without counting.  An entry is 64 bits, a bf16 value
+// under a 48-bit tag, written and read as one word: the tag is the number of
+// such launches on this workspace so far plus one, so an entry that carries it
+// was written by this launch (zeroed memory carries none), and nothing has to
+// be cleared, counted or fenced.  Only those launches touch the region, and it
+// lies at the same place whatever the batch.
+constexpr int kTaggedTokens = 2;
+constexpr int kCtrlTagged = 64;
+constexpr int kTaggedWidth = 12288;   // entries per token: the widest h of a prepared stack
+constexpr int kCtrlHeader = kCtrlTagged + kTaggedTokens * kTaggedWidth * 2;   // then one word per token:
 // low half: workgroups that have written their part of the token's h;
-// high half: workgroups that have waited for it (the last of them clears the word)
+// high half: workgroups that have waited for it (the last of them clears the word).
+// The words lie 64 bytes apart: every workgroup of a token adds to its word and
+// polls it, and words that share a 64-byte sector queue behind each other in
+// the L2 (16 tokens' words in one sector cost a 16-token launch 1.5-2.5 us).
 constexpr int kTokenWaited = 1 << 16;
+#ifndef SUB1_TOKEN_STRIDE
+#define SUB1_TOKEN_STRIDE 16
+#endif
+constexpr int kCtrlTokenStride = SUB1_TOKEN_STRIDE;
+
+__host__ __device__ constexpr int token_word(int token) { return kCtrlHeader + token * kCtrlTokenStride; }
 
 inline int64_t control_bytes(int tokens) {
-  return (static_cast<int64_t>(kCtrlHeader + tokens) * 4 + 255) / 256 * 256;
+  return (static_cast<int64_t>(kCtrlHeader) * 4 + static_cast<int64_t>(tokens) * kCtrlTokenStride * 4 + 255) / 256 * 256;
+}
+
+// Where a launch of `tokens` tokens keeps h: the last tokens * d_ff * 2 bytes
+// of the workspace (down to a multiple of 256).  A workspace serves launches of
+// any size that fits it, in any order: h of a small launch must not land on the
+// words that a larger launch counts with afterwards, and from the end it
+// cannot, because the words of the largest launch that fits end before its h
+// begins, and every smaller launch's h lies inside that one's.
+inline char *h_base(void *workspace, int64_t workspace_bytes, int tokens, int d_ff) {
+  const int64_t at = (workspace_bytes - static_cast<int64_t>(tokens) * d_ff * 2) & ~static_cast<int64_t>(255);
+  return static_cast<char *>(workspace) + at;
 }
 
 // Thread 0's bounded wait until the low half of *counter reaches `expect`: relaxed looks at

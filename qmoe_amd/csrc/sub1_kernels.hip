@@ -569,7 +569,7 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
       sub1::drain_stores();
       __syncthreads();
       if (threadIdx.x == 0 && e >= 0)   // a dropped token's word stays untouched
-        __hip_atomic_fetch_add(&a.ctrl[kCtrlHeader + t], 1, __ATOMIC_RELAXED,
+        __hip_atomic_fetch_add(&a.ctrl[sub1::token_word(t)], 1, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
     } else {
       const int j = ticket - n_wi;
@@ -591,7 +591,7 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
         continue;
       }
       if (threadIdx.x == 0)
-        sub1::bounded_wait(&a.ctrl[kCtrlHeader + t], a.wi_expect, a.wait_ticks, a.sticky,
+        sub1::bounded_wait(&a.ctrl[sub1::token_word(t)], a.wi_expect, a.wait_ticks, a.sticky,
                            &a.ctrl[sub1::kCtrlGaveUp]);
       __syncthreads();  // thread 0's acquire now covers the whole workgroup
       stage_activations<kThreads>(lds, a.h + static_cast<int64_t>(t) * a.d_ff, a.d_ff);
@@ -607,7 +607,7 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
         a.y[static_cast<int64_t>(t) * a.d_model + row] = f32_to_bf16(res);
       }
       // said once the tile's work is done: it takes a round trip to memory
-      if (threadIdx.x == 0) sub1::waited_on(&a.ctrl[kCtrlHeader + t], a.wo_tiles);
+      if (threadIdx.x == 0) sub1::waited_on(&a.ctrl[sub1::token_word(t)], a.wo_tiles);
     }
   }
   if (threadIdx.x == 0) sub1::leave_launch(a.ctrl, gridDim.x);
@@ -852,7 +852,7 @@ extern "C" int sub1_moe_grouped(const sub1_moe_stack *st, const int32_t *token_e
   a.x = static_cast<const uint16_t *>(x);
   a.y = static_cast<uint16_t *>(y);
   a.ctrl = static_cast<int32_t *>(workspace);
-  a.h = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + sub1::control_bytes(tokens));
+  a.h = reinterpret_cast<uint16_t *>(sub1::h_base(workspace, workspace_bytes, tokens, st->d_ff));
   a.tokens = tokens;
   a.d_model = st->d_model;
   a.d_ff = st->d_ff;

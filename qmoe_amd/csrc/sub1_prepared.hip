@@ -448,6 +448,7 @@ struct PreparedArgs {
   int tail_room;                 // persistent kernel: partial sums (groups x 64 lanes) LDS has room for
   int wi_expect;                 // workgroups of a token's wi a wait expects (k[0].parts outside tests)
   int by_ticket;                 // shared-token kernel: a workgroup's place comes from the ticket
+  unsigned long long *tagged;    // shared-token kernel: h is handed over by tag (NULL: by count)
   int64_t wait_ticks;            // longest wait between workgroups, ticks of wall_clock64
   int32_t *sticky;               // fault flags in pinned host memory
 };
@@ -1092,7 +1093,7 @@ __device__ __forceinline__ void await_activations(const PreparedArgs &a, const K
                                                   int kind, int t, uint32_t *xa) {
   if (kind == 1) {
     if (threadIdx.x == 0)
-      sub1::bounded_wait(&a.ctrl[kCtrlHeader + t], a.wi_expect, a.wait_ticks, a.sticky,
+      sub1::bounded_wait(&a.ctrl[sub1::token_word(t)], a.wi_expect, a.wait_ticks, a.sticky,
                          &a.ctrl[kCtrlGaveUp]);
     __syncthreads();
   }
@@ -1103,7 +1104,7 @@ __device__ __forceinline__ void await_activations(const PreparedArgs &a, const K
 }
 
 __device__ __forceinline__ void done_waiting(const PreparedArgs &a, int t) {
-  if (threadIdx.x == 0) sub1::waited_on(&a.ctrl[kCtrlHeader + t], a.k[1].parts);
+  if (threadIdx.x == 0) sub1::waited_on(&a.ctrl[sub1::token_word(t)], a.k[1].parts);
 }
 
 // What a ticket stands for.  Every field is the same in all lanes.
@@ -1159,7 +1160,7 @@ __device__ __forceinline__ void publish_h(const PreparedArgs &a, int t) {
   sub1::drain_stores();
   __syncthreads();
   if (threadIdx.x == 0)
-    __hip_atomic_fetch_add(&a.ctrl[kCtrlHeader + t], 1, __ATOMIC_RELAXED,
+    __hip_atomic_fetch_add(&a.ctrl[sub1::token_word(t)], 1, __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -1630,6 +1631,87 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_fused_kernel(Prepare
   if (threadIdx.x == 0) sub1::leave_launch(a.ctrl, gridDim.x);
 }
 
+// ---- h by tag ----------------------------------------------------------------
+//
+// A row of relu(h) into the tagged copy: value and tag in one 64-bit store,
+// written through like the plain rows of h.
+__device__ __forceinline__ void write_tagged(unsigned long long *dst, int ridx, float res,
+                                             unsigned long long tag) {
+  if (ridx == 0xffff) return;   // padding lane
+  uint16_t out = f32_to_bf16(res);
+  if (out & 0x8000u) out = 0;   // relu between the projections, on the bf16 value
+  __hip_atomic_store(&dst[ridx], (tag << 16) | out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The activations of wo from the tagged copy into LDS: a thread reads its
+// entries, all in flight at once, until each carries `want` (the value then
+// belongs to this launch: no count, no fence).  Bounded in time like the other
+// waits; a thread that gives up raises the flag, counts itself and stages what
+// it has.  Ends with a barrier.  The launch runs 1024 threads a workgroup.
+constexpr int kTaggedWidthPerThread = sub1::kTaggedWidth / kMaxThreads;
+__device__ __forceinline__ void await_tagged(const PreparedArgs &a, const KindArgs &k,
+                                             const unsigned long long *src,
+                                             unsigned long long want, uint32_t *xa) {
+  constexpr int kMine = kTaggedWidthPerThread;   // entries a thread may have (width / 1024)
+  const int width = k.width;
+  const int step = blockDim.x;
+  for (int z = threadIdx.x * kZeroPeriod; z < physical_columns(width); z += step * kZeroPeriod) {
+    xa[2 * z] = 0u;
+    xa[2 * z + 1] = 0u;
+  }
+  unsigned long long v[kMine];
+#pragma unroll
+  for (int u = 0; u < kMine; u++) v[u] = 0;
+  int looks = 0;
+  int64_t t0 = 0;
+  for (;;) {
+    bool all = true;
+#pragma unroll
+    for (int u = 0; u < kMine; u++) {
+      const int i = threadIdx.x + u * step;
+      if (i < width && (v[u] >> 16) != want) {
+        v[u] = __hip_atomic_load(&src[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        all = all && (v[u] >> 16) == want;
+      }
+    }
+    if (all) break;
+    if ((++looks & 15) == 1) {
+      const int64_t now = static_cast<int64_t>(wall_clock64());
+      if (looks == 1) t0 = now;
+      if (now - t0 > a.wait_ticks) {
+        sub1::raise_fault(a.sticky, sub1::kFaultWait);
+        __hip_atomic_fetch_add(&a.ctrl[kCtrlGaveUp], 1, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
+    }
+    __builtin_amdgcn_s_sleep(1);
+  }
+#pragma unroll
+  for (int u = 0; u < kMine; u++) {
+    const int i = threadIdx.x + u * step;
+    if (i < width) {
+      uint32_t *p = xa + 2 * physical_column(i);
+      const uint32_t value = static_cast<uint32_t>(v[u]) & 0xffffu;
+      p[0] = value;
+      p[1] = value << 16;
+    }
+  }
+  __syncthreads();
+}
+
+// Thread 0 of a workgroup that leaves a launch of the tagged kind: the last one
+// out makes the next launch's tag.
+__device__ __forceinline__ void leave_tagged(int32_t *ctrl, int workgroups) {
+  const int32_t before = __hip_atomic_fetch_add(&ctrl[sub1::kCtrlExits], 1, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+  if (before + 1 == workgroups) {
+    __hip_atomic_store(&ctrl[sub1::kCtrlExits], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_fetch_add(reinterpret_cast<unsigned long long *>(ctrl + sub1::kCtrlLaunch), 1ull,
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 // Between the latency form and a token per workgroup: with fewer tokens than
 // half the compute units, `parts` workgroups share a token.  Each takes every
 // parts-th slice of wi (the slices are ordered longest first, so the shares are
@@ -1696,6 +1778,56 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_shared_kernel(Prepar
             [&](int ridx, float res) { write_row(y, ridx, res, kStore); });
   done_waiting(a, t);
   if (a.by_ticket && threadIdx.x == 0) sub1::leave_launch(a.ctrl, gridDim.x);
+}
+
+// The shared-token kernel for a token or two, h handed over by tag (see
+// await_tagged): no drain, no barrier, no count between the projections, and no
+// word to give back at the end.  A workgroup's place is its index: the grid is
+// at most 64 workgroups.
+__global__ __launch_bounds__(kMaxThreads) void moe_prepared_tagged_kernel(PreparedArgs a) {
+  extern __shared__ __align__(16) uint32_t lds[];
+  uint32_t *xa = lds;
+  float *partials = reinterpret_cast<float *>(xa + a.xdwords);
+  const KindArgs &ki = a.k[0];
+  const KindArgs &ko = a.k[1];
+  const int parts = ki.parts;
+  const int t = blockIdx.x / parts;
+  const int part = blockIdx.x - t * parts;
+  // the token's activations and this launch's tag (one more than the launches
+  // so far) are asked for before anything else is known
+  const uint16_t *x = a.x + static_cast<int64_t>(t) * a.ldx;
+  const StagedPairs x_ahead = stage_request(x, ki.width);
+  const unsigned long long tag =
+      __hip_atomic_load(reinterpret_cast<unsigned long long *>(a.ctrl + sub1::kCtrlLaunch),
+                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+  int e = __builtin_amdgcn_readfirstlane(a.token_expert[t]);
+  if (e >= a.experts) {
+    if (part == 0 && threadIdx.x == 0)
+      __hip_atomic_fetch_add(&a.ctrl[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    e = -1;
+  }
+  if (e < 0) {
+    if (part == 0) pass_through(a, ko, t, 0, ko.slices);
+    if (threadIdx.x == 0) leave_tagged(a.ctrl, gridDim.x);
+    return;
+  }
+  unsigned long long *ht = a.tagged + static_cast<int64_t>(t) * sub1::kTaggedWidth;
+  walk_tile(a, ki, static_cast<int64_t>(e) * ki.slices + part, parts,
+            (ki.slices - part + parts - 1) / parts, xa, partials,
+            [&]() {
+              stage_finish(xa, x, ki.width, x_ahead);
+              __syncthreads();
+            },
+            [&](int ridx, float res) { write_tagged(ht, ridx, res, tag); });
+  __syncthreads();   // every wavefront is done with x before h takes its place
+  uint16_t *y = a.y + static_cast<int64_t>(t) * a.ldy;
+  // (a test that overstates the wait looks for a tag that nobody writes)
+  const unsigned long long want = a.wi_expect == parts ? tag : tag + 1;
+  walk_tile(a, ko, static_cast<int64_t>(e) * ko.slices + part, parts,
+            (ko.slices - part + parts - 1) / parts, xa, partials,
+            [&]() { await_tagged(a, ko, ht, want, xa); },
+            [&](int ridx, float res) { write_row(y, ridx, res, kStore); });
+  if (threadIdx.x == 0) leave_tagged(a.ctrl, gridDim.x);
 }
 
 // For the batches too small to occupy the GPU with a wavefront per slice: built
@@ -2128,6 +2260,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
 
   PreparedArgs a;
   a.by_ticket = 0;
+  a.tagged = nullptr;
   a.stream = static_cast<const uint2 *>(p.codes);
   a.ckpt = reinterpret_cast<const uint16_t *>(a.stream + p.total_chunks * 64);
   a.kinds = p.kinds;
@@ -2167,7 +2300,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   a.groups = nullptr;
   if (p.kinds == 2) {
     a.ctrl = static_cast<int32_t *>(workspace);
-    a.h = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + sub1::control_bytes(tokens));
+    a.h = reinterpret_cast<uint16_t *>(sub1::h_base(workspace, workspace_bytes, tokens, d_ff));
   }
   a.tokens = tokens;
   a.experts = p.count;
@@ -2377,6 +2510,19 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     const void *fn = reinterpret_cast<const void *>(moe_prepared_shared_kernel);
     HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(lds_shared)));
+    // a token or two: h goes from the wi to the wo workgroups by tag (every
+    // workgroup reads all of it, eight bytes an entry: for small grids only)
+    if (tokens <= sub1::kTaggedTokens && static_cast<int64_t>(tokens) * shared_parts <= 64 &&
+        64 * waves == kMaxThreads) {
+      a.tagged = reinterpret_cast<unsigned long long *>(a.ctrl + sub1::kCtrlTagged);
+      const void *tagged_fn = reinterpret_cast<const void *>(moe_prepared_tagged_kernel);
+      HIP_TRY(hipFuncSetAttribute(tagged_fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  static_cast<int>(lds_shared)));
+      sub1::note_kernel("moe_prepared_tagged_kernel");
+      moe_prepared_tagged_kernel<<<tokens * shared_parts, 64 * waves, lds_shared, s>>>(a);
+      HIP_TRY(hipGetLastError());
+      return SUB1_OK;
+    }
     sub1::note_kernel("moe_prepared_shared_kernel");
     moe_prepared_shared_kernel<<<tokens * shared_parts, 64 * waves, lds_shared, s>>>(a);
     HIP_TRY(hipGetLastError());

@@ -75,9 +75,22 @@ def test_bad_arguments_are_refused_on_the_host():
 
 
 def test_workspace_size():
+    """The workspace holds a fixed head (control words and the tagged copy of h
+    for launches of a token or two), a 64-byte word per token and h; its size
+    is a multiple of 256, grows with the batch, and 64 tokens of a
+    Switch-c-2048 layer fit the static array of the entry point that does not
+    allocate."""
     lib = _lib.load()
-    assert lib.sub1_moe_workspace_bytes(0, 3072) == 256
-    assert lib.sub1_moe_workspace_bytes(64, 6144) == 512 + 64 * 6144 * 2
+    head = lib.sub1_moe_workspace_bytes(0, 3072)
+    assert head == lib.sub1_moe_workspace_bytes(0, 8) and head % 256 == 0
+    assert head >= 64 * 4 + 2 * 12288 * 8
+    last = head
+    for tokens in (1, 2, 3, 64, 65, 1000):
+        need = lib.sub1_moe_workspace_bytes(tokens, 6144)
+        assert need % 256 == 0 and need > last
+        assert head + tokens * (64 + 6144 * 2) <= need < head + tokens * (64 + 6144 * 2) + 256
+        last = need
+    assert lib.sub1_moe_workspace_bytes(64, 6144) <= _lib.STATIC_SCRATCH_BYTES
     assert lib.sub1_moe_workspace_bytes(-1, 8) == 0
 
 

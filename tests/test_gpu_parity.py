@@ -508,6 +508,32 @@ def test_tokens_shared_between_workgroups(gpu, oracle, d_model, d_ff, p0):
     assert np.array_equal(bits_host(y[t]), ref)
 
 
+def test_one_workspace_serves_batches_in_any_order(gpu):
+    """A workspace made for the largest batch then serves smaller and larger
+    ones in any order: a small launch's h must not land on the words a larger
+    launch counts with afterwards (h lies at the end of the workspace, the
+    words at its head).  Both layouts, every launch against the same launch on
+    a fresh workspace."""
+    from qmoe_amd import synthetic
+    experts, d_model, d_ff = 4, 200, 330
+    stack = synthetic.build_stack(experts, d_model, d_ff, 0.8, seed=41)
+    prep = stack.prepare()
+    sizes = (150, 1, 150, 7, 100, 2, 128, 60, 150)
+    xs = {t: synthetic.activations(t, d_model, seed=42 + t) for t in set(sizes)}
+    route = {t: (torch.arange(t, dtype=torch.int32, device='cuda') * 3 + 1) % experts for t in xs}
+    for layer in (prep, stack):
+        want = {}
+        for t in xs:
+            layer._ws.clear()
+            want[t] = layer.forward(xs[t], route[t]).clone()
+        layer._ws.clear()
+        for t in sizes:
+            got = layer.forward(xs[t], route[t])
+            assert torch.equal(got, want[t]), (type(layer).__name__, t)
+        assert len(layer._ws) == 1
+        assert layer.launch_faults(max(sizes)) == (0, 0)
+
+
 def test_shared_token_launches_on_several_streams(gpu):
     """Launches whose workgroups wait for each other (several per token) from
     three streams at once: together they ask for three times the compute

@@ -55,6 +55,14 @@ def test_static_scratch_launch_equals_workspace_launch(oracle):
     for i, e in enumerate(route):
         ref, _ = oracle.expert_ffn(wi[e], wo[e], xs[i], order=2)
         assert np.array_equal(got[i], ref)
+    # and a larger one again: the small call's h must not have landed on the
+    # words that this one's workgroups count with
+    route = [(5 * i + 1) % experts for i in range(40)]
+    xs, got, want = both(route, 1800)
+    assert np.array_equal(got, want)
+    for i in (0, 21, 39):
+        ref, _ = oracle.expert_ffn(wi[route[i]], wo[route[i]], xs[i], order=2)
+        assert np.array_equal(got[i], ref)
     _lib.check_faults()
 
     # more scratch than the array holds: refused, with the size in the message
