@@ -508,6 +508,29 @@ def test_tokens_shared_between_workgroups(gpu, oracle, d_model, d_ff, p0):
     assert np.array_equal(bits_host(y[t]), ref)
 
 
+def test_one_or_two_tokens_dropped_or_out_of_range(gpu):
+    """Launches of one or two tokens hand h over by tag and count nothing per
+    token; a dropped token or one whose expert does not exist still passes
+    through, is counted, and leaves the other token's result and the next
+    launches on the workspace as they were."""
+    from qmoe_amd import _lib, synthetic
+    experts, d_model, d_ff = 3, 512, 1536
+    prep = synthetic.build_stack(experts, d_model, d_ff, 0.85, seed=61).prepare()
+    x = synthetic.activations(2, d_model, seed=62)
+    both = prep.forward(x, torch.tensor([1, 2], dtype=torch.int32, device='cuda')).clone()
+    assert _lib.load().sub1_last_kernel() == b'moe_prepared_tagged_kernel'
+    for route, bad in (([-1, 2], 0), ([1, experts], 1), ([-1, -7], 0), ([experts + 5, -1], 1),
+                       ([1, 2], 0)):
+        y = prep.forward(x, torch.tensor(route, dtype=torch.int32, device='cuda'))
+        assert prep.launch_faults(2) == (0, bad), route
+        for t, e in enumerate(route):
+            assert torch.equal(y[t], both[t] if 0 <= e < experts else x[t]), (route, t)
+    for e, bad in ((-1, 0), (experts, 1), (1, 0)):
+        y = prep.forward(x[:1].contiguous(), torch.tensor([e], dtype=torch.int32, device='cuda'))
+        assert prep.launch_faults(1) == (0, bad), e
+        assert torch.equal(y[0], both[0] if e == 1 else x[0]), e
+
+
 def test_one_workspace_serves_batches_in_any_order(gpu):
     """A workspace made for the largest batch then serves smaller and larger
     ones in any order: a small launch's h must not land on the words a larger
