@@ -146,10 +146,19 @@ __device__ __forceinline__ int for_each_nonzero(const uint16_t *codes, int n,
                                                 const int32_t *__restrict__ dec, int width,
                                                 F &&nz) {
   int col = 0;
+  // the code after next and the next code's entry are asked for before this
+  // code's digits are walked: a row is a chain of dependent loads otherwise
+  int e_next = n > 1 ? codes[1] : 0;
+  const int e_first = n > 0 ? codes[0] : 0;
+  int32_t next0 = dec[2 * e_first], next1 = dec[2 * e_first + 1];
   for (int i = 0; i < n; i++) {
-    const int e = codes[i];
-    const uint32_t w0 = static_cast<uint32_t>(dec[2 * e]);
-    const uint32_t w1 = static_cast<uint32_t>(dec[2 * e + 1]);
+    const uint32_t w0 = static_cast<uint32_t>(next0);
+    const uint32_t w1 = static_cast<uint32_t>(next1);
+    if (i + 1 < n) {
+      next0 = dec[2 * e_next];
+      next1 = dec[2 * e_next + 1];
+    }
+    if (i + 2 < n) e_next = codes[i + 2];
     unsigned long long digits = static_cast<unsigned long long>(w0 >> 4) |
                                 (static_cast<unsigned long long>(w1 >> 4) << 28);
     while (digits) {
