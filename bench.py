@@ -498,6 +498,14 @@ def main():
     also['routed_64_tokens'] = {'us_per_layer': round(us5, 2),
                                 'experts_hit': int(torch.unique(r5).numel()),
                                 'vs_reference_layout_kernel_rel_diff': rel_diff(y5, y5b)}
+    # the batches in between, routed the same way
+    also['routed_tokens_us'] = {}
+    for t in (2, 4, 16, 32):
+        xt = synthetic.activations(t, d_model, args.seed + 3)
+        rt = synthetic.softmax_router(t, experts, args.seed + 4)
+        yt = torch.empty_like(xt)
+        _, us_t = time_launches(lambda: prep.forward(xt, rt, yt), 200, 20, stream_ptr)
+        also['routed_tokens_us'][str(t)] = round(us_t, 2)
     if not args.no_dense:
         n = min(experts, 128)
         d_us = dense_gemv_us(stack, x, n)
