@@ -169,6 +169,21 @@ int sub1_moe_grouped(const sub1_moe_stack *stack, const int32_t *token_expert,
                      int64_t workspace_bytes, void *stream);
 
 /*
+ * token_expert from a top-1 router's mask, in one launch: replaces
+ * `expert_index = torch.argmax(router_mask, dim=-1)` (reference sub1.py:311)
+ * and the test for tokens without an expert (sub1.py:315-318 runs no expert on
+ * a token whose mask row is all zero; such a token keeps its input).
+ *   mask          [tokens, experts], contiguous, integers of element_bytes
+ *                 (8: int64, 4: int32, 1: uint8 / bool)
+ *   route[t]      index of the row's first largest element, or -1 where the row
+ *                 is all zero: the token_expert of the grouped launches
+ *   expert_index  NULL, or int64 [tokens]: the argmax itself (0 for an all-zero
+ *                 row), which the reference returns beside the hidden states
+ */
+int sub1_route_from_mask(const void *mask, int element_bytes, int tokens, int experts,
+                         int32_t *route, int64_t *expert_index, void *stream);
+
+/*
  * Prepared stack: the fast form of sub1_moe_grouped (no counterpart in the
  * reference).  Preparing decodes the stack once and stores every row's
  * non-zero weights as a gap-coded stream the GPU walks at full width:

@@ -92,6 +92,7 @@ PROTOTYPES = {
     'sub1_tiles_entries': (_int, [ctypes.POINTER(MatrixSet), ctypes.POINTER(Tiles), _vp]),
     'sub1_matvec_tiles': (_int, [ctypes.POINTER(Tiles), _int, _vp, _i64, _vp, _i64, _int, _vp]),
     'sub1_tiles_decode': (_int, [ctypes.POINTER(Tiles), _int, _vp, _vp]),
+    'sub1_route_from_mask': (_int, [_vp, _int, _int, _int, _vp, _vp, _vp]),
     'sub1_timing_begin': (_int, [_vp]),
     'sub1_timing_end': (_int, [_vp, ctypes.POINTER(ctypes.c_double)]),
     'sub1_init': (_int, []),

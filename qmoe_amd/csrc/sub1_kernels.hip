@@ -884,6 +884,74 @@ extern "C" int sub1_moe_grouped(const sub1_moe_stack *st, const int32_t *token_e
   return SUB1_OK;
 }
 
+// ---------------------------------------------------------- routing ------
+//
+// A wavefront per token: the first largest element of the token's row of the
+// router's mask (what torch.argmax returns, reference sub1.py:311) and whether
+// the row has a non-zero element at all (a token that the router's capacity
+// limit dropped has none and keeps its input, reference sub1.py:312-318).
+template <typename T>
+__global__ __launch_bounds__(256) void route_from_mask_kernel(const T *__restrict__ mask,
+                                                              int tokens, int experts,
+                                                              int32_t *__restrict__ route,
+                                                              int64_t *__restrict__ index) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= tokens) return;
+  const int lane = threadIdx.x & 63;
+  const T *row = mask + static_cast<int64_t>(t) * experts;
+  long long best = 0;
+  int at = experts;   // no element yet
+  bool any = false;
+  for (int e = lane; e < experts; e += 64) {
+    const long long v = static_cast<long long>(row[e]);
+    any = any || v != 0;
+    if (at == experts || v > best) {
+      best = v;
+      at = e;
+    }
+  }
+  // the lanes' candidates, largest value first, lowest index among equals
+  for (int m = 1; m < 64; m <<= 1) {
+    const long long v = __shfl_xor(best, m, 64);
+    const int a = __shfl_xor(at, m, 64);
+    if (a < experts && (at == experts || v > best || (v == best && a < at))) {
+      best = v;
+      at = a;
+    }
+  }
+  const bool some = __ballot(any) != 0ull;
+  if (lane == 0) {
+    route[t] = some ? at : -1;
+    if (index) index[t] = at;
+  }
+}
+
+extern "C" int sub1_route_from_mask(const void *mask, int element_bytes, int tokens, int experts,
+                                    int32_t *route, int64_t *expert_index, void *stream) {
+  if (!mask || !route) return fail(SUB1_ERR_NULL, "sub1_route_from_mask: NULL argument");
+  if (tokens < 0 || experts < 1)
+    return fail(SUB1_ERR_SHAPE, "sub1_route_from_mask: tokens %d experts %d", tokens, experts);
+  if (element_bytes != 1 && element_bytes != 4 && element_bytes != 8)
+    return fail(SUB1_ERR_SHAPE, "sub1_route_from_mask: elements of %d bytes (1, 4 or 8)",
+                element_bytes);
+  if (misaligned(mask, element_bytes) || misaligned(route, 4) || misaligned(expert_index, 8))
+    return fail(SUB1_ERR_ALIGN, "sub1_route_from_mask: misaligned pointer");
+  if (tokens == 0) return SUB1_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const unsigned grid = static_cast<unsigned>((tokens + 3) / 4);
+  if (element_bytes == 8)
+    route_from_mask_kernel<<<grid, 256, 0, s>>>(static_cast<const int64_t *>(mask), tokens,
+                                                experts, route, expert_index);
+  else if (element_bytes == 4)
+    route_from_mask_kernel<<<grid, 256, 0, s>>>(static_cast<const int32_t *>(mask), tokens,
+                                                experts, route, expert_index);
+  else
+    route_from_mask_kernel<<<grid, 256, 0, s>>>(static_cast<const uint8_t *>(mask), tokens,
+                                                experts, route, expert_index);
+  HIP_TRY(hipGetLastError());
+  return SUB1_OK;
+}
+
 extern "C" int sub1_fault_flags(int32_t *flags) {
   if (!flags) return fail(SUB1_ERR_NULL, "sub1_fault_flags: NULL argument");
   flags[0] = sub1::fault_flag_host(sub1::kFaultWait) ? 1 : 0;

@@ -319,11 +319,11 @@ class FasterMLP(nn.Module):
         their input (reference sub1.py:312-318)."""
         router_mask, router_probs, router_logits = _router_outputs(
             self.router(hidden_states), len(self.experts))
-        expert_index = torch.argmax(router_mask, dim=-1)
-        # a token the capacity limit dropped has an all-zero mask row: expert -1
-        route = torch.where(router_mask.any(dim=-1), expert_index, -1).to(torch.int32)
+        # expert_index = argmax of the mask; a token the capacity limit dropped
+        # has an all-zero mask row: expert -1 for the launch
+        route, expert_index = sub1_hip.route_from_mask(router_mask)
         x = hidden_states.reshape(-1, hidden_states.shape[-1]).to(torch.bfloat16).contiguous()
-        next_states = self._launcher().forward(x, route.reshape(-1))
+        next_states = self._launcher().forward(x, route)
         hidden_states = router_probs * next_states.view(hidden_states.shape).to(hidden_states.dtype)
         if self.router_outputs:
             return hidden_states, (router_logits, expert_index)

@@ -65,6 +65,30 @@ def _need(t, dtype, name, device=None, numel=None, dim=None):
     return t.data_ptr()
 
 
+def route_from_mask(router_mask):
+    """(route int32 [T], expert_index int64 shaped like the mask without its
+    last dimension) from a top-1 router's mask [..., E] in one launch:
+    expert_index = argmax over the experts (reference sub1.py:311), route the
+    same with -1 for a token whose row is all zero (dropped by the router's
+    capacity limit: it keeps its input, reference sub1.py:312-318)."""
+    if not isinstance(router_mask, torch.Tensor) or not router_mask.is_cuda:
+        raise ValueError('router_mask must be a tensor on the GPU')
+    size = {torch.int64: 8, torch.int32: 4, torch.uint8: 1, torch.bool: 1}.get(router_mask.dtype)
+    if size is None:
+        raise TypeError('router_mask must be int64, int32, uint8 or bool, got %s' % router_mask.dtype)
+    mask = router_mask.contiguous()
+    experts = mask.shape[-1]
+    tokens = mask.numel() // experts if experts else 0
+    route = torch.empty(tokens, dtype=torch.int32, device=mask.device)
+    index = torch.empty(mask.shape[:-1], dtype=torch.int64, device=mask.device)
+    if tokens == 0:
+        return route, index
+    with _on_device(mask.device):
+        _lib.check(_lib.load().sub1_route_from_mask(mask.data_ptr(), size, tokens, experts,
+                                                    route.data_ptr(), index.data_ptr(), _stream()))
+    return route, index
+
+
 def build_tables():
     """(dec int32 [131072], trie int32 [65537, 9]) on the CPU: the fixed
     dictionary of reference sub1.py:29-102, built by the library (C++)."""

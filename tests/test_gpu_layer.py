@@ -79,6 +79,43 @@ def test_ternarize_make_forward(gpu):
     assert lin.w_comp.numel() * 2 < 0.2 * w.numel() * 2
 
 
+@pytest.mark.parametrize('dtype', [torch.int64, torch.int32, torch.uint8, torch.bool])
+def test_route_from_mask_is_argmax_with_dropped_tokens(gpu, dtype):
+    """token_expert from a router's mask in one launch: the argmax over the
+    experts (reference sub1.py:311), -1 where a token's row is all zero
+    (reference sub1.py:312-318); one-hot rows, all-zero rows, expert counts
+    that are no multiple of the wavefront, and rows with several ones (the first
+    wins, as in torch.argmax)."""
+    from qmoe_amd import sub1_hip
+    g = torch.Generator().manual_seed(5)
+    for batch, seq, experts in ((2, 37, 128), (1, 1, 2048), (3, 5, 7), (1, 300, 1), (1, 9, 65)):
+        pick = torch.randint(0, experts, (batch, seq), generator=g)
+        mask = torch.nn.functional.one_hot(pick, experts)
+        mask[0, 0] = 0                       # a dropped token
+        if seq > 3:
+            mask[-1, 3] = 0
+            mask[-1, 2, experts // 2:] = 1   # several ones
+        mask = mask.to(dtype).cuda()
+        route, index = sub1_hip.route_from_mask(mask)
+        want = torch.argmax(mask.to(torch.int64), dim=-1)
+        assert index.dtype == torch.int64 and index.shape == mask.shape[:-1]
+        assert torch.equal(index, want)
+        dropped = ~mask.to(torch.bool).any(dim=-1)
+        assert route.dtype == torch.int32 and route.shape == (batch * seq,)
+        assert torch.equal(route, torch.where(dropped, -1, want).reshape(-1).to(torch.int32))
+    if dtype == torch.int64:
+        # a general integer mask: the first largest element, negative values are non-zero
+        mask = torch.tensor([[0, 3, 3, 1], [-2, -1, -1, -5], [0, 0, 0, 0]], device='cuda')
+        route, index = sub1_hip.route_from_mask(mask)
+        assert index.tolist() == [1, 1, 0] and route.tolist() == [1, 1, -1]
+    empty = torch.zeros((0, 8), dtype=dtype, device='cuda')
+    route, index = sub1_hip.route_from_mask(empty)
+    assert route.numel() == 0 and index.numel() == 0
+    with pytest.raises(TypeError):
+        sub1_hip.route_from_mask(torch.zeros((2, 4), device='cuda'))
+
+
+
 @pytest.mark.parametrize('order', ['mask_first', 'probs_first'])
 def test_faster_mlp_equals_the_expert_loop(gpu, order):
     from qmoe_amd import sub1
