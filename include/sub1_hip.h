@@ -145,8 +145,13 @@ int sub1_decode(const int32_t *dec, const int16_t *w_comp, const int32_t *row_of
  * a larger one counts with.  Launches that share a workspace must not overlap
  * in time.  Words 1 and 2 (int32) count, over all launches, the waits that gave
  * up and the tokens whose expert id was >= experts (those tokens are passed
- * through like dropped ones).  After a wait fault (sub1_fault_flags) zero the
- * workspace again.
+ * through like dropped ones).  After a wait fault (sub1_fault_flags) the words
+ * may be left at other values than zero (a workgroup that reports after the
+ * waiters of its token have given up), and no later launch would notice: once
+ * the faulting work has ended, ZERO THE WORKSPACE AGAIN before its next launch.
+ * sub1_fault_epoch() counts the wait faults that sub1_clear_faults() has
+ * cleared; an owner of workspaces keeps the count it saw when it zeroed each
+ * and zeroes again when the count has moved on.
  */
 typedef struct sub1_moe_stack {
   const int32_t *dec;
@@ -271,18 +276,29 @@ int sub1_moe_prepared_decode(const sub1_moe_prepared *prepared, int expert, int 
  * kernels need no scratch memory).  The control words and h live in a static
  * device array of SUB1_STATIC_SCRATCH_BYTES that every GPU the library runs on
  * holds until the process ends; the call allocates nothing, on the device or
- * pinned (so sub1_init() must have run once in the process), and refuses a
- * batch whose sub1_moe_workspace_bytes(tokens, d_ff) exceeds the array (64
- * tokens of a Switch-c-2048 layer fit).  Same kernels and same results as
- * sub1_moe_grouped_prepared.  All calls on one GPU share the one array: two
- * that overlap there (different streams, different threads) race; calls on one
- * stream run in order and are safe.
+ * pinned (so sub1_init() must have run once in the process).  The array is
+ * split once and for all: control words for SUB1_STATIC_MAX_TOKENS tokens at
+ * its head, h in the rest, so that stacks of different d_ff can take turns on
+ * it; a batch of more tokens, or whose h (tokens * d_ff * 2 bytes) is larger
+ * than that rest (799 KB: 66 tokens of a Switch-c-2048 layer), is refused.
+ * Same kernels and same results as sub1_moe_grouped_prepared.  All calls on
+ * one GPU share the one array: two that overlap there (different streams,
+ * different threads) race; calls on one stream run in order and are safe.
+ * After a wait fault (sub1_fault_flags) the control words may be left at other
+ * values than zero: sub1_static_scratch_reset(stream) zeroes them again with one
+ * small kernel on `stream` (no allocation, no memset node), once the work that
+ * faulted has ended.
  */
 #define SUB1_STATIC_SCRATCH_BYTES (1 << 20)
+#define SUB1_STATIC_MAX_TOKENS 512
 
 int sub1_moe_grouped_prepared_static(const sub1_moe_prepared *prepared,
                                      const int32_t *token_expert, const void *x, void *y,
                                      int tokens, void *stream);
+int sub1_static_scratch_reset(void *stream);
+/* The current device's address of that array (its words 1 and 2 count waits
+ * that gave up and tokens with an expert id >= experts, as in a workspace). */
+int sub1_static_scratch_pointer(void **address);
 
 /*
  * The same preparation for plain products: `count` matrices of one shape
@@ -342,16 +358,21 @@ int sub1_matrix_prepared_decode(const sub1_matrix_prepared *prepared, int matrix
  * Many tokens through one matrix on the matrix cores (no counterpart in the
  * reference, whose Sub1Linear.forward launches one product per token,
  * sub1.py:137-142): y[t, :] += W_m x[t, :] for all tokens in one launch, the
- * weights decoded once per tile of 64 tokens into a dense bf16 tile in LDS and
- * multiplied by MFMA.  For that the matrices are copied once into a tile form:
- * rows in their own order in blocks of 64, columns in windows of 128, per
- * (block, window) and row the non-zero weights inside the window as one byte
- * each ((column in the window) * 2 + symbol - 1), eight to an 8-byte chunk
- * interleaved by lane like the prepared stream (about 1.1 to 1.6 bit per
- * weight at 10% non-zeros).  Worth it from a few dozen tokens on; below that
- * sub1_matvec_tokens or sub1_matvec_prepared walk the non-zeros per token.
- * Products are exact and summed in fp32 in the matrix cores' order: results
- * agree with the other kernels to rounding (1e-2 bar), not to the bit.
+ * weights turned back into bf16 values in registers and multiplied by MFMA
+ * (v_mfma_f32_32x32x16_bf16), 64 rows x 64 tokens per workgroup.  For that the
+ * matrices are copied once into a tile form of 2 bits per weight whatever the
+ * density (0 = row min, 1 = row max, 2 = zero): units of 32 rows x 128 columns
+ * of 1 KB, each laid out as the 64 lanes' shares of the MFMA B operand, so that
+ * a wavefront fetches a unit with one 16-byte load per lane and builds the
+ * operands with a byte permute of the row's (min, max) word, without a table;
+ * rows are padded to 64, columns to 128 (c-2048 wi: 3.4 MB against 1.1 MB of
+ * codes).  Worth it from 64 tokens on; below that sub1_matvec_tokens or
+ * sub1_matvec_prepared walk the non-zeros per token.  Products are exact and
+ * summed in fp32 in the matrix cores' order: results agree with the other
+ * kernels to rounding (1e-2 bar), not to the bit.  A zero weight is multiplied
+ * like any other (as the reference kernel does, sub1_cuda_kernel.cu:190): an
+ * infinite or NaN activation makes every row of its token NaN, where the
+ * walking kernels only touch the rows that have a weight in that column.
  *
  *   meta_bytes = sub1_tiles_meta_bytes(count, height, width);
  *   sub1_tiles t;
@@ -424,7 +445,12 @@ int sub1_timing_end(void *stream, double *elapsed_us);
  *   sub1_fault_words_host()   the two flags as int32 words in host memory (NULL
  *                             before sub1_init or a first launch): a caller
  *                             that polls between launches reads them directly.
- *   sub1_clear_faults()       resets both.
+ *   sub1_clear_faults()       resets both; a wait fault among them moves
+ *                             sub1_fault_epoch() on by one.
+ *   sub1_fault_epoch()        wait faults cleared so far: every workspace that
+ *                             was in use before the count moved must be zeroed
+ *                             again before its next launch (and the static
+ *                             scratch by sub1_static_scratch_reset).
  *   sub1_set_wait_limit_us(n) the bound, 1 .. 60 000 000 us, for later launches.
  *   sub1_test_overstate_wait(k)  for tests of the above: later launches expect k
  *                             more workgroups in every wait than will ever
@@ -434,6 +460,7 @@ int sub1_init(void);
 int sub1_fault_flags(int32_t *flags);
 const int32_t *sub1_fault_words_host(void);
 int sub1_clear_faults(void);
+int64_t sub1_fault_epoch(void);
 int sub1_set_wait_limit_us(int64_t microseconds);
 int sub1_test_overstate_wait(int extra);
 

@@ -12,6 +12,7 @@ TRIE_ROWS = DICT_ENTRIES + 1
 MAX_WIDTH = 12288
 PREPARED_MAX_WIDTH = 12288
 STATIC_SCRATCH_BYTES = 1 << 20   # SUB1_STATIC_SCRATCH_BYTES
+STATIC_MAX_TOKENS = 512           # SUB1_STATIC_MAX_TOKENS
 
 _vp = ctypes.c_void_p
 _int = ctypes.c_int
@@ -99,6 +100,9 @@ PROTOTYPES = {
     'sub1_fault_flags': (_int, [ctypes.POINTER(ctypes.c_int32)]),
     'sub1_fault_words_host': (_vp, []),
     'sub1_clear_faults': (_int, []),
+    'sub1_fault_epoch': (_i64, []),
+    'sub1_static_scratch_reset': (_int, [_vp]),
+    'sub1_static_scratch_pointer': (_int, [ctypes.POINTER(ctypes.c_void_p)]),
     'sub1_set_wait_limit_us': (_int, [_i64]),
     'sub1_test_overstate_wait': (_int, [_int]),
     'sub1_unregister_dec': (_int, [_vp]),
@@ -165,9 +169,19 @@ def check_faults():
         raise Sub1Fault('libsub1_hip: ' + '; '.join(what) + ' [sticky: clear_faults() resets]')
 
 
-def clear_faults():
-    """Reset the fault flags.  After a wait fault the workspace of the launch
-    that raised it may hold stale counts: make the stack allocate new ones
-    (`stack._ws.clear()`), or zero the workspace again, before launching from
-    it once more."""
-    check(load().sub1_clear_faults())
+def clear_faults(stream=None):
+    """Reset the fault flags, once the work that raised them has ended.  A wait
+    fault may have left control words of its workspace at other values than
+    zero: the stacks zero their workspaces again before the next launch (they
+    compare fault_epoch(), which this call moves on), and the static scratch
+    is zeroed here, on `stream` (the legacy default stream if None)."""
+    lib = load()
+    before = lib.sub1_fault_epoch()
+    check(lib.sub1_clear_faults())
+    if lib.sub1_fault_epoch() != before:
+        check(lib.sub1_static_scratch_reset(stream))
+
+
+def fault_epoch():
+    """Wait faults cleared so far (see clear_faults)."""
+    return load().sub1_fault_epoch()

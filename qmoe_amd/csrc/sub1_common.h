@@ -102,10 +102,7 @@ constexpr int kCtrlHeader = kCtrlTagged + kTaggedTokens * kTaggedWidth * 2;   //
 // polls it, and words that share a 64-byte sector queue behind each other in
 // the L2 (16 tokens' words in one sector cost a 16-token launch 1.5-2.5 us).
 constexpr int kTokenWaited = 1 << 16;
-#ifndef SUB1_TOKEN_STRIDE
-#define SUB1_TOKEN_STRIDE 16
-#endif
-constexpr int kCtrlTokenStride = SUB1_TOKEN_STRIDE;
+constexpr int kCtrlTokenStride = 16;   // int32 words from one token's word to the next
 
 __host__ __device__ constexpr int token_word(int token) { return kCtrlHeader + token * kCtrlTokenStride; }
 

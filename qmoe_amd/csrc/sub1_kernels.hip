@@ -1,12 +1,16 @@
-// gfx950 kernels and C ABI of libsub1_hip: decode-fused matrix-vector product
-// over dictionary-coded ternary weights, the encoder, a plain decoder and the
-// grouped expert-FFN launch.  Written for 64-wide wavefronts: one LANE walks
-// one ROW of the matrix, so a wavefront advances 64 independent code streams,
-// there is no cross-lane reduction, and work per codeword is proportional to
-// the non-zero weights in it (at most three for the fixed dictionary).
+// gfx950 kernels and C ABI of libsub1_hip on the reference's packed layout:
+// the decode-fused matrix-vector product over dictionary-coded ternary
+// weights, the encoder, a plain decoder and the grouped expert-FFN launch that
+// needs no preparation.  Written for 64-wide wavefronts.  The single product
+// (matvec_wave_kernel) gives a wavefront to a row: lane j takes codeword j of
+// each run of 64, a prefix sum across the lanes places it, a butterfly adds the
+// lanes' sums.  The expert launch (moe_kernel) gives a lane to a row, so a
+// wavefront advances 64 independent code streams without cross-lane traffic.
+// Either way the work per codeword is proportional to the non-zero weights in
+// it (at most three for the fixed dictionary).
 //
 // Reference behaviour being reproduced (not its implementation):
-//   sub1_cuda_kernel.cu:129-202  Sub1MatVec       -> matvec_kernel / moe_kernel
+//   sub1_cuda_kernel.cu:129-202  Sub1MatVec       -> matvec_wave_kernel / moe_kernel
 //   sub1_cuda_kernel.cu:211-239  Sub1PreparePack  -> pack_count_kernel
 //   sub1_cuda_kernel.cu:241-250  Sub1Pack         -> pack_emit_kernel
 //   test.py:103-115              decompress       -> decode_kernel
@@ -964,6 +968,16 @@ extern "C" const int32_t *sub1_fault_words_host(void) {
   return sub1::g_fault_host;
 }
 
+// Wait faults cleared so far.  A wait that gave up may have left the control
+// words of its workspace at other values than zero (a writer that reports after
+// the waiters have given up and cleared the word), and nothing in a later
+// launch would notice: whoever owns a workspace compares this count with the
+// one it saw when it last zeroed the buffer, and zeroes it again when they
+// differ (ExpertStack.workspace and PreparedStack.workspace do).
+std::atomic<int64_t> g_fault_epoch{0};
+
+extern "C" int64_t sub1_fault_epoch(void) { return g_fault_epoch.load(); }
+
 extern "C" int sub1_clear_faults(void) {
   // a standing kFaultDec flag means a cached table is stale: drop them all, so
   // that the calls after the reset derive theirs afresh
@@ -971,6 +985,7 @@ extern "C" int sub1_clear_faults(void) {
     std::lock_guard<std::mutex> lock(g_tab_mutex);
     drop_tables_locked(nullptr, true);
   }
+  if (sub1::fault_flag_host(sub1::kFaultWait)) g_fault_epoch.fetch_add(1);
   std::lock_guard<std::mutex> lock(sub1::g_fault_mutex);
   if (sub1::g_fault_host)
     for (int i = 0; i < sub1::kFaultWords; i++)

@@ -2796,18 +2796,39 @@ extern "C" int sub1_moe_grouped_prepared_static(const sub1_moe_prepared *p,
     return fail(SUB1_ERR_SHAPE, "%s: experts %d d_model %d d_ff %d", who, p->experts, p->d_model,
                 p->d_ff);
   if (tokens < 0) return fail(SUB1_ERR_SHAPE, "%s: tokens %d", who, tokens);
-  const int64_t need = sub1_moe_workspace_bytes(tokens, p->d_ff);
-  if (need > SUB1_STATIC_SCRATCH_BYTES)
+  // The array is split for good: control words for SUB1_STATIC_MAX_TOKENS at its
+  // head, h in what follows.  Stacks of different d_ff share the array, and h of
+  // one launch must never lie on words that another, larger launch counts with.
+  const int64_t h_room = SUB1_STATIC_SCRATCH_BYTES - sub1::control_bytes(SUB1_STATIC_MAX_TOKENS);
+  const int64_t h_bytes = static_cast<int64_t>(tokens) * p->d_ff * 2;
+  if (tokens > SUB1_STATIC_MAX_TOKENS || h_bytes > h_room)
     return fail(SUB1_ERR_SHAPE,
-                "%s: %d tokens of d_ff %d need %lld bytes of scratch, the static buffer holds "
-                "%d; use sub1_moe_grouped_prepared with a workspace",
-                who, tokens, p->d_ff, static_cast<long long>(need), SUB1_STATIC_SCRATCH_BYTES);
+                "%s: %d tokens of d_ff %d need %lld bytes for h, the static buffer serves up to "
+                "%d tokens and %lld bytes of h; use sub1_moe_grouped_prepared with a workspace",
+                who, tokens, p->d_ff, static_cast<long long>(h_bytes), SUB1_STATIC_MAX_TOKENS,
+                static_cast<long long>(h_room));
   void *ws = nullptr;
   const int rc = scratch_of_current_device(&ws);
   if (rc) return rc;
   return launch_prepared(from_moe(p), token_expert, x, p->d_model, y, p->d_model, tokens, ws,
                          SUB1_STATIC_SCRATCH_BYTES, static_cast<hipStream_t>(stream), who, 0,
                          /*may_allocate=*/false);
+}
+
+extern "C" int sub1_static_scratch_pointer(void **out) {
+  if (!out) return fail(SUB1_ERR_NULL, "sub1_static_scratch_pointer: NULL argument");
+  return scratch_of_current_device(out);
+}
+
+extern "C" int sub1_static_scratch_reset(void *stream) {
+  void *ws = nullptr;
+  const int rc = scratch_of_current_device(&ws);
+  if (rc) return rc;
+  const int words = static_cast<int>(sub1::control_bytes(SUB1_STATIC_MAX_TOKENS) / 4);
+  zero_words_kernel<<<(words + 255) / 256, 256, 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<int32_t *>(ws), words);
+  HIP_TRY(hipGetLastError());
+  return SUB1_OK;
 }
 
 extern "C" int sub1_moe_prepare_codes(const sub1_moe_stack *st, const sub1_moe_prepared *p,

@@ -57,19 +57,24 @@ class Sub1Linear(nn.Module):
         self.register_buffer('ter_minmax', torch.zeros(2 * height, dtype=torch.bfloat16))
         self.register_buffer('weight', torch.zeros(0, dtype=torch.bfloat16))
 
-    # forward() on one or two tokens runs straight from the packed buffers, a
-    # wavefront per row (nothing is faster for a single product: 3.8 to 7.8 us
-    # of kernel time on the Switch shapes).  More tokens go through copies of
-    # the weights made from the codes on first use (each costs about as much
-    # memory again as w_comp and is remade when a buffer is replaced or written
-    # in place): up to `tile_tokens` - 1 tokens the prepared stream of the
-    # non-zero weights, walked per token; from `tile_tokens` tokens on the tile
-    # form that the matrix cores multiply from, the weights decoded once per 64
-    # tokens.  Set `fast` to False to run straight from the packed buffers
-    # whatever the number of tokens.  (The three add a row's terms in different
-    # orders and agree to rounding, not to the bit.)
+    # forward() goes through copies of the weights made from the codes on first
+    # use (remade when a buffer is replaced or written in place): up to
+    # `tile_tokens` - 1 tokens the prepared stream of the non-zero weights,
+    # walked per token (about 1.1 times the bytes of w_comp: 0.78 against 0.69
+    # bit per weight at 10% non-zeros), so that a token gets the same bits
+    # whatever the number of tokens it comes with, as in the reference; from
+    # `tile_tokens` tokens on the tile form that the matrix cores multiply from
+    # (2 bits per weight whatever the density, about 2.9 times w_comp; results
+    # equal to rounding, not to the bit; `tile_tokens = None` keeps long
+    # sequences on the prepared stream and the tile copy unmade).
+    # `packed_tokens = 2` sends one or two tokens straight through the packed
+    # buffers instead, a wavefront per row: nothing is faster for a single
+    # product (3.8 to 7.8 us of kernel time on the Switch shapes against 6.3 to
+    # 8.4) and nothing is copied for it, but that kernel adds a row's terms in
+    # another order, so a token's last bit then depends on the size of its batch.
+    # `fast = False` runs from the packed buffers whatever the number of tokens.
     fast = True
-    packed_tokens = 2
+    packed_tokens = 0
     tile_tokens = 64
 
     def _copy(self, kind, width):
@@ -97,7 +102,7 @@ class Sub1Linear(nn.Module):
         if x.shape[0] == 0:
             return y
         x = x.contiguous()
-        if self.fast and x.shape[0] >= self.tile_tokens:
+        if self.fast and self.tile_tokens is not None and x.shape[0] >= self.tile_tokens:
             self._copy('tiles', x.shape[1]).matvec_tokens(x, y)
         elif (self.fast and x.shape[0] > self.packed_tokens
               and x.shape[1] <= sub1_hip.PREPARED_MAX_WIDTH):

@@ -20,7 +20,14 @@ DICT_ENTRIES = _lib.DICT_ENTRIES
 PREPARED_MAX_WIDTH = _lib.PREPARED_MAX_WIDTH
 Sub1Fault = _lib.Sub1Fault
 check_faults = _lib.check_faults
-clear_faults = _lib.clear_faults
+
+
+def clear_faults():
+    """Reset the library's fault flags once the work that raised them has
+    ended (synchronise first).  The stacks zero their workspaces again before
+    their next launch, and the static scratch of the launch that does not
+    allocate is zeroed here, on the current stream."""
+    _lib.clear_faults(_stream())
 
 
 def _stream():
@@ -174,6 +181,33 @@ def sub1decode(dec, w_comp, row_off, ter_minmax, width, want_tern=True, want_w=T
     return tern, w, int(bad.item())
 
 
+def _workspace(stack, tokens):
+    """The launch's scratch memory (control words and h), one buffer per
+    stream: launches on different streams may run at once, launches on one
+    stream run in order and share theirs.  Zeroed when it is made; the
+    launches leave its control words at zero again, except that a wait which
+    gave up may not: once such a fault has been cleared (clear_faults moves
+    fault_epoch on), every buffer made before that is zeroed again at its next
+    use.  A buffer that has to grow is replaced; the old one goes back to
+    torch's allocator, which hands it out again only in the order of the stream
+    it was allocated on."""
+    need = _lib.load().sub1_moe_workspace_bytes(tokens, stack.d_ff)
+    key = _stream().value
+    epoch = _lib.fault_epoch()
+    ws = stack._ws.get(key)
+    if ws is None or ws.numel() < need:
+        with _on_device(stack.device):
+            ws = torch.zeros(need, dtype=torch.uint8, device=stack.device)
+        stack._ws[key] = ws
+        stack._seen[key] = (0, 0)
+        stack._ws_epoch[key] = epoch
+    elif stack._ws_epoch.get(key) != epoch:
+        ws.zero_()
+        stack._seen[key] = (0, 0)
+        stack._ws_epoch[key] = epoch
+    return ws
+
+
 def _fault_delta(stack, tokens):
     # words 1 and 2 of the workspace count over all launches; report what is new
     key = _stream().value
@@ -212,6 +246,7 @@ class ExpertStack:
             _need(wo_minmax, torch.bfloat16, 'wo_minmax', dev, numel=experts * 2 * d_model),
             experts, d_model, d_ff)
         self._ws = {}
+        self._ws_epoch = {}  # per workspace: fault_epoch() when it was last zeroed
         self._seen = {}      # per workspace: the fault counts launch_faults() last returned from
 
     @classmethod
@@ -236,23 +271,7 @@ class ExpertStack:
                 + 4 * self.wo_row_off.numel() + 2 * self.wi_minmax.numel()
                 + 2 * self.wo_minmax.numel())
 
-    def workspace(self, tokens):
-        """The launch's scratch memory (control words and h), one buffer per
-        stream: launches on different streams may run at once, launches on one
-        stream run in order and share theirs.  Zeroed when it is made; the
-        launches leave its control words at zero again.  A buffer that has to
-        grow is replaced; the old one goes back to torch's allocator, which
-        hands it out again only in the order of the stream it was allocated on."""
-        need = _lib.load().sub1_moe_workspace_bytes(tokens, self.d_ff)
-        key = _stream().value
-        ws = self._ws.get(key)
-        if ws is None or ws.numel() < need:
-            with _on_device(self.device):
-                # zeroed once: every launch leaves its control words at zero again
-                ws = torch.zeros(need, dtype=torch.uint8, device=self.device)
-            self._ws[key] = ws
-            self._seen[key] = (0, 0)
-        return ws
+    workspace = _workspace
 
     def forward(self, x, token_expert, y=None):
         """y[t] = wo_e(relu(wi_e(x[t]))), e = token_expert[t]; tokens with a
@@ -326,25 +345,10 @@ class PreparedStack:
             _lib.check(lib.sub1_moe_prepare_codes(ctypes.byref(stack._c), ctypes.byref(self._c),
                                                   _stream()))
         self._ws = {}
+        self._ws_epoch = {}  # per workspace: fault_epoch() when it was last zeroed
         self._seen = {}      # per workspace: the fault counts launch_faults() last returned from
 
-    def workspace(self, tokens):
-        """The launch's scratch memory (control words and h), one buffer per
-        stream: launches on different streams may run at once, launches on one
-        stream run in order and share theirs.  Zeroed when it is made; the
-        launches leave its control words at zero again.  A buffer that has to
-        grow is replaced; the old one goes back to torch's allocator, which
-        hands it out again only in the order of the stream it was allocated on."""
-        need = _lib.load().sub1_moe_workspace_bytes(tokens, self.d_ff)
-        key = _stream().value
-        ws = self._ws.get(key)
-        if ws is None or ws.numel() < need:
-            with _on_device(self.device):
-                # zeroed once: every launch leaves its control words at zero again
-                ws = torch.zeros(need, dtype=torch.uint8, device=self.device)
-            self._ws[key] = ws
-            self._seen[key] = (0, 0)
-        return ws
+    workspace = _workspace
 
     def forward(self, x, token_expert, y=None):
         dev = self.device

@@ -163,3 +163,60 @@ def test_launches_of_one_stack_on_two_streams(lib, oracle):
                          for i, e in enumerate(r)])
         for y in outs[k]:
             assert np.array_equal(bits_host(y), want)
+
+
+@pytest.mark.parametrize('static', [False, True])
+def test_control_words_left_behind_by_a_wait_fault_are_cleared(lib, oracle, static):
+    """A wait that gives up can leave a token's control word at another value
+    than zero (a workgroup that reports after the waiters have gone), which no
+    later launch would notice.  Here the host writes such a word after a forced
+    give-up; clear_faults() must make the next launch from the same stack (and
+    from the static scratch) right again."""
+    import ctypes
+    from qmoe_amd import _lib, sub1_hip
+    experts, d_model, d_ff = 3, 768, 3072
+    stack, wi, wo = small_stack(oracle, experts, d_model, d_ff, 0.9, seed=960)
+    prep = stack.prepare()
+    route = [0, 1, 2, 1, 0, 2]
+    xs = np.stack([so.synthetic_activation(d_model, 970 + i) for i in range(len(route))])
+    x, te = bf16_dev(xs), torch.tensor(route, dtype=torch.int32, device='cuda')
+    want = np.stack([oracle.expert_ffn(wi[e], wo[e], xs[i], order=2)[0] for i, e in enumerate(route)])
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def forward():
+        if not static:
+            return prep.forward(x, te)
+        y = torch.empty_like(x)
+        _lib.check(lib.sub1_moe_grouped_prepared_static(
+            ctypes.byref(prep._c), te.data_ptr(), x.data_ptr(), y.data_ptr(), len(route), stream))
+        return y
+
+    assert np.array_equal(bits_host(forward()), want)
+    assert lib.sub1_last_kernel().decode() == 'moe_prepared_shared_kernel'
+    _lib.check(lib.sub1_set_wait_limit_us(300))
+    _lib.check(lib.sub1_test_overstate_wait(1))
+    forward()
+    torch.cuda.synchronize()
+    _lib.check(lib.sub1_test_overstate_wait(0))
+    _lib.check(lib.sub1_set_wait_limit_us(250000))
+    with pytest.raises(sub1_hip.Sub1Fault):
+        sub1_hip.check_faults()
+    # what a late writer leaves behind: one report and one wait on token 1's word
+    epoch = lib.sub1_fault_epoch()
+    words = torch.tensor([0x10001], dtype=torch.int32, device='cuda')
+    at = _lib.load().sub1_moe_workspace_bytes(0, 0) + 64          # head, then 64 bytes per token
+    if static:
+        base = ctypes.c_void_p()
+        _lib.check(lib.sub1_static_scratch_pointer(ctypes.byref(base)))
+        hip = ctypes.CDLL('libamdhip64.so')
+        hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+        assert hip.hipMemcpy(base.value + at, words.data_ptr(), 4, 3) == 0     # device to device
+    else:
+        ws = prep.workspace(len(route))
+        ws[at:at + 4].copy_(words.view(torch.uint8))
+    torch.cuda.synchronize()
+    sub1_hip.clear_faults()
+    assert lib.sub1_fault_epoch() == epoch + 1
+    assert np.array_equal(bits_host(forward()), want)
+    torch.cuda.synchronize()
+    sub1_hip.check_faults()

@@ -39,6 +39,21 @@ def check_tokens(oracle, c, xs, pre, got, rows):
         assert np.linalg.norm(y - lanes) <= REL_TOL * max(np.linalg.norm(lanes), 1e-30), i
 
 
+def check_all_tokens(oracle, c, xs, pre, got):
+    """Every token of the launch against the double-precision product of the
+    decoded matrix (numpy, not the kernel's arithmetic): the same bound as in
+    check_tokens."""
+    w = so.bf16_bits_to_f32(oracle.dequant(c['t'].astype(np.uint8), c['mm'])).astype(np.float64)
+    x = so.bf16_bits_to_f32(xs).astype(np.float64)
+    exact, sum_abs = x @ w.T, np.abs(x) @ np.abs(w).T
+    y_old = so.bf16_bits_to_f32(pre).astype(np.float64)
+    y = so.bf16_bits_to_f32(got).astype(np.float64)
+    bound = (2.0 ** -8 * np.abs(exact) + 64 * 2.0 ** -24 * sum_abs
+             + 2.0 ** -8 * np.abs(y_old + exact) + 1e-30)
+    worst = np.abs(y - (y_old + exact)) - bound
+    assert np.all(worst <= 0), np.unravel_index(np.argmax(worst), worst.shape)
+
+
 @pytest.mark.parametrize('height,width,p0,tokens', [
     (3072, 768, 0.9, 568), (768, 3072, 0.9, 200), (4096, 1024, 0.88, 64), (1024, 4096, 0.88, 129),
     (6144, 2080, 0.9, 70), (2080, 6144, 0.9, 65), (2080, 6144, 0.9, 300),
@@ -59,6 +74,7 @@ def test_tiles_product(gpu, oracle, height, width, p0, tokens):
     rows = sorted(set(list(range(0, tokens, 41)) + [tokens - 1, min(63, tokens - 1),
                                                     min(64, tokens - 1)]))
     check_tokens(oracle, c, xs, pre, got, rows)
+    check_all_tokens(oracle, c, xs, pre, got)
     # the same launch again gives the same bits, and so does any split of the
     # tokens into launches (a token's result does not depend on its tile mates)
     y2 = bf16_dev(pre).clone()
@@ -137,9 +153,10 @@ def test_tiles_matrix_set_and_arguments(gpu, oracle):
 
 def test_sub1linear_takes_the_tiles_from_64_tokens_on(gpu, oracle):
     """Sub1Linear.forward on a sequence: the tile form from `tile_tokens` tokens
-    on, the prepared stream below, the packed buffers for one or two tokens; all
-    within the tolerance of the dense product, and the tile copy follows the
-    buffers like the prepared one."""
+    on, the prepared stream below (the same bits for a token whatever its
+    batch), the packed buffers for one or two tokens on request; all within the
+    tolerance of the dense product, and the tile copy follows the buffers like
+    the prepared one."""
     sub1, op = gpu
     from qmoe_amd import _lib
     t, mm = so.synthetic_ternary(320, 512, 0.85, seed=77)
@@ -153,9 +170,52 @@ def test_sub1linear_takes_the_tiles_from_64_tokens_on(gpu, oracle):
     y_few = lin(x[:10])
     assert _lib.load().sub1_last_kernel() != b'matvec_tiles_kernel'
     assert torch.linalg.norm(y_few.float() - ref[:10]) <= REL_TOL * torch.linalg.norm(ref[:10])
-    # one or two tokens: straight from the packed buffers, a wavefront per row
+    # below the tile form a token's bits do not depend on the tokens it comes with
+    for n in (1, 2, 3, 63):
+        assert torch.equal(lin(x[:n]), lin(x[:63])[:n]), n
+    # on request one or two tokens go straight from the packed buffers, a wavefront per row
+    lin.packed_tokens = 2
     y_two = lin(x[:2])
     assert _lib.load().sub1_last_kernel() == b'matvec_wave_kernel<4>'
     assert torch.linalg.norm(y_two.float() - ref[:2]) <= REL_TOL * torch.linalg.norm(ref[:2])
+    # and long sequences stay on the prepared stream, to the bit, where the tile form is switched off
+    lin.packed_tokens, lin.tile_tokens = 0, None
+    assert torch.equal(lin(x)[:63], lin(x[:63]))
+    assert not _lib.load().sub1_last_kernel().startswith(b'matvec_tiles_kernel')
+    lin.tile_tokens = 64
     lin.ter_minmax = (lin.ter_minmax.float() * 2).bfloat16()
     assert torch.equal(lin(x).float(), 2 * y.float())
+
+
+def test_tiles_multiply_zero_weights_like_the_reference(gpu, oracle):
+    """An infinite activation: the matrix cores multiply a zero weight by it
+    like any other (0 x inf = NaN, which is what reference
+    sub1_cuda_kernel.cu:190 computes too), so no row of that token stays
+    finite; the row-walking kernels leave the rows that have no weight in the
+    column as they would be with a zero there.  Other tokens are untouched."""
+    sub1, op = gpu
+    height, width, tokens, col = 128, 256, 66, 37
+    c = dev_case(oracle, height, width, 0.8, seed=8080)
+    rng = np.random.default_rng(5)
+    xs = so.f32_to_bf16_bits(rng.standard_normal((tokens, width)).astype(np.float32))
+    clean = xs.copy()
+    clean[3, col] = 0
+    xs[3, col] = 0x7f80                      # +inf
+    tm = op.TiledMatrix(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], width)
+    y_inf = torch.zeros((tokens, height), dtype=torch.bfloat16, device='cuda')
+    y_clean = torch.zeros_like(y_inf)
+    tm.matvec_tokens(bf16_dev(xs), y_inf)
+    tm.matvec_tokens(bf16_dev(clean), y_clean)
+    assert not torch.isfinite(y_inf[3].float()).any()
+    others = [i for i in range(tokens) if i != 3]
+    assert torch.equal(y_inf[others], y_clean[others])
+    pm = op.PreparedMatrix(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], width)
+    w_inf = torch.zeros_like(y_inf)
+    w_clean = torch.zeros_like(y_inf)
+    pm.matvec_tokens(bf16_dev(xs), w_inf)
+    pm.matvec_tokens(bf16_dev(clean), w_clean)
+    no_weight = torch.from_numpy(c['t'][:, col] == 0).cuda()
+    assert no_weight.any() and (~no_weight).any()
+    assert torch.equal(w_inf[3][no_weight], w_clean[3][no_weight])
+    assert not torch.isfinite(w_inf[3][~no_weight].float()).any()
+    assert torch.equal(w_inf[others], w_clean[others])
