@@ -262,6 +262,46 @@ int sub1_moe_prepare_layout(const sub1_moe_stack *stack, void *meta, int64_t met
 int sub1_moe_prepare_codes(const sub1_moe_stack *stack, const sub1_moe_prepared *prepared,
                            void *stream);
 
+/*
+ * The same preparation straight from the layers' own buffers, wherever they
+ * lie: per projection and buffer a DEVICE array [experts] of device pointers to
+ * what expert e's Sub1Linear holds (reference sub1.py:116-130: w_comp int16,
+ * row_off int32 [rows + 1] starting at 0, ter_minmax bf16 [2 * rows]; 2-, 4-
+ * and 4-byte aligned).  Nothing is stacked first: a layer is loaded into its
+ * Sub1Linear buffers as the reference does (sub1.py:284-292) and prepared from
+ * there, and the only memory a launch needs afterwards is the prepared pair.
+ * Both calls copy the six tables to the host to look at them (they synchronise
+ * the stream).  Same results as preparing the stacked copy of these buffers.
+ */
+typedef struct sub1_moe_layers {
+  const int32_t *dec;
+  const void *const *wi_w_comp;
+  const void *const *wo_w_comp;
+  const void *const *wi_row_off;
+  const void *const *wo_row_off;
+  const void *const *wi_minmax;
+  const void *const *wo_minmax;
+  int32_t experts;
+  int32_t d_model;
+  int32_t d_ff;
+} sub1_moe_layers;
+
+int sub1_moe_prepare_layout_from_layers(const sub1_moe_layers *layers, void *meta,
+                                        int64_t meta_bytes, sub1_moe_prepared *prepared,
+                                        void *stream);
+
+int sub1_moe_prepare_codes_from_layers(const sub1_moe_layers *layers,
+                                       const sub1_moe_prepared *prepared, void *stream);
+
+/*
+ * What the stream spends on padding: *walked = entries a sweep of all experts
+ * walks (64 lanes x the length of every slice), *in_rows = entries of the rows
+ * themselves (their non-zero weights and the steps over zeros that long gaps
+ * need).  Reads two small tables back from meta; synchronises the stream.
+ */
+int sub1_moe_prepared_entry_counts(const sub1_moe_prepared *prepared, int64_t *walked,
+                                   int64_t *in_rows, void *stream);
+
 int sub1_moe_grouped_prepared(const sub1_moe_prepared *prepared, const int32_t *token_expert,
                               const void *x, void *y, int tokens, void *workspace,
                               int64_t workspace_bytes, void *stream);

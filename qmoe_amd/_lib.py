@@ -27,6 +27,13 @@ class MoeStack(ctypes.Structure):
                 ('d_model', ctypes.c_int32), ('d_ff', ctypes.c_int32)]
 
 
+class MoeLayers(ctypes.Structure):
+    """struct sub1_moe_layers"""
+    _fields_ = [('dec', _vp), ('wi_w_comp', _vp), ('wo_w_comp', _vp), ('wi_row_off', _vp),
+                ('wo_row_off', _vp), ('wi_minmax', _vp), ('wo_minmax', _vp),
+                ('experts', ctypes.c_int32), ('d_model', ctypes.c_int32), ('d_ff', ctypes.c_int32)]
+
+
 class MoePrepared(ctypes.Structure):
     """struct sub1_moe_prepared"""
     _fields_ = [('meta', _vp), ('codes', _vp), ('meta_bytes', _i64), ('code_bytes', _i64),
@@ -75,6 +82,12 @@ PROTOTYPES = {
                                        ctypes.POINTER(MoePrepared), _vp]),
     'sub1_moe_prepare_codes': (_int, [ctypes.POINTER(MoeStack), ctypes.POINTER(MoePrepared),
                                       _vp]),
+    'sub1_moe_prepare_layout_from_layers': (_int, [ctypes.POINTER(MoeLayers), _vp, _i64,
+                                                   ctypes.POINTER(MoePrepared), _vp]),
+    'sub1_moe_prepare_codes_from_layers': (_int, [ctypes.POINTER(MoeLayers),
+                                                  ctypes.POINTER(MoePrepared), _vp]),
+    'sub1_moe_prepared_entry_counts': (_int, [ctypes.POINTER(MoePrepared),
+                                              ctypes.POINTER(_i64), ctypes.POINTER(_i64), _vp]),
     'sub1_moe_grouped_prepared': (_int, [ctypes.POINTER(MoePrepared), _vp, _vp, _vp, _int,
                                          _vp, _i64, _vp]),
     'sub1_moe_grouped_prepared_static': (_int, [ctypes.POINTER(MoePrepared), _vp, _vp, _vp, _int,

@@ -221,28 +221,43 @@ struct EntryWriter {
   }
 };
 
-__device__ __forceinline__ const uint16_t *row_codes(const uint16_t *src, const int64_t *code_base,
-                                                     const int32_t *row_off_all, int e, int r,
+// Where the matrices of one kind come from: one buffer of codes with a base
+// offset per matrix and [count, height + 1] / [count, height] arrays of row
+// offsets and (min, max) - an expert stack - or, with the *_of tables set, a
+// device array of device pointers per buffer, one entry per matrix - the
+// layers' own tensors, wherever they lie.
+struct KindSource {
+  const uint16_t *w_comp;
+  const int64_t *code_base;      // NULL with one matrix: its codes start at w_comp
+  const int32_t *row_off;
+  const uint32_t *minmax;
+  const uint16_t *const *w_comp_of;
+  const int32_t *const *row_off_of;
+  const uint32_t *const *minmax_of;
+};
+
+__device__ __forceinline__ const uint16_t *row_codes(const KindSource &ks, int e, int r,
                                                      int height, int width, int &n) {
-  const int32_t *ro = row_off_all + static_cast<int64_t>(e) * (height + 1);
+  const int32_t *ro = ks.row_off_of ? ks.row_off_of[e]
+                                    : ks.row_off + static_cast<int64_t>(e) * (height + 1);
   n = ro[r + 1] - ro[r];
   if (n < 1 || n > (width + 1) / 2) n = 0;   // counted as a bad row by count_entries_kernel
-  return src + (code_base ? code_base[e] : 0) + ro[r];   // one matrix: no base array
+  const uint16_t *codes = ks.w_comp_of ? ks.w_comp_of[e]
+                                       : ks.w_comp + (ks.code_base ? ks.code_base[e] : 0);
+  return codes + ro[r];
 }
 
 // One thread per row: how many entries its non-zeros take (the step onto a zero
 // column that a padded row makes after them is not counted: it fits the padding).
 __global__ __launch_bounds__(256) void count_entries_kernel(
-    const uint16_t *__restrict__ src, const int64_t *__restrict__ code_base,
-    const int32_t *__restrict__ row_off_all, const int32_t *__restrict__ dec,
-    uint16_t *__restrict__ row_len, int32_t *__restrict__ status, int height, int width,
-    int64_t rows_total) {
+    KindSource ks, const int32_t *__restrict__ dec, uint16_t *__restrict__ row_len,
+    int32_t *__restrict__ status, int height, int width, int64_t rows_total) {
   const int64_t g = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (g >= rows_total) return;
   const int e = static_cast<int>(g / height);
   const int r = static_cast<int>(g % height);
   int n;
-  const uint16_t *codes = row_codes(src, code_base, row_off_all, e, r, height, width, n);
+  const uint16_t *codes = row_codes(ks, e, r, height, width, n);
   int entries = 0;
   auto emit = [&](int, int) { entries++; };
   EntryWriter wr;
@@ -260,7 +275,7 @@ __global__ __launch_bounds__(256) void count_entries_kernel(
 // 1024 slices.
 constexpr size_t kOrderRowsLds = (kMaxRowEntries + 2 + 1024) * sizeof(int);
 __global__ __launch_bounds__(256) void order_rows_kernel(
-    const uint16_t *__restrict__ row_len_all, const uint32_t *__restrict__ minmax_all,
+    const uint16_t *__restrict__ row_len_all, KindSource ks,
     uint16_t *__restrict__ row_idx, uint32_t *__restrict__ minmax_sorted,
     uint16_t *__restrict__ slice_len, int32_t *__restrict__ counts,
     int32_t *__restrict__ status, int height, int slices, int kind) {
@@ -269,7 +284,7 @@ __global__ __launch_bounds__(256) void order_rows_kernel(
   int *first_len = order_lds + kMaxRowEntries + 2;
   const int e = blockIdx.x;
   const uint16_t *rl = row_len_all + static_cast<int64_t>(e) * height;
-  const uint32_t *mm = minmax_all + static_cast<int64_t>(e) * height;
+  const uint32_t *mm = ks.minmax_of ? ks.minmax_of[e] : ks.minmax + static_cast<int64_t>(e) * height;
   const int64_t lane0 = static_cast<int64_t>(e) * slices * 64;
   for (int i = threadIdx.x; i < kMaxRowEntries + 2; i += blockDim.x) hist[i] = 0;
   __syncthreads();
@@ -347,8 +362,7 @@ __device__ __forceinline__ int64_t checkpoint_entry(uint32_t slice_base, int64_t
 // chunk; and the row's position at the start of every group of chunks into the
 // checkpoints.
 __global__ __launch_bounds__(256) void emit_entries_kernel(
-    const uint16_t *__restrict__ src, const int64_t *__restrict__ code_base,
-    const int32_t *__restrict__ row_off_all, const int32_t *__restrict__ dec,
+    KindSource ks, const int32_t *__restrict__ dec,
     const uint32_t *__restrict__ slice_base, const uint16_t *__restrict__ slice_len,
     const uint16_t *__restrict__ row_idx, uint2 *__restrict__ dst, uint16_t *__restrict__ ckpt,
     int height, int width, int slices, int64_t first_slice, int64_t lanes_total) {
@@ -379,7 +393,7 @@ __global__ __launch_bounds__(256) void emit_entries_kernel(
   EntryWriter wr;
   if (ridx != 0xffff) {
     int n;
-    const uint16_t *codes = row_codes(src, code_base, row_off_all, e, ridx, height, width, n);
+    const uint16_t *codes = row_codes(ks, e, ridx, height, width, n);
     for_each_nonzero(codes, n, dec, width, [&](int col, int sym) { wr.nonzero(col, sym, emit); });
     if (c * kFields + q < len) wr.park(emit);   // padding follows: it must read zeros
   }
@@ -1731,9 +1745,13 @@ __device__ __forceinline__ void leave_tagged(int32_t *ctrl, int workgroups) {
 // phase and workgroup, and h crosses memory once.
 // The workgroups of a token wait for each other.  A grid (tokens x parts) of at
 // most one workgroup per compute unit runs all at once on a GPU that does
-// nothing else, and a workgroup's place in it is its index (no round trip
-// before the work starts; where other work holds compute units, the missing
-// workgroups start when that work ends, and the waits are bounded in any case).
+// nothing else, whatever order the hardware starts them in, and a workgroup's
+// place in it is its index: no round trip before the work starts, which
+// measured 1.5 to 2.0 us per launch against places by ticket (c-2048 shapes: 4
+// tokens 15.9 against 17.4 us, 16 tokens 22.5 against 24.6, 64 tokens 43.0
+// against 45.0, 128 tokens 75.9 against 77.9).  Where other work holds compute
+// units, the missing workgroups start when that work ends, and the waits are
+// bounded in any case.
 // A larger grid cannot be on the GPU at once, and there a workgroup takes its
 // place by ticket when it starts (by_ticket): the workgroups that are running
 // then hold the lowest places, the places of a token are consecutive, so at
@@ -1967,46 +1985,80 @@ int check_dec(const int32_t *dec, hipStream_t stream) {
 // What the prepare passes read: `kinds` groups of `count` matrices each.
 struct Source {
   const int32_t *dec;
-  const uint16_t *w_comp;
-  const int64_t *code_base[2];   // [count] first codeword of each matrix, NULL = 0
-  const int32_t *row_off[2];     // [count, height+1]
-  const uint32_t *minmax[2];     // [count, height]
+  KindSource k[2];
   int kinds, count;
   int height[2], width[2];
 };
 
-int check_source(const Source &src, const char *who) {
-  if (!src.dec || !src.w_comp) return fail(SUB1_ERR_NULL, "%s: NULL pointer", who);
+// Pointer tables are copied to the host once and looked at entry by entry.
+int check_pointer_table(const void *const *table, int count, size_t align, const char *what,
+                        const char *who, hipStream_t s) {
+  if (!table) return fail(SUB1_ERR_NULL, "%s: NULL table of %s pointers", who, what);
+  if (misaligned(table, 8)) return fail(SUB1_ERR_ALIGN, "%s: misaligned table of %s pointers", who, what);
+  std::vector<const void *> host(count);
+  HIP_TRY(hipMemcpyAsync(host.data(), table, sizeof(void *) * count, hipMemcpyDeviceToHost, s));
+  HIP_TRY(hipStreamSynchronize(s));
+  for (int i = 0; i < count; i++) {
+    if (!host[i]) return fail(SUB1_ERR_NULL, "%s: %s of matrix %d is NULL", who, what, i);
+    if (misaligned(host[i], align))
+      return fail(SUB1_ERR_ALIGN, "%s: %s of matrix %d is not %zu-byte aligned", who, what, i, align);
+  }
+  return SUB1_OK;
+}
+
+int check_source(const Source &src, const char *who, hipStream_t s = nullptr) {
+  if (!src.dec) return fail(SUB1_ERR_NULL, "%s: NULL pointer", who);
   if (src.count < 1) return fail(SUB1_ERR_SHAPE, "%s: %d matrices", who, src.count);
   int64_t slices = 0;
   for (int i = 0; i < src.kinds; i++) {
-    if (!src.row_off[i] || !src.minmax[i] || (src.count > 1 && !src.code_base[i]))
-      return fail(SUB1_ERR_NULL, "%s: NULL pointer", who);
+    const KindSource &k = src.k[i];
     if (src.height[i] < 1 || src.height[i] > 65534 || src.width[i] < 1 ||
         src.width[i] > SUB1_PREPARED_MAX_WIDTH)
       return fail(SUB1_ERR_SHAPE, "%s: matrix %d x %d (height 1..65534, width 1..%d)", who,
                   src.height[i], src.width[i], SUB1_PREPARED_MAX_WIDTH);
-    if (misaligned(src.row_off[i], 4) || misaligned(src.minmax[i], 4) ||
-        misaligned(src.code_base[i], 8))
-      return fail(SUB1_ERR_ALIGN, "%s: misaligned pointer", who);
+    if (k.w_comp_of || k.row_off_of || k.minmax_of) {
+      int rc = check_pointer_table(reinterpret_cast<const void *const *>(k.w_comp_of), src.count, 2,
+                                   "w_comp", who, s);
+      if (!rc)
+        rc = check_pointer_table(reinterpret_cast<const void *const *>(k.row_off_of), src.count, 4,
+                                 "row_off", who, s);
+      if (!rc)
+        rc = check_pointer_table(reinterpret_cast<const void *const *>(k.minmax_of), src.count, 4,
+                                 "ter_minmax", who, s);
+      if (rc) return rc;
+    } else {
+      if (!k.w_comp || !k.row_off || !k.minmax || (src.count > 1 && !k.code_base))
+        return fail(SUB1_ERR_NULL, "%s: NULL pointer", who);
+      if (misaligned(k.row_off, 4) || misaligned(k.minmax, 4) || misaligned(k.code_base, 8) ||
+          misaligned(k.w_comp, 2))
+        return fail(SUB1_ERR_ALIGN, "%s: misaligned pointer", who);
+    }
     slices += static_cast<int64_t>(src.count) * ((src.height[i] + 63) / 64);
   }
   if (slices > (1 << 24)) return fail(SUB1_ERR_SHAPE, "%s: too many 64-row slices", who);
-  if (misaligned(src.dec, 4) || misaligned(src.w_comp, 2))
-    return fail(SUB1_ERR_ALIGN, "%s: misaligned pointer", who);
+  if (misaligned(src.dec, 4)) return fail(SUB1_ERR_ALIGN, "%s: misaligned pointer", who);
   return SUB1_OK;
+}
+
+KindSource stacked(const void *w_comp, const int64_t *code_base, const int32_t *row_off,
+                   const void *minmax) {
+  return KindSource{static_cast<const uint16_t *>(w_comp), code_base, row_off,
+                    static_cast<const uint32_t *>(minmax), nullptr, nullptr, nullptr};
+}
+
+KindSource scattered(const void *const *w_comp, const void *const *row_off,
+                     const void *const *minmax) {
+  return KindSource{nullptr, nullptr, nullptr, nullptr,
+                    reinterpret_cast<const uint16_t *const *>(w_comp),
+                    reinterpret_cast<const int32_t *const *>(row_off),
+                    reinterpret_cast<const uint32_t *const *>(minmax)};
 }
 
 Source moe_source(const sub1_moe_stack *st) {
   Source src;
   src.dec = st->dec;
-  src.w_comp = reinterpret_cast<const uint16_t *>(st->w_comp);
-  src.code_base[0] = st->wi_code_base;
-  src.code_base[1] = st->wo_code_base;
-  src.row_off[0] = st->wi_row_off;
-  src.row_off[1] = st->wo_row_off;
-  src.minmax[0] = static_cast<const uint32_t *>(st->wi_minmax);
-  src.minmax[1] = static_cast<const uint32_t *>(st->wo_minmax);
+  src.k[0] = stacked(st->w_comp, st->wi_code_base, st->wi_row_off, st->wi_minmax);
+  src.k[1] = stacked(st->w_comp, st->wo_code_base, st->wo_row_off, st->wo_minmax);
   src.kinds = 2;
   src.count = st->experts;
   src.height[0] = st->d_ff;
@@ -2016,16 +2068,25 @@ Source moe_source(const sub1_moe_stack *st) {
   return src;
 }
 
+Source layers_source(const sub1_moe_layers *l) {
+  Source src;
+  src.dec = l->dec;
+  src.k[0] = scattered(l->wi_w_comp, l->wi_row_off, l->wi_minmax);
+  src.k[1] = scattered(l->wo_w_comp, l->wo_row_off, l->wo_minmax);
+  src.kinds = 2;
+  src.count = l->experts;
+  src.height[0] = l->d_ff;
+  src.width[0] = l->d_model;
+  src.height[1] = l->d_model;
+  src.width[1] = l->d_ff;
+  return src;
+}
+
 Source matrix_source(const sub1_matrix_set *ms) {
   Source src;
   src.dec = ms->dec;
-  src.w_comp = reinterpret_cast<const uint16_t *>(ms->w_comp);
-  src.code_base[0] = ms->code_base;
-  src.code_base[1] = nullptr;
-  src.row_off[0] = ms->row_off;
-  src.row_off[1] = nullptr;
-  src.minmax[0] = static_cast<const uint32_t *>(ms->ter_minmax);
-  src.minmax[1] = nullptr;
+  src.k[0] = stacked(ms->w_comp, ms->code_base, ms->row_off, ms->ter_minmax);
+  src.k[1] = KindSource{};
   src.kinds = 1;
   src.count = ms->count;
   src.height[0] = ms->height;
@@ -2072,10 +2133,9 @@ int prepare_layout(const Source &src, void *meta, int64_t meta_bytes, LayoutResu
     uint16_t *row_len = reinterpret_cast<uint16_t *>(base + k.row_len);
     const int64_t rows = static_cast<int64_t>(src.count) * k.height;
     count_entries_kernel<<<static_cast<unsigned>((rows + 255) / 256), 256, 0, s>>>(
-        src.w_comp, src.code_base[i], src.row_off[i], src.dec, row_len, status, k.height,
-        k.width, rows);
+        src.k[i], src.dec, row_len, status, k.height, k.width, rows);
     order_rows_kernel<<<src.count, 256, kOrderRowsLds, s>>>(
-        row_len, src.minmax[i], reinterpret_cast<uint16_t *>(base + k.row_idx),
+        row_len, src.k[i], reinterpret_cast<uint16_t *>(base + k.row_idx),
         reinterpret_cast<uint32_t *>(base + k.minmax),
         reinterpret_cast<uint16_t *>(base + k.slice_len), counts + slice0, status, k.height,
         k.slices, i);
@@ -2122,8 +2182,7 @@ int prepare_codes(const Source &src, const Prepared &p, hipStream_t s, const cha
     const int64_t kslices = static_cast<int64_t>(src.count) * k.slices;
     const int64_t lanes = kslices * 64;
     emit_entries_kernel<<<static_cast<unsigned>((lanes + 255) / 256), 256, 0, s>>>(
-        src.w_comp, src.code_base[i], src.row_off[i], src.dec,
-        reinterpret_cast<const uint32_t *>(base + k.slice_base),
+        src.k[i], src.dec, reinterpret_cast<const uint32_t *>(base + k.slice_base),
         reinterpret_cast<const uint16_t *>(base + k.slice_len),
         reinterpret_cast<const uint16_t *>(base + k.row_idx), stream, ckpt, k.height, k.width,
         k.slices, first_slice, lanes);
@@ -2665,6 +2724,28 @@ int check_moe_stack(const sub1_moe_stack *st, const char *who) {
   return check_source(moe_source(st), who);
 }
 
+int check_moe_layers(const sub1_moe_layers *l, const char *who, hipStream_t s) {
+  if (!l) return fail(SUB1_ERR_NULL, "%s: NULL layers", who);
+  if (l->experts < 1 || l->d_model < 1 || l->d_ff < 1)
+    return fail(SUB1_ERR_SHAPE, "%s: experts %d d_model %d d_ff %d", who, l->experts, l->d_model,
+                l->d_ff);
+  return check_source(layers_source(l), who, s);
+}
+
+void fill_moe_prepared(sub1_moe_prepared *out, void *meta, const LayoutResult &r, int experts,
+                       int d_model, int d_ff) {
+  out->meta = meta;
+  out->codes = nullptr;
+  out->meta_bytes = r.meta_bytes;
+  out->code_bytes = r.code_bytes;
+  out->total_chunks = r.total_chunks;
+  out->experts = experts;
+  out->d_model = d_model;
+  out->d_ff = d_ff;
+  out->max_chunks[0] = r.max_chunks[0];
+  out->max_chunks[1] = r.max_chunks[1];
+}
+
 int check_matrix_set(const sub1_matrix_set *ms, const char *who) {
   if (!ms) return fail(SUB1_ERR_NULL, "%s: NULL matrix set", who);
   return check_source(matrix_source(ms), who);
@@ -2689,16 +2770,47 @@ extern "C" int sub1_moe_prepare_layout(const sub1_moe_stack *st, void *meta, int
   rc = prepare_layout(moe_source(st), meta, meta_bytes, &r, static_cast<hipStream_t>(stream),
                       "sub1_moe_prepare_layout");
   if (rc) return rc;
-  out->meta = meta;
-  out->codes = nullptr;
-  out->meta_bytes = r.meta_bytes;
-  out->code_bytes = r.code_bytes;
-  out->total_chunks = r.total_chunks;
-  out->experts = st->experts;
-  out->d_model = st->d_model;
-  out->d_ff = st->d_ff;
-  out->max_chunks[0] = r.max_chunks[0];
-  out->max_chunks[1] = r.max_chunks[1];
+  fill_moe_prepared(out, meta, r, st->experts, st->d_model, st->d_ff);
+  return SUB1_OK;
+}
+
+extern "C" int sub1_moe_prepare_layout_from_layers(const sub1_moe_layers *layers, void *meta,
+                                                   int64_t meta_bytes, sub1_moe_prepared *out,
+                                                   void *stream) {
+  const char *who = "sub1_moe_prepare_layout_from_layers";
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int rc = check_moe_layers(layers, who, s);
+  if (rc) return rc;
+  if (!out) return fail(SUB1_ERR_NULL, "%s: NULL argument", who);
+  LayoutResult r;
+  rc = prepare_layout(layers_source(layers), meta, meta_bytes, &r, s, who);
+  if (rc) return rc;
+  fill_moe_prepared(out, meta, r, layers->experts, layers->d_model, layers->d_ff);
+  return SUB1_OK;
+}
+
+extern "C" int sub1_moe_prepared_entry_counts(const sub1_moe_prepared *p, int64_t *walked,
+                                              int64_t *in_rows, void *stream) {
+  const char *who = "sub1_moe_prepared_entry_counts";
+  if (!p || !walked || !in_rows) return fail(SUB1_ERR_NULL, "%s: NULL argument", who);
+  if (!p->meta) return fail(SUB1_ERR_NULL, "%s: NULL meta", who);
+  const MetaLayout m = moe_layout(p->experts, p->d_model, p->d_ff);
+  if (p->meta_bytes < m.bytes) return fail(SUB1_ERR_SHAPE, "%s: meta smaller than its layout", who);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const char *base = static_cast<const char *>(p->meta);
+  *walked = *in_rows = 0;
+  for (int i = 0; i < 2; i++) {
+    const KindMeta &k = m.k[i];
+    const int64_t nslices = static_cast<int64_t>(p->experts) * k.slices;
+    const int64_t nrows = static_cast<int64_t>(p->experts) * k.height;
+    std::vector<uint16_t> slice_len(nslices), row_len(nrows);
+    HIP_TRY(hipMemcpyAsync(slice_len.data(), base + k.slice_len, nslices * 2, hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipMemcpyAsync(row_len.data(), base + k.row_len, nrows * 2, hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    // the rows that pad a matrix's last slice are walked like any other lane
+    for (int64_t g = 0; g < nslices; g++) *walked += 64ll * slice_len[g];
+    for (int64_t g = 0; g < nrows; g++) *in_rows += row_len[g];
+  }
   return SUB1_OK;
 }
 
@@ -2840,6 +2952,18 @@ extern "C" int sub1_moe_prepare_codes(const sub1_moe_stack *st, const sub1_moe_p
     return fail(SUB1_ERR_SHAPE, "sub1_moe_prepare_codes: the layout belongs to another stack");
   return prepare_codes(moe_source(st), from_moe(p), static_cast<hipStream_t>(stream),
                        "sub1_moe_prepare_codes");
+}
+
+extern "C" int sub1_moe_prepare_codes_from_layers(const sub1_moe_layers *layers,
+                                                  const sub1_moe_prepared *p, void *stream) {
+  const char *who = "sub1_moe_prepare_codes_from_layers";
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int rc = check_moe_layers(layers, who, s);
+  if (rc) return rc;
+  if (!p) return fail(SUB1_ERR_NULL, "%s: NULL argument", who);
+  if (p->experts != layers->experts || p->d_model != layers->d_model || p->d_ff != layers->d_ff)
+    return fail(SUB1_ERR_SHAPE, "%s: the layout belongs to other layers", who);
+  return prepare_codes(layers_source(layers), from_moe(p), s, who);
 }
 
 extern "C" int sub1_moe_grouped_prepared(const sub1_moe_prepared *p, const int32_t *token_expert,

@@ -143,42 +143,61 @@ class Sub1Experts(nn.Module):
     def __init__(self, wi_layers, wo_layers):
         super().__init__()
         dev = wi_layers[0].w_comp.device
-        self.stack = sub1_hip.ExpertStack.from_layers(
-            DEC[dev.index],
-            [(l.w_comp, l.row_off, l.ter_minmax) for l in wi_layers],
-            [(l.w_comp, l.row_off, l.ter_minmax) for l in wo_layers])
+        self._dec = DEC[dev.index]
+        # the layers' own tensors: read when a launcher is made, never copied whole
+        self._wi = [(l.w_comp, l.row_off, l.ter_minmax) for l in wi_layers]
+        self._wo = [(l.w_comp, l.row_off, l.ter_minmax) for l in wo_layers]
+        self._d_ff = self._wi[0][1].numel() - 1
+        self._d_model = self._wo[0][1].numel() - 1
+        self._prepared = None
+        self._stack = None
 
     # forward() goes through the prepared stream of the experts' non-zero
-    # weights, made on first use (about as much memory again as the stack); set
-    # to False to run from the packed buffers.  The stack is taken as fixed: after
-    # writing to its tensors call refresh().
+    # weights, made on first use straight from the layers' tensors (about 1.1
+    # times their bytes; nothing else is allocated); set to False to run from the
+    # packed buffers, through a stacked copy of them made on first use.  The
+    # tensors are taken as fixed: after writing to them call refresh().
     fast = True
 
+    @property
+    def stack(self):
+        """The experts' packed buffers back to back (an ExpertStack, a copy made
+        on first use): what the launch that needs no preparation reads."""
+        if self._wi is None:
+            return None
+        if self._stack is None:
+            self._stack = sub1_hip.ExpertStack.from_layers(self._dec, self._wi, self._wo)
+        return self._stack
+
+    def can_prepare(self):
+        return max(self._d_model, self._d_ff) <= sub1_hip.PREPARED_MAX_WIDTH
+
     def refresh(self):
-        if self.stack is None:
-            raise RuntimeError('the packed stack was released; build the layer again')
+        if self._wi is None:
+            raise RuntimeError('the packed buffers were released; build the layer again')
         self._prepared = None
+        self._stack = None
 
     def release_packed(self):
-        """Keep only the prepared stream: makes it if need be and frees the
-        stacked copy of the packed buffers (the larger half of the layer's
-        memory; the per-expert tensors the layer was built from are the
-        caller's to drop).  What is lost is the way back: no refresh(), no run
-        from the packed buffers.  A c-2048 model's 30 layers are ~135 GB packed
-        and ~150 GB prepared: one 288 GB GPU holds one of the two."""
-        if not self.stack.can_prepare():
-            raise RuntimeError('these shapes have no prepared form; the packed stack stays')
+        """Keep only the prepared stream: makes it if need be and drops this
+        module's references to the packed tensors and any stacked copy of them
+        (the per-expert tensors the layer was built from are the caller's to
+        drop).  What is lost is the way back: no refresh(), no run from the
+        packed buffers.  A c-2048 model's 30 layers are ~135 GB packed and ~150 GB
+        prepared: one 288 GB GPU holds one of the two."""
+        if not self.can_prepare():
+            raise RuntimeError('these shapes have no prepared form; the packed buffers stay')
         self.fast = True
         self._launcher()
-        self.stack = None
+        self._wi = self._wo = self._stack = None
 
     def _launcher(self):
-        if self.stack is None:
+        if self._wi is None:
             return self._prepared
-        if not (self.fast and self.stack.can_prepare()):
+        if not (self.fast and self.can_prepare()):
             return self.stack
-        if getattr(self, '_prepared', None) is None:
-            self._prepared = self.stack.prepare()
+        if self._prepared is None:
+            self._prepared = sub1_hip.PreparedStack.from_layers(self._dec, self._wi, self._wo)
         return self._prepared
 
     def forward(self, x, expert_index):

@@ -327,23 +327,66 @@ class PreparedStack:
 
     def __init__(self, stack):
         lib = _lib.load()
-        dev = stack.device
+        self._make(stack.device, stack.experts, stack.d_model, stack.d_ff,
+                   lambda *a: lib.sub1_moe_prepare_layout(ctypes.byref(stack._c), *a),
+                   lambda *a: lib.sub1_moe_prepare_codes(ctypes.byref(stack._c), *a))
+
+    @classmethod
+    def from_layers(cls, dec, wi_layers, wo_layers):
+        """Prepared straight from per-expert (w_comp, row_off, ter_minmax)
+        triples, as the experts' Sub1Linear modules hold them: nothing is
+        stacked first, the triples are only read."""
+        lib = _lib.load()
+        dev = dec.device
+        experts = len(wi_layers)
+        if experts < 1 or len(wo_layers) != experts:
+            raise ValueError('as many wi as wo layers, at least one')
+        d_ff = wi_layers[0][1].numel() - 1
+        d_model = wo_layers[0][1].numel() - 1
+        tables = []
+        for layers, rows in ((wi_layers, d_ff), (wo_layers, d_model)):
+            columns = ([], [], [])
+            for w_comp, row_off, minmax in layers:
+                columns[0].append(_need(w_comp, torch.int16, 'w_comp', dev))
+                columns[1].append(_need(row_off, torch.int32, 'row_off', dev, numel=rows + 1))
+                columns[2].append(_need(minmax, torch.bfloat16, 'ter_minmax', dev, numel=2 * rows))
+            tables.append([torch.tensor(c, dtype=torch.int64).to(dev) for c in columns])
+        (wi_c, wi_r, wi_m), (wo_c, wo_r, wo_m) = tables
+        c_layers = _lib.MoeLayers(
+            _need(dec, torch.int32, 'dec', numel=_lib.DEC_WORDS), wi_c.data_ptr(), wo_c.data_ptr(),
+            wi_r.data_ptr(), wo_r.data_ptr(), wi_m.data_ptr(), wo_m.data_ptr(), experts, d_model, d_ff)
+        self = cls.__new__(cls)
+        self._make(dev, experts, d_model, d_ff,
+                   lambda *a: lib.sub1_moe_prepare_layout_from_layers(ctypes.byref(c_layers), *a),
+                   lambda *a: lib.sub1_moe_prepare_codes_from_layers(ctypes.byref(c_layers), *a))
+        return self
+
+    def entry_counts(self):
+        """(entries a sweep of all experts walks, entries of the rows
+        themselves): the difference is what the stream spends on padding rows
+        to the length of their slice."""
+        walked, in_rows = ctypes.c_int64(), ctypes.c_int64()
+        with _on_device(self.device):
+            _lib.check(_lib.load().sub1_moe_prepared_entry_counts(
+                ctypes.byref(self._c), ctypes.byref(walked), ctypes.byref(in_rows), _stream()))
+        return walked.value, in_rows.value
+
+    def _make(self, dev, experts, d_model, d_ff, layout, codes):
+        lib = _lib.load()
         self.device = dev
-        self.experts, self.d_model, self.d_ff = stack.experts, stack.d_model, stack.d_ff
-        meta_bytes = lib.sub1_moe_prepared_meta_bytes(stack.experts, stack.d_model, stack.d_ff)
+        self.experts, self.d_model, self.d_ff = experts, d_model, d_ff
+        meta_bytes = lib.sub1_moe_prepared_meta_bytes(experts, d_model, d_ff)
         if meta_bytes <= 0:
             raise ValueError('bad stack dimensions')
         self.meta = torch.empty(meta_bytes, dtype=torch.uint8, device=dev)
         self._c = _lib.MoePrepared()
         with _on_device(dev):
-            _lib.check(lib.sub1_moe_prepare_layout(ctypes.byref(stack._c), self.meta.data_ptr(),
-                                                   meta_bytes, ctypes.byref(self._c), _stream()))
+            _lib.check(layout(self.meta.data_ptr(), meta_bytes, ctypes.byref(self._c), _stream()))
             self.code_bytes = self._c.code_bytes
             self.stream_bytes = self._c.total_chunks * 512     # without the checkpoints
             self.codes = torch.empty(max(self.code_bytes, 256), dtype=torch.uint8, device=dev)
             self._c.codes = self.codes.data_ptr()
-            _lib.check(lib.sub1_moe_prepare_codes(ctypes.byref(stack._c), ctypes.byref(self._c),
-                                                  _stream()))
+            _lib.check(codes(ctypes.byref(self._c), _stream()))
         self._ws = {}
         self._ws_epoch = {}  # per workspace: fault_epoch() when it was last zeroed
         self._seen = {}      # per workspace: the fault counts launch_faults() last returned from

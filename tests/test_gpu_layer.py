@@ -367,3 +367,54 @@ def test_layer_launch_replays_from_a_graph(gpu):
             eager = prep.forward(x, route)   # eager work between the replays
             torch.cuda.synchronize()
             assert torch.equal(got, eager), (tokens, rep)
+
+
+def test_a_large_layer_is_prepared_without_a_second_packed_copy(gpu):
+    """256 experts of the Switch-c-2048 shapes (0.58 GB packed): building the
+    one-launch layer from the experts' own tensors and running it allocates the
+    prepared pair and little else (no stacked copy of the packed buffers on the
+    way), and with the packed tensors released the layer holds the prepared pair
+    alone.  The stream is the one that preparing a stacked copy gives."""
+    sub1 = gpu
+    from qmoe_amd import sub1_hip, synthetic
+    d_model, d_ff = synthetic.SHAPES['c2048']
+    experts = 256
+    torch.cuda.synchronize()
+    before_stack = torch.cuda.memory_allocated()      # whatever earlier tests still hold
+    stack = synthetic.build_stack(experts, d_model, d_ff, 0.9, seed=4242)
+    packed = stack.compressed_bytes()
+    triples = [synthetic.expert_layers(stack, e) for e in range(experts)]
+
+    def as_layer(t):
+        return types.SimpleNamespace(w_comp=t[0], row_off=t[1], ter_minmax=t[2])
+
+    wi_layers = [as_layer(wi) for wi, _ in triples]
+    wo_layers = [as_layer(wo) for _, wo in triples]
+    x = synthetic.activations(48, d_model, seed=5)
+    route = (torch.arange(48, dtype=torch.int32, device='cuda') * 5) % experts
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    layer = sub1.Sub1Experts(wi_layers, wo_layers)
+    y = layer(x, route)
+    torch.cuda.synchronize()
+    prep = layer._launcher()
+    assert isinstance(prep, sub1_hip.PreparedStack)
+    prepared = prep.codes.numel() + prep.meta.numel()
+    peak = torch.cuda.max_memory_allocated() - base
+    assert peak <= 1.05 * prepared, (peak, prepared, packed)
+    assert base + peak - before_stack <= 1.05 * (packed + prepared)
+    # the same stream as from the stacked copy, and the same results
+    other = stack.prepare()
+    assert prep.meta.numel() == other.meta.numel()       # (the gaps between its arrays hold anything)
+    assert torch.equal(prep.codes[:int(prep._c.total_chunks) * 512], other.codes[:int(other._c.total_chunks) * 512])
+    assert torch.equal(y, other.forward(x, route))
+    del other
+    # one resident form: the prepared pair alone
+    layer.release_packed()
+    del stack, triples, wi_layers, wo_layers
+    torch.cuda.synchronize()
+    held = torch.cuda.memory_allocated() - before_stack
+    small = x.numel() * 2 * 2 + route.numel() * 4 + sum(w.numel() for w in prep._ws.values())
+    assert held <= 1.05 * prepared + small, (held, prepared)
+    assert torch.equal(layer(x, route), y)
