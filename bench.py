@@ -254,7 +254,11 @@ def single_matrix_protocol(seed, stream_ptr):
             'dense_bf16_us': round(time_launches(matmul, 1000, 100, stream_ptr)[1], 2),
             'sync_each_packed_us': round(sync_each_us(packed), 2),
             'sync_each_dense_us': round(sync_each_us(matmul), 2),
-            'compressed_bytes': 2 * w_comp.numel(), 'dense_bytes': 2 * h * w}
+            'compressed_bytes': 2 * w_comp.numel(), 'dense_bytes': 2 * h * w,
+            # the ratio reference test.py:178 prints: 16 bits per weight against the
+            # codes plus 64 bits per row of offsets and min/max
+            'reference_compression_ratio': round(
+                16.0 * h * w / (16.0 * w_comp.numel() + 64.0 * (h + 1)), 3)}
         # a sequence through the same layer (the encoder side): 568 tokens in one
         # launch, the stream walked once per four tokens, against a dense bf16 GEMM
         xt = torch.randn((568, w), generator=g, device='cuda').bfloat16()
@@ -334,6 +338,82 @@ def faster_mlp_protocol(stack, seed, stream_ptr, tokens=64):
     return {'tokens': tokens, 'router': which, 'module_us': round(us_fast, 1),
             'router_alone_us': round(us_router, 1), 'expert_loop_us': round(us_loop, 1),
             'vs_expert_loop_rel_diff': diff}
+
+
+def density_sweep(seed, stream_ptr, experts=512):
+    """The headline sweep at other weight statistics: the Switch-c-2048 shapes,
+    `experts` experts (a stream of 1.0 to 1.9 GB, beyond every cache), a token
+    per expert, at four shares of zeros and on rows whose share of zeros
+    differs from row to row (synthetic.ROWS).  The dictionary stays the fixed
+    one (tuned for 88.5% zeros); the prepared stream costs 7.1 bits per
+    non-zero whatever the statistics, so its size follows the non-zeros while
+    the compressed bytes follow the dictionary's fit."""
+    import torch
+    from qmoe_amd import synthetic
+    d_model, d_ff = synthetic.SHAPES['c2048']
+    x = synthetic.activations(experts, d_model, seed + 1)
+    route = torch.arange(experts, dtype=torch.int32, device='cuda')
+    y = torch.empty_like(x)
+    rows = {}
+    for name, p0 in (('p0_0.80', 0.80), ('p0_0.85', 0.85), ('p0_0.88', 0.88), ('p0_0.95', 0.95),
+                     ('rows_0.75_to_0.98', synthetic.ROWS)):
+        st = synthetic.build_stack(experts, d_model, d_ff, p0, seed)
+        pr = st.prepare()
+        _, us = time_launches(lambda: pr.forward(x, route, y), 30, 5, stream_ptr)
+        walked, in_rows = pr.entry_counts()
+        cb = st.compressed_bytes()
+        rows[name] = {
+            'us_per_layer': round(us, 1), 'experts': experts,
+            'compressed_bytes': cb,
+            'bits_per_weight': round(16.0 * st.w_comp.numel() / (2.0 * experts * d_model * d_ff), 4),
+            'prepared_stream_bytes': int(pr.stream_bytes),
+            'frac_on_compressed_bytes': round(cb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            'frac_on_stream_bytes': round(pr.stream_bytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            'padding_share_of_entries': round(1.0 - in_rows / walked, 4)}
+        del st, pr
+    return rows
+
+
+def hbm_rate_by_rotation(name, seed, stream_ptr, copies=6):
+    """A layer whose compressed stack fits the 256 MB last-level cache, timed
+    from HBM all the same: `copies` different stacks of it taken in turn, so
+    that more than the cache holds passes between two uses of the same bytes."""
+    import torch
+    from qmoe_amd import synthetic
+    shp, n_e, p_z, _ = WORKLOADS[name]
+    dm, df = synthetic.SHAPES[shp]
+    stacks = [synthetic.build_stack(n_e, dm, df, p_z, seed + 100 + i) for i in range(copies)]
+    preps = [st.prepare() for st in stacks]
+    ab = sum(algorithmic_bytes(st, range(n_e)) for st in stacks) / copies
+    stream = sum(int(pr.stream_bytes) for pr in preps)
+    del stacks
+    xs = synthetic.activations(n_e, dm, seed + 11)
+    rt = torch.arange(n_e, dtype=torch.int32, device='cuda')
+    ys = torch.empty_like(xs)
+    turn = [0]
+
+    def step():
+        preps[turn[0] % copies].forward(xs, rt, ys)
+        turn[0] += 1
+
+    _, us = time_launches(step, 20 * copies, 2 * copies, stream_ptr)
+    return {'us_per_layer_from_hbm': round(us, 2), 'stacks_rotated': copies,
+            'streams_in_rotation_bytes': stream,
+            'GBps_from_hbm': round(ab / us / 1e3, 1),
+            'frac_from_hbm': round(ab / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+
+def cpu_layer_baseline(stack, x, cores):
+    """The CPU oracle on a whole small layer (a token per expert): one core on
+    a bounded sample, then `cores` threads, microseconds per layer each."""
+    experts = stack.experts
+    done1, spent1 = cpu_baseline(stack, x, min(experts, 32), 1, budget_s=2.0)
+    done, spent = cpu_baseline(stack, x, experts, cores, budget_s=3.0)
+    return {'one_core_us_per_layer': round(spent1 / done1 * experts * 1e6, 1),
+            'one_core_sample': '%d of %d expert FFNs, %.1f s' % (done1, experts, spent1),
+            'threads': cores,
+            'threads_us_per_layer': round(spent / done * experts * 1e6, 1),
+            'threads_sample': '%d of %d expert FFNs, %.1f s' % (done, experts, spent)}
 
 
 def main():
@@ -456,12 +536,24 @@ def main():
                    'prepared_bits_per_weight': round(
                        8.0 * (int(prep.code_bytes) + int(prep.meta.numel()))
                        / (2.0 * experts * d_model * d_ff), 4),
-                   'both_forms_resident': True},
+                   # this process keeps the packed stack too (the other kernels and the CPU
+                   # baseline read it); a layer needs the prepared pair alone to run
+                   # (Sub1Experts.release_packed, checkpoint.load_prepared_experts)
+                   'both_forms_resident': True,
+                   'resident_bytes': {'packed': stack.compressed_bytes(),
+                                      'prepared': int(prep.code_bytes) + int(prep.meta.numel()),
+                                      'needed_to_run': int(prep.code_bytes) + int(prep.meta.numel())}},
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS,
                      'unit': 'GB/s', 'frac': round(achieved / HBM_PEAK_GBS, 4),
                      'traffic': traffic, 'traffic_source': traffic_source,
                      'kernel': kernel,
                      'algorithmic_bytes': abytes, 'us_per_launch': round(us_launch, 2),
+                     # h (bf16 [d_ff] per token) is written by wi and read by wo in the
+                     # algorithmic count; the fused kernel keeps it in LDS and moves neither
+                     'algorithmic_bytes_excluding_h': abytes - 4 * d_ff * experts,
+                     # codes, row offsets and min/max alone: the compressed bytes proper
+                     'frac_on_compressed_bytes': round(
+                         stack.compressed_bytes() / (us_launch * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                      'fetched_bytes_by_layout': fetched,
                      'frac_on_fetched_bytes': round(
                          (traffic or fetched) / (us_launch * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)},
@@ -534,6 +626,9 @@ def main():
                      'GBps_cache_resident': round(ab / us_s / 1e3, 1)}
             if name == 'large128' and not args.no_dense:
                 entry['dense_bf16_gemv_us_per_layer'] = round(dense_gemv_us(st, xs, n_e) * n_e, 1)
+            entry.update(hbm_rate_by_rotation(name, args.seed + 40, stream_ptr))
+            if not args.no_cpu:
+                entry['cpu'] = cpu_layer_baseline(st, xs, min(16, len(os.sched_getaffinity(0))))
             if name == 'base128':
                 # a large batch: 4096 tokens routed uniformly (32 per expert on
                 # average), grouped by expert on the GPU, four tokens per walk
@@ -548,6 +643,8 @@ def main():
             del st, pr
     if not args.no_dense:
         also['single_matrix_1_token'] = single_matrix_protocol(args.seed + 30, stream_ptr)
+    if not args.experts and args.workload == 'c2048-sweep':
+        also['other_weight_statistics'] = density_sweep(args.seed + 50, stream_ptr)
     out['also'] = also
 
     if not args.no_cpu:

@@ -15,11 +15,27 @@ from . import sub1, sub1_hip
 SHAPES = {'base': (768, 3072), 'large': (1024, 4096), 'c2048': (2080, 6144)}
 
 
+ROWS = 'rows'     # p_zero: the share of zeros differs from row to row (draw_symbols)
+
+
 def draw_symbols(rows, width, p_zero, generator, device):
-    """int32 [rows, width], iid: P(0)=p_zero, P(1)=P(2)=(1-p_zero)/2."""
+    """int32 [rows, width].  p_zero a number: iid, P(0)=p_zero,
+    P(1)=P(2)=(1-p_zero)/2.  p_zero = ROWS: every row has its own share of
+    zeros, uniform in 0.75..0.98, except that one row in a hundred is all zero
+    and one in a hundred has no zero at all; within a row iid as above.  (What
+    a quantiser leaves is not iid: the fixed dictionary and the row order of the
+    prepared stream see rows of very different lengths.)"""
     u = torch.rand((rows, width), generator=generator, device=device)
-    t = (u >= p_zero).to(torch.int32)
-    t += (u >= p_zero + (1 - p_zero) / 2).to(torch.int32)
+    if p_zero == ROWS:
+        kind = torch.rand(rows, generator=generator, device=device)
+        share = 0.75 + 0.23 * torch.rand(rows, generator=generator, device=device)
+        share = torch.where(kind < 0.01, torch.ones_like(share), share)
+        share = torch.where(kind >= 0.99, torch.zeros_like(share), share)
+        p = share[:, None]
+    else:
+        p = p_zero
+    t = (u >= p).to(torch.int32)
+    t += (u >= p + (1 - p) / 2).to(torch.int32)
     return t
 
 

@@ -947,3 +947,55 @@ def test_full_size_large128_layer(gpu, oracle):
     for proj, layer, width in ((0, wi, d_model), (1, wo, d_ff)):
         tern, _, bad = op.sub1decode(sub1.DEC[0], layer[0], layer[1], layer[2], width, want_w=False)
         assert bad == 0 and torch.equal(prep.decode(41, proj), tern)
+
+
+def test_rows_of_very_different_lengths_at_c2048_shapes(gpu, oracle):
+    """Weights that are not iid: every row with its own share of zeros between
+    75% and 98%, one row in a hundred all zero and one in a hundred without a
+    zero (synthetic.ROWS), at the Switch-c-2048 shapes.  Rows from 0 to 6144
+    non-zeros share the row order and the slices of one matrix; the stream
+    must still hold every weight (decoded back against the symbols it was made
+    from) and every token must equal the oracle to the bit, in the batch sizes
+    that pick the different kernels."""
+    sub1, op = gpu
+    from qmoe_amd import synthetic
+    experts = 5
+    d_model, d_ff = synthetic.SHAPES['c2048']
+    stack, wi_sym, wo_sym = synthetic.build_stack(experts, d_model, d_ff, synthetic.ROWS, seed=31337,
+                                                  keep_symbols=True)
+    # the statistics asked for are there: empty rows, rows without a zero, and all in between
+    nz = (wo_sym[0] != 0).sum(1)
+    assert int((nz == 0).sum()) > 0 and int((nz == d_ff).sum()) > 0
+    assert int(((nz > 0.02 * d_ff) & (nz < 0.25 * d_ff)).sum()) > 0.9 * d_model
+    prep = stack.prepare()
+    for e in range(experts):
+        assert torch.equal(prep.decode(e, 0), wi_sym[e]), e
+        assert torch.equal(prep.decode(e, 1), wo_sym[e]), e
+    walked, in_rows = prep.entry_counts()
+    assert 0 < in_rows <= walked
+
+    def expert_on_host(e):
+        wi, wo = synthetic.expert_layers(stack, e)
+        return [tuple(bits_host(t) if t.dtype != torch.int32 else t.cpu().numpy() for t in l)
+                for l in (wi, wo)]
+
+    hosts = [expert_on_host(e) for e in range(experts)]
+    kernels = set()
+    for tokens in (1, 7, 300):
+        x = synthetic.activations(tokens, d_model, seed=90 + tokens)
+        route = (torch.arange(tokens, dtype=torch.int32, device='cuda') * 3 + 1) % experts
+        y = prep.forward(x, route)
+        kernels.add(_kernel_name())
+        assert prep.launch_faults(tokens) == (0, 0)
+        assert close(y, stack.forward(x, route))
+        xs, got = bits_host(x), bits_host(y)
+        for t in sorted({0, tokens // 2, tokens - 1}):
+            e = int(route[t])
+            want, _ = oracle.expert_ffn(hosts[e][0], hosts[e][1], xs[t], order=2)
+            assert np.array_equal(got[t], want), (tokens, t, e)
+    assert len(kernels) >= 2, kernels
+
+
+def _kernel_name():
+    from qmoe_amd import _lib
+    return _lib.load().sub1_last_kernel().decode()
