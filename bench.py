@@ -431,6 +431,10 @@ def main():
                     help='instead of the benchmark, run the expert layer of the workload on '
                          'this many tokens (1: one token to one expert; more: softmax router) '
                          '`--steps` times, for a profiler')
+    ap.add_argument('--reference-layout-only', action='store_true',
+                    help='instead of the benchmark, run the sweep `--steps` times through the launch '
+                         'that reads the reference\'s packed layout and decodes the dictionary in '
+                         'the kernel (no preparation), for a profiler')
     ap.add_argument('--single-matrix-only', action='store_true',
                     help='instead of the benchmark, run only the one-product-per-shape protocol')
     ap.add_argument('--seed', type=int, default=20231116)
@@ -461,6 +465,23 @@ def main():
     torch.cuda.synchronize()
     print('built %d experts in %.1f s, %.3f GB compressed' %
           (experts, time.perf_counter() - tick, stack.compressed_bytes() / 1e9), file=sys.stderr)
+
+    if args.reference_layout_only:
+        x = synthetic.activations(experts, d_model, args.seed + 1)
+        route = torch.arange(experts, dtype=torch.int32, device='cuda')
+        y = torch.empty_like(x)
+        stream_ptr = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        cal = torch.zeros(2, 1 << 28, dtype=torch.int32, device='cuda')     # the copy of known size
+        torch.add(cal[0], 1, out=cal[1])
+        torch.cuda.synchronize()
+        del cal
+        _, us = time_launches(lambda: stack.forward(x, route, y), args.steps, args.warmup, stream_ptr)
+        abytes = algorithmic_bytes(stack, range(experts))
+        print(json.dumps({'workload': desc, 'kernel': _lib.load().sub1_last_kernel().decode(),
+                          'us_per_launch': round(us, 1), 'algorithmic_bytes': abytes,
+                          'compressed_bytes': stack.compressed_bytes(),
+                          'frac': round(abytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}))
+        return
 
     tick = time.perf_counter()
     prep = stack.prepare()

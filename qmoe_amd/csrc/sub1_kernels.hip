@@ -209,7 +209,22 @@ __device__ __forceinline__ void load_codes8(const uint16_t *p, uint32_t (&w)[4])
 // partial sum per group taken left to right from zero, the partial sums added
 // first group first.  (The grouping lets the prepared kernels split a row
 // between wavefronts without changing a bit of the result.)
-__device__ __forceinline__ void row_sums(const uint32_t *__restrict__ tab,
+// The table word of a code: from the copy of the table's first `held` words in
+// LDS where the code lies in it, from the table in global memory otherwise.  A
+// gather from the 256 KB table costs a compute unit about 54 ns per wavefront
+// instruction (every lane fetches a cache line of its own through the L1), one
+// from LDS 3 ns, and the low codes are the frequent ones: the first 21 500
+// entries take 64% of the codes of weights with 90% zeros.
+struct TableView {
+  const uint32_t *tab;
+  const uint32_t *held_words;
+  uint32_t held;
+  __device__ __forceinline__ uint32_t operator[](uint32_t code) const {
+    return code < held ? held_words[code] : tab[code];
+  }
+};
+
+__device__ __forceinline__ void row_sums(const TableView tab,
                                          const uint16_t *__restrict__ codes, int len,
                                          const float *M, float &s1, float &s2) {
   s1 = 0.f;
@@ -516,6 +531,9 @@ struct MoeArgs {
   int32_t *ctrl;  // the control words (sub1_common.h): ticket, fault counts, a word per token
   int tokens, d_model, d_ff, experts;
   int wi_tiles, wo_tiles;  // per token
+  int tile_rows;           // rows of a tile: the workgroup's threads (a row each) or more (rows in turn)
+  int act_dwords;          // LDS dwords of the activations; the table's first words follow
+  int held;                // words of the table kept in LDS (0: none)
   int wi_expect;           // wi tiles a wo tile waits for (wi_tiles outside tests)
   int64_t wait_ticks;      // longest wait, in ticks of wall_clock64
   int32_t *sticky;         // fault flags in pinned host memory
@@ -532,6 +550,10 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
   const int n_wi = a.tokens * a.wi_tiles;
   const int n_all = n_wi + a.tokens * a.wo_tiles;
   if (blockIdx.x == 0) compare_print(a.dec, a.print, a.sticky);
+  // the table's first words into LDS, once per workgroup (a persistent grid)
+  uint32_t *held_words = reinterpret_cast<uint32_t *>(lds + a.act_dwords);
+  for (int i = threadIdx.x; i < a.held; i += kThreads) held_words[i] = a.tab[i];
+  const TableView table{a.tab, held_words, static_cast<uint32_t>(a.held)};
   for (;;) {
     __syncthreads();  // previous tile's readers of lds and s_ticket are done
     if (threadIdx.x == 0)
@@ -550,13 +572,13 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
         stage_activations<kThreads>(lds, a.x + static_cast<int64_t>(t) * a.d_model,
                                     a.d_model);
         __syncthreads();
-        const int row = blk * kThreads + threadIdx.x;
-        if (row < a.d_ff) {
+        const int row_end = min(a.d_ff, (blk + 1) * a.tile_rows);
+        for (int row = blk * a.tile_rows + threadIdx.x; row < row_end; row += kThreads) {
           const int32_t *ro = a.wi_row_off + static_cast<int64_t>(e) * (a.d_ff + 1);
           const int off = ro[row];
           const int len = ro[row + 1] - off;
           float s1, s2;
-          row_sums(a.tab, a.w_comp + a.wi_code_base[e] + off, len, lds + 1, s1, s2);
+          row_sums(table, a.w_comp + a.wi_code_base[e] + off, len, lds + 1, s1, s2);
           float res = row_result(
               a.wi_minmax[static_cast<int64_t>(e) * a.d_ff + row], s1, s2);
           uint16_t hb = f32_to_bf16(res);
@@ -586,9 +608,9 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
                                  __HIP_MEMORY_SCOPE_AGENT);
         e = -1;
       }
-      const int row = blk * kThreads + threadIdx.x;
+      const int row_end = min(a.d_model, (blk + 1) * a.tile_rows);
       if (e < 0) {
-        if (row < a.d_model) {
+        for (int row = blk * a.tile_rows + threadIdx.x; row < row_end; row += kThreads) {
           int64_t i = static_cast<int64_t>(t) * a.d_model + row;
           a.y[i] = a.x[i];
         }
@@ -600,12 +622,12 @@ __global__ __launch_bounds__(kThreads) void moe_kernel(MoeArgs a) {
       __syncthreads();  // thread 0's acquire now covers the whole workgroup
       stage_activations<kThreads>(lds, a.h + static_cast<int64_t>(t) * a.d_ff, a.d_ff);
       __syncthreads();
-      if (row < a.d_model) {
+      for (int row = blk * a.tile_rows + threadIdx.x; row < row_end; row += kThreads) {
         const int32_t *ro = a.wo_row_off + static_cast<int64_t>(e) * (a.d_model + 1);
         const int off = ro[row];
         const int len = ro[row + 1] - off;
         float s1, s2;
-        row_sums(a.tab, a.w_comp + a.wo_code_base[e] + off, len, lds + 1, s1, s2);
+        row_sums(table, a.w_comp + a.wo_code_base[e] + off, len, lds + 1, s1, s2);
         float res = row_result(
             a.wo_minmax[static_cast<int64_t>(e) * a.d_model + row], s1, s2);
         a.y[static_cast<int64_t>(t) * a.d_model + row] = f32_to_bf16(res);
@@ -693,6 +715,7 @@ int slot_table_for(const int32_t *dec, hipStream_t stream, TableSlot *out, int32
 
 constexpr int kMatvecThreads = 256;
 constexpr int kMoeThreads = 256;
+constexpr int kMoeSweepThreads = 1024;   // one workgroup per compute unit, the table's head in its LDS
 
 template <typename K>
 int allow_lds(K kernel, size_t bytes) {
@@ -861,29 +884,56 @@ extern "C" int sub1_moe_grouped(const sub1_moe_stack *st, const int32_t *token_e
   a.d_model = st->d_model;
   a.d_ff = st->d_ff;
   a.experts = st->experts;
-  a.wi_tiles = (st->d_ff + kMoeThreads - 1) / kMoeThreads;
-  a.wo_tiles = (st->d_model + kMoeThreads - 1) / kMoeThreads;
-  a.wi_expect = a.wi_tiles + sub1::expect_extra();
   a.wait_ticks = sub1::wait_limit_ticks();
-  int64_t tiles = static_cast<int64_t>(tokens) * (a.wi_tiles + a.wo_tiles);
-  if (tiles > INT32_MAX - (1 << 20))
-    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped: too many tiles");
-
-  int wmax = st->d_model > st->d_ff ? st->d_model : st->d_ff;
-  size_t lds = lds_dwords_for_width(wmax) * sizeof(float);
-  rc = allow_lds(moe_kernel<kMoeThreads>, lds);
-  if (rc) return rc;
   int device = 0, cus = 0, per_cu = 0;
   HIP_TRY(hipGetDevice(&device));
   HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
-  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, moe_kernel<kMoeThreads>,
-                                                       kMoeThreads, lds));
+  const int wmax = st->d_model > st->d_ff ? st->d_model : st->d_ff;
+  a.act_dwords = lds_dwords_for_width(wmax);
+  // With at least a token per compute unit the launch is a sweep, and what
+  // bounds it is the table: one workgroup of 16 wavefronts per compute unit,
+  // whole projections as tiles (a thread takes rows in turn), and all the LDS
+  // that the activations leave for the table's first words.  Fewer tokens: tiles
+  // of 256 rows, several workgroups per compute unit, the table from memory
+  // (staging it would cost every workgroup more than it saves on one tile).
+  const size_t lds_limit = 160 * 1024 - 64;
+  const bool sweep = tokens >= cus &&
+                     a.act_dwords * sizeof(float) + 16384 * sizeof(uint32_t) <= lds_limit;
+  const int threads = sweep ? kMoeSweepThreads : kMoeThreads;
+  a.tile_rows = sweep ? wmax : kMoeThreads;
+  a.held = 0;
+  if (sweep) {
+    const size_t room = (lds_limit - a.act_dwords * sizeof(float)) / sizeof(uint32_t);
+    a.held = static_cast<int>(room < SUB1_DICT_ENTRIES ? room : SUB1_DICT_ENTRIES);
+  }
+  a.wi_tiles = (st->d_ff + a.tile_rows - 1) / a.tile_rows;
+  a.wo_tiles = (st->d_model + a.tile_rows - 1) / a.tile_rows;
+  a.wi_expect = a.wi_tiles + sub1::expect_extra();
+  int64_t tiles = static_cast<int64_t>(tokens) * (a.wi_tiles + a.wo_tiles);
+  if (tiles > INT32_MAX - (1 << 20))
+    return fail(SUB1_ERR_SHAPE, "sub1_moe_grouped: too many tiles");
+  const size_t lds = (static_cast<size_t>(a.act_dwords) + a.held) * sizeof(float);
+  if (sweep) {
+    rc = allow_lds(moe_kernel<kMoeSweepThreads>, lds);
+    per_cu = 1;
+  } else {
+    rc = allow_lds(moe_kernel<kMoeThreads>, lds);
+    if (!rc)
+      HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, moe_kernel<kMoeThreads>,
+                                                           kMoeThreads, lds));
+  }
+  if (rc) return rc;
   if (per_cu < 1) return fail(SUB1_ERR_INTERNAL, "sub1_moe_grouped: kernel does not fit a CU");
   int64_t grid = static_cast<int64_t>(cus) * per_cu;
   if (grid > tiles) grid = tiles;
 
-  sub1::note_kernel("moe_kernel<256>");
-  moe_kernel<kMoeThreads><<<static_cast<unsigned>(grid), kMoeThreads, lds, s>>>(a);
+  if (sweep) {
+    sub1::note_kernel("moe_kernel<1024>");
+    moe_kernel<kMoeSweepThreads><<<static_cast<unsigned>(grid), threads, lds, s>>>(a);
+  } else {
+    sub1::note_kernel("moe_kernel<256>");
+    moe_kernel<kMoeThreads><<<static_cast<unsigned>(grid), threads, lds, s>>>(a);
+  }
   HIP_TRY(hipGetLastError());
   return SUB1_OK;
 }

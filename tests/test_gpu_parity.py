@@ -261,6 +261,40 @@ def test_grouped_launch_against_oracle(gpu, oracle, experts, d_model, d_ff, p0):
     assert torch.equal(y, y2)
 
 
+@pytest.mark.parametrize('experts,d_model,d_ff,p0', [(4, 768, 3072, 0.9), (3, 333, 77, 0.7),
+                                                     (2, 2080, 6144, 0.9)])
+def test_grouped_launch_in_its_sweep_form_against_oracle(gpu, oracle, experts, d_model, d_ff, p0):
+    """With at least a token per compute unit the packed-layout launch runs one
+    workgroup of 16 wavefronts per compute unit, whole projections as tiles (a
+    thread takes rows in turn) and the head of the table from LDS: the same
+    sums in the same order, so sampled tokens equal the oracle to the bit,
+    dropped and out-of-range tokens keep their input."""
+    from qmoe_amd import _lib
+    stack, wi, wo = small_stack(oracle, experts, d_model, d_ff, p0, seed=150)
+    tokens = 300
+    route = [(5 * i + 1) % experts for i in range(tokens)]
+    route[7], route[123], route[299] = -1, experts + 2, -1
+    xs = np.stack([so.synthetic_activation(d_model, 250 + i) for i in range(tokens)])
+    x = bf16_dev(xs)
+    te = torch.tensor(route, dtype=torch.int32, device='cuda')
+    y = stack.forward(x, te)
+    assert _lib.load().sub1_last_kernel() == b'moe_kernel<1024>'
+    got = bits_host(y)
+    assert stack.launch_faults(tokens) == (0, 1)
+    for i in (0, 1, 7, 64, 123, 150, 298, 299):
+        e = route[i]
+        if e < 0 or e >= experts:
+            assert np.array_equal(got[i], xs[i]), i
+        else:
+            want, _ = oracle.expert_ffn(wi[e], wo[e], xs[i], order=1)
+            assert np.array_equal(got[i], want), (i, e)
+    # the same tokens a few at a time go through the other form of the launch: the same bits
+    few = stack.forward(x[:9].contiguous(), te[:9].contiguous())
+    assert _lib.load().sub1_last_kernel() == b'moe_kernel<256>'
+    assert torch.equal(few, y[:9])
+    assert torch.equal(stack.forward(x, te), y)
+
+
 def test_grouped_launch_no_tokens_and_all_dropped(gpu, oracle):
     stack, _, _ = small_stack(oracle, 2, 64, 128, 0.8, seed=300)
     x = torch.zeros((0, 64), dtype=torch.bfloat16, device='cuda')
