@@ -1190,7 +1190,7 @@ __device__ __forceinline__ void publish_h(const PreparedArgs &a, int t) {
 // The wavefronts of a workgroup walk `all` slices of one matrix: slice `first`
 // of the stream's slices and every `stride`-th after it.  `before()` runs once
 // the first loads of the stream are out (it stages the activations `act` and
-// ends with a barrier); `out(row, sum)` takes every row's result.  A short last
+// ends with a barrier); `out(row, sum, slice)` takes every row's result.  A short last
 // pass (at most half the wavefronts busy) is shared out: `split` wavefronts per
 // slice, each a run of its chunk groups, partial sums in `partials`
 // (a.tail_room groups of 64 lanes).
@@ -1248,7 +1248,7 @@ __device__ __forceinline__ void walk_tile(const PreparedArgs &a, const KindArgs 
     SliceWalk nxt;
     if (s_next < count) nxt = load_slice(a, k, first + static_cast<int64_t>(s_next) * stride);
     const float res = run_slice(cur, a.stream, act, nullptr, pass, passes);
-    out(cur.ridx, res);
+    out(cur.ridx, res, first + static_cast<int64_t>(s) * stride);
     if (s_next < count) cur = nxt;
     s = s_next;
   }
@@ -1270,7 +1270,7 @@ __device__ __forceinline__ void walk_tile(const PreparedArgs &a, const KindArgs 
     if (sub == 0 && tail_sl < all) {
       float sum = 0.f;
       for (int g = 0; g < groups; g++) sum += mine[g * 64 + lane];
-      out(tail_ridx, sum);
+      out(tail_ridx, sum, tail_slice);
     }
   }
 }
@@ -1331,7 +1331,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_kernel(PreparedArgs 
       walk_tile(a, k, static_cast<int64_t>(e) * k.slices + s_lo, 1, s_hi - s_lo, xa,
                 reinterpret_cast<float *>(xa + a.xdwords),
                 [&]() { await_activations(a, k, kind, t, xa); },
-                [&](int ridx, float res) { write_row(dst, ridx, res, mode); });
+                [&](int ridx, float res, int64_t) { write_row(dst, ridx, res, mode); });
     }
     fetch_next();
     if (a.kinds == 2 && kind == 0 && e >= 0) publish_h(a, t);   // a dropped token's word stays untouched
@@ -1666,6 +1666,16 @@ __device__ __forceinline__ void write_tagged(unsigned long long *dst, int ridx, 
   __hip_atomic_store(&dst[ridx], (tag << 16) | out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// The same into a copy kept in wi's row order: `where` is the row's place in
+// that order, so that a wavefront's 64 results are 512 consecutive bytes.
+__device__ __forceinline__ void write_tagged_placed(unsigned long long *dst, int ridx, int where,
+                                                    float res, unsigned long long tag) {
+  if (ridx == 0xffff) return;   // padding lane
+  uint16_t out = f32_to_bf16(res);
+  if (out & 0x8000u) out = 0;   // relu between the projections, on the bf16 value
+  __hip_atomic_store(&dst[where], (tag << 16) | out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // The activations of wo from the tagged copy into LDS: a thread reads its
 // entries, all in flight at once, until each carries `want` (the value then
 // belongs to this launch: no count, no fence).  Bounded in time like the other
@@ -1716,6 +1726,81 @@ __device__ __forceinline__ void await_tagged(const PreparedArgs &a, const KindAr
     if (i < width) {
       uint32_t *p = xa + 2 * physical_column(i);
       const uint32_t value = static_cast<uint32_t>(v[u]) & 0xffffu;
+      p[0] = value;
+      p[1] = value << 16;
+    }
+  }
+  __syncthreads();
+}
+
+// The same from a copy kept in wi's row order (write_tagged_placed): entry p
+// belongs to row `order[p]` of h (0xffff: a padding lane, never written).  A
+// thread asks for its part of `order` first - the workgroups that call this
+// have nothing else to do until h is there - and then reads its entries, all
+// in flight at once, until each
+// carries `want` (the value then belongs to this launch: no count, no fence).
+// Bounded in time like the other waits; a thread that gives up raises the flag,
+// counts itself and stages what it has.  Ends with a barrier.  The launch runs
+// 1024 threads a workgroup.
+__device__ __forceinline__ void await_tagged_placed(const PreparedArgs &a, const KindArgs &k,
+                                             const unsigned long long *src,
+                                             const uint16_t *order, int places,
+                                             unsigned long long want, uint32_t *xa) {
+  constexpr int kMine = kTaggedWidthPerThread;   // entries a thread may have (places / 1024)
+  static_assert(kMine % 2 == 0, "rows and values are kept two to a register");
+  const int width = k.width;
+  const int step = blockDim.x;
+  // two 16-bit row indices, and later two bf16 values, to a register: the
+  // wavefronts of this workgroup hold their chunks of wo in registers meanwhile
+  uint32_t rows[kMine / 2], vals[kMine / 2];
+  uint32_t pending = 0;   // bit u: entry u is a row of h and has not been seen with the tag yet
+#pragma unroll
+  for (int u = 0; u < kMine; u++) {
+    const int i = threadIdx.x + u * step;
+    const uint32_t r = i < places ? static_cast<uint32_t>(order[i]) : 0xffffu;
+    if (u & 1) rows[u / 2] |= r << 16;
+    else rows[u / 2] = r;
+    if (r != 0xffffu) pending |= 1u << u;
+  }
+#pragma unroll
+  for (int u = 0; u < kMine / 2; u++) vals[u] = 0u;
+  for (int z = threadIdx.x * kZeroPeriod; z < physical_columns(width); z += step * kZeroPeriod) {
+    xa[2 * z] = 0u;
+    xa[2 * z + 1] = 0u;
+  }
+  int looks = 0;
+  int64_t t0 = 0;
+  while (pending) {
+#pragma unroll
+    for (int u = 0; u < kMine; u++) {
+      if (pending & (1u << u)) {
+        const unsigned long long v = __hip_atomic_load(&src[threadIdx.x + u * step], __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT);
+        if ((v >> 16) == want) {
+          pending &= ~(1u << u);
+          vals[u / 2] |= (static_cast<uint32_t>(v) & 0xffffu) << (16 * (u & 1));
+        }
+      }
+    }
+    if (!pending) break;
+    if ((++looks & 15) == 1) {
+      const int64_t now = static_cast<int64_t>(wall_clock64());
+      if (looks == 1) t0 = now;
+      if (now - t0 > a.wait_ticks) {
+        sub1::raise_fault(a.sticky, sub1::kFaultWait);
+        __hip_atomic_fetch_add(&a.ctrl[kCtrlGaveUp], 1, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
+    }
+    __builtin_amdgcn_s_sleep(1);
+  }
+#pragma unroll
+  for (int u = 0; u < kMine; u++) {
+    const uint32_t r = (rows[u / 2] >> (16 * (u & 1))) & 0xffffu;
+    if (r != 0xffffu) {
+      uint32_t *p = xa + 2 * physical_column(static_cast<int>(r));
+      const uint32_t value = (vals[u / 2] >> (16 * (u & 1))) & 0xffffu;
       p[0] = value;
       p[1] = value << 16;
     }
@@ -1796,13 +1881,13 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_shared_kernel(Prepar
               stage_finish(xa, x, ki.width, x_ahead);
               __syncthreads();
             },
-            [&](int ridx, float res) { write_row(h, ridx, res, kStoreRelu); });
+            [&](int ridx, float res, int64_t) { write_row(h, ridx, res, kStoreRelu); });
   publish_h(a, t);
   uint16_t *y = a.y + static_cast<int64_t>(t) * a.ldy;
   walk_tile(a, ko, static_cast<int64_t>(e) * ko.slices + part, parts,
             (ko.slices - part + parts - 1) / parts, xa, partials,
             [&]() { await_activations(a, ko, 1, t, xa); },
-            [&](int ridx, float res) { write_row(y, ridx, res, kStore); });
+            [&](int ridx, float res, int64_t) { write_row(y, ridx, res, kStore); });
   done_waiting(a, t);
   if (a.by_ticket && threadIdx.x == 0) sub1::leave_launch(a.ctrl, gridDim.x);
 }
@@ -1845,7 +1930,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_tagged_kernel(Prepar
               stage_finish(xa, x, ki.width, x_ahead);
               __syncthreads();
             },
-            [&](int ridx, float res) { write_tagged(ht, ridx, res, tag); });
+            [&](int ridx, float res, int64_t) { write_tagged(ht, ridx, res, tag); });
   __syncthreads();   // every wavefront is done with x before h takes its place
   uint16_t *y = a.y + static_cast<int64_t>(t) * a.ldy;
   // (a test that overstates the wait looks for a tag that nobody writes)
@@ -1853,7 +1938,77 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_tagged_kernel(Prepar
   walk_tile(a, ko, static_cast<int64_t>(e) * ko.slices + part, parts,
             (ko.slices - part + parts - 1) / parts, xa, partials,
             [&]() { await_tagged(a, ko, ht, want, xa); },
-            [&](int ridx, float res) { write_row(y, ridx, res, kStore); });
+            [&](int ridx, float res, int64_t) { write_row(y, ridx, res, kStore); });
+  if (threadIdx.x == 0) leave_tagged(a.ctrl, gridDim.x);
+}
+
+// The same for shapes whose wo rows are long (the c-2048 shapes): wo has
+// workgroups of its own.  The first k[0].parts of a token's workgroups walk wi
+// (every k[0].parts-th slice from their own) and leave; the other k[1].parts
+// belong to wo and ask for all they need of the stream - the descriptions of
+// their slices, the row indices and every chunk they will walk (a wavefront's
+// share is one group of chunks, which its ring holds) - while wi is still being
+// walked elsewhere.  Between the last row of h and the first row of y then lie
+// the hand-over and a walk whose chunks are in registers already (one token
+// through a c-2048 expert: 13.4 -> 12.7 us, a different expert every launch
+// 14.8 -> 13.3, two tokens 15.4 -> 13.9; the base and large shapes, whose wo rows are shorter, measured
+// 0.5 us slower this way and keep the kernel above).
+__global__ __launch_bounds__(kMaxThreads) void moe_prepared_tagged_split_kernel(PreparedArgs a) {
+  extern __shared__ __align__(16) uint32_t lds[];
+  uint32_t *xa = lds;
+  float *partials = reinterpret_cast<float *>(xa + a.xdwords);
+  const KindArgs &ki = a.k[0];
+  const KindArgs &ko = a.k[1];
+  const int per_token = ki.parts + ko.parts;
+  const int t = blockIdx.x / per_token;
+  const int place = blockIdx.x - t * per_token;
+  const bool for_wo = place >= ki.parts;
+  // this launch's tag (one more than the launches so far), and for wi the
+  // token's activations, are asked for before anything else is known
+  const uint16_t *x = a.x + static_cast<int64_t>(t) * a.ldx;
+  StagedPairs x_ahead;
+  if (!for_wo) x_ahead = stage_request(x, ki.width);
+  const unsigned long long tag =
+      __hip_atomic_load(reinterpret_cast<unsigned long long *>(a.ctrl + sub1::kCtrlLaunch),
+                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+  int e = __builtin_amdgcn_readfirstlane(a.token_expert[t]);
+  if (e >= a.experts) {
+    if (place == 0 && threadIdx.x == 0)
+      __hip_atomic_fetch_add(&a.ctrl[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    e = -1;
+  }
+  if (e < 0) {
+    if (place == 0) pass_through(a, ko, t, 0, ko.slices);
+    if (threadIdx.x == 0) leave_tagged(a.ctrl, gridDim.x);
+    return;
+  }
+  unsigned long long *ht = a.tagged + static_cast<int64_t>(t) * sub1::kTaggedWidth;
+  if (!for_wo) {
+    walk_tile(a, ki, static_cast<int64_t>(e) * ki.slices + place, ki.parts,
+              (ki.slices - place + ki.parts - 1) / ki.parts, xa, partials,
+              [&]() {
+                stage_finish(xa, x, ki.width, x_ahead);
+                __syncthreads();
+              },
+              [&](int ridx, float res, int64_t slice) {
+                const int where = static_cast<int>(slice - static_cast<int64_t>(e) * ki.slices) * 64 +
+                                  (threadIdx.x & 63);
+                write_tagged_placed(ht, ridx, where, res, tag);
+              });
+  } else {
+    const int part = place - ki.parts;
+    uint16_t *y = a.y + static_cast<int64_t>(t) * a.ldy;
+    // (a test that overstates the wait looks for a tag that nobody writes)
+    const unsigned long long want = a.wi_expect == ki.parts ? tag : tag + 1;
+    walk_tile(a, ko, static_cast<int64_t>(e) * ko.slices + part, ko.parts,
+              (ko.slices - part + ko.parts - 1) / ko.parts, xa, partials,
+              [&]() {
+                await_tagged_placed(a, ko, ht,
+                                    ki.row_idx + static_cast<int64_t>(e) * ki.slices * 64,
+                                    ki.slices * 64, want, xa);
+              },
+              [&](int ridx, float res, int64_t) { write_row(y, ridx, res, kStore); });
+  }
   if (threadIdx.x == 0) leave_tagged(a.ctrl, gridDim.x);
 }
 
@@ -2578,18 +2733,36 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     const void *fn = reinterpret_cast<const void *>(moe_prepared_shared_kernel);
     HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(lds_shared)));
-    // a token or two: h goes from the wi to the wo workgroups by tag (every
-    // workgroup reads all of it, eight bytes an entry: for small grids only)
-    if (tokens <= sub1::kTaggedTokens && static_cast<int64_t>(tokens) * shared_parts <= 64 &&
-        64 * waves == kMaxThreads) {
-      a.tagged = reinterpret_cast<unsigned long long *>(a.ctrl + sub1::kCtrlTagged);
-      const void *tagged_fn = reinterpret_cast<const void *>(moe_prepared_tagged_kernel);
-      HIP_TRY(hipFuncSetAttribute(tagged_fn, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  static_cast<int>(lds_shared)));
-      sub1::note_kernel("moe_prepared_tagged_kernel");
-      moe_prepared_tagged_kernel<<<tokens * shared_parts, 64 * waves, lds_shared, s>>>(a);
-      HIP_TRY(hipGetLastError());
-      return SUB1_OK;
+    // A token or two: h goes from wi to wo by tag (every workgroup of wo reads
+    // all of it, eight bytes an entry: for small grids only).  Where wo's rows
+    // are long (eight groups of chunks and more: the c-2048 shapes) wo gets
+    // workgroups of its own, as many as give every wavefront at most one group
+    // of chunks, so that all of wo's stream is in registers before h is there.
+    if (tokens <= sub1::kTaggedTokens && 64 * waves == kMaxThreads) {
+      const KindArgs &ko = a.k[1];
+      const int per_wg = std::max(1, waves / std::max(1, ko.groups_max));
+      const int wo_parts = (ko.slices + per_wg - 1) / per_wg;
+      const bool own_wo = ko.groups_max >= 8 &&
+                          static_cast<int64_t>(tokens) * (shared_parts + wo_parts) <= cus;
+      if (own_wo || static_cast<int64_t>(tokens) * shared_parts <= 64) {
+        a.tagged = reinterpret_cast<unsigned long long *>(a.ctrl + sub1::kCtrlTagged);
+        const void *tagged_fn =
+            own_wo ? reinterpret_cast<const void *>(moe_prepared_tagged_split_kernel)
+                   : reinterpret_cast<const void *>(moe_prepared_tagged_kernel);
+        HIP_TRY(hipFuncSetAttribute(tagged_fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    static_cast<int>(lds_shared)));
+        if (own_wo) {
+          a.k[1].parts = wo_parts;
+          sub1::note_kernel("moe_prepared_tagged_split_kernel");
+          moe_prepared_tagged_split_kernel<<<tokens * (shared_parts + wo_parts), 64 * waves,
+                                             lds_shared, s>>>(a);
+        } else {
+          sub1::note_kernel("moe_prepared_tagged_kernel");
+          moe_prepared_tagged_kernel<<<tokens * shared_parts, 64 * waves, lds_shared, s>>>(a);
+        }
+        HIP_TRY(hipGetLastError());
+        return SUB1_OK;
+      }
     }
     sub1::note_kernel("moe_prepared_shared_kernel");
     moe_prepared_shared_kernel<<<tokens * shared_parts, 64 * waves, lds_shared, s>>>(a);

@@ -29,14 +29,15 @@ def lib():
     _lib.clear_faults()
 
 
-@pytest.mark.parametrize('form', ['prepared', 'packed', 'tagged'])
+@pytest.mark.parametrize('form', ['prepared', 'packed', 'tagged', 'tagged_split'])
 def test_a_wait_that_gives_up_is_reported(lib, oracle, form):
     from qmoe_amd import _lib, sub1_hip
-    experts, d_model, d_ff = 3, 768, 3072
+    # (rows of wo as long as d_ff = 8192 makes them: wo gets workgroups of its own)
+    experts, d_model, d_ff = 3, 768, 8192 if form == 'tagged_split' else 3072
     stack, wi, wo = small_stack(oracle, experts, d_model, d_ff, 0.9, seed=900)
     runner = stack if form == 'packed' else stack.prepare()
     # two tokens: the launch whose workgroups wait for tagged values instead of a count
-    route = [2, 1] if form == 'tagged' else [0, 1, 2, 1, 0, 2]
+    route = [2, 1] if form.startswith('tagged') else [0, 1, 2, 1, 0, 2]
     xs = np.stack([so.synthetic_activation(d_model, 950 + i) for i in range(len(route))])
     x, te = bf16_dev(xs), torch.tensor(route, dtype=torch.int32, device='cuda')
     order = 1 if form == 'packed' else 2
@@ -46,8 +47,8 @@ def test_a_wait_that_gives_up_is_reported(lib, oracle, form):
     assert runner.launch_faults(len(route)) == (0, 0)
     sub1_hip.check_faults()
     # a kernel whose workgroups wait for each other (whole tokens per workgroup do not)
-    if form == 'tagged':
-        assert lib.sub1_last_kernel().decode() == 'moe_prepared_tagged_kernel'
+    if form.startswith('tagged'):
+        assert lib.sub1_last_kernel().decode() == 'moe_prepared_' + form + '_kernel'
     else:
         assert lib.sub1_last_kernel().decode() in ('moe_prepared_shared_kernel', 'moe_prepared_kernel',
                                                    'moe_prepared_small_kernel', 'moe_kernel<256>')
