@@ -275,6 +275,18 @@ def single_matrix_protocol(seed, stream_ptr):
         rows[name]['tiles_bytes'] = int(tm.entries.numel() + tm.meta.numel())
         rows[name]['tokens568_dense_bf16_us'] = round(
             time_launches(lambda: torch.matmul(dense, xdt, out=ydt), 100, 10, stream_ptr)[1], 2)
+        # longer sequences (two and four of those): from the length at which the
+        # tile kernel's workgroups no longer fit the chip at once, workgroups
+        # that share their activations take over
+        for tokens in (1136, 2272):
+            xl = torch.randn((tokens, w), generator=g, device='cuda').bfloat16()
+            yl = torch.zeros((tokens, h), dtype=torch.bfloat16, device='cuda')
+            ydl = torch.zeros((h, tokens), dtype=torch.bfloat16, device='cuda')
+            xdl = xl.t().contiguous()
+            rows[name]['tokens%d_tiles_us' % tokens] = round(
+                time_launches(lambda: tm.matvec_tokens(xl, yl), 100, 10, stream_ptr)[1], 2)
+            rows[name]['tokens%d_dense_bf16_us' % tokens] = round(
+                time_launches(lambda: torch.matmul(dense, xdl, out=ydl), 100, 10, stream_ptr)[1], 2)
     return rows
 
 

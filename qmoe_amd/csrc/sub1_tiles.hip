@@ -42,10 +42,17 @@
 // depends on the matrix alone, so a token's result does not depend on the
 // launch it is part of.
 //
-// Bound: building the B operands, four plain instructions per pair of weights
-// and 64 per step of four MFMAs, takes a wavefront twice as long to issue as
-// the matrix core needs for the four; with the one wavefront per SIMD that the
-// LDS leaves room for, a window takes 1.25 us where its MFMAs alone take 0.43.
+// Long sequences go through workgroups of four wavefronts that share each
+// window of activations in LDS instead (matvec_tiles_shared_kernel, below).
+//
+// Bound: a wavefront alone on its SIMD issues an MFMA of this shape every
+// 18 ns (the matrix core needs 13.4); with the four plain instructions per
+// pair of weights that build the B operands behind it, and the LDS reads of
+// the A operands, 22 to 24 ns where an operand serves 128 tokens (four
+// instructions per MFMA) and 27 to 30 ns where it serves 64 (eight), measured
+// on loops of just these instructions; the kernels here take 28 and 35 ns.
+// A second wavefront on the SIMD fills part of the gap, and then the issue of
+// the decoding instructions is what the SIMD runs out of.
 //
 // Results: each product x * w is exact in fp32 and the sums are fp32, but in
 // the matrix cores' own order; they agree with the row-walking kernels and the
@@ -54,6 +61,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstring>
+#include <type_traits>
 
 #include "sub1_common.h"
 
@@ -603,6 +611,348 @@ void matvec_tiles_kernel(TileArgs a) {
   finish_tile<kTokens / kWaves>(a, l, wave, kWaves, reinterpret_cast<float *>(tiles), acc);
 }
 
+// ---- the same alignment, y rows 4-byte aligned, an even height ---------------
+//
+// Workgroups of four wavefronts that share what they fetch.  The wavefronts
+// form kKP parts of the windows (part k takes windows k, k + kKP, ...: the sums
+// and their order are those of matvec_tiles_kernel<kKP>) times kRG groups of 64
+// rows; a workgroup owns 64 kRG rows and 32 kNB tokens.  The kRG wavefronts of
+// a part bring each window of activations into LDS together, once, and every
+// one of them multiplies its own rows with it: a window's activations cross the
+// L1 once per 64 kRG rows instead of once per 64, and with kNB = 4 a B operand
+// serves 128 tokens.  The codes go straight into registers.
+//
+// The steps of 16 columns form one pipeline across the windows: while the
+// MFMAs of a step run, the B operands of the next step are built and its A
+// operands read, also from the last step of a window to the first of the
+// next.  A part has two tiles and a wavefront two sets of code registers.
+// Before the last step of a window a wavefront waits for all it has asked for
+// (its share of the next window, asked for a window ago) and meets the others
+// at a barrier: then the next window is there whole, and everyone has read
+// the last operands of this one, so during that step the window after the
+// next is asked for into this window's tile and registers.  Nothing is counted
+// by hand: at the barrier nothing of this wavefront is on its way.  Blocks of
+// 32 tokens past the last token are neither multiplied nor stored.
+
+template <int kOff>
+__device__ __forceinline__ void lds_request_at(uint32_t at, u32x4 &v) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(v) : "v"(at), "n"(kOff) : "memory");
+}
+// The operands of kN blocks of 32 tokens (8 KB apart), requested only.
+template <int kN>
+__device__ __forceinline__ void lds_request_blocks(uint32_t at, u32x4 (&v)[kN]) {
+  lds_request_at<0>(at, v[0]);
+  if constexpr (kN > 1) lds_request_at<8192>(at, v[1]);
+  if constexpr (kN > 2) lds_request_at<16384>(at, v[2]);
+  if constexpr (kN > 3) lds_request_at<24576>(at, v[3]);
+}
+template <int kN>
+__device__ __forceinline__ void lds_arrived_blocks(u32x4 (&v)[kN]) {
+  static_assert(kN == 1 || kN == 2 || kN == 4, "one, two or four blocks");
+  if constexpr (kN == 1) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0])::"memory");
+  if constexpr (kN == 2) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1])::"memory");
+  if constexpr (kN == 4)
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3])::"memory");
+}
+
+// What a wavefront carries from one step of 16 columns to the next: the A
+// operands of kLive blocks of 32 tokens and the B operands of its two units of
+// rows.
+template <int kLive>
+struct StepOperands {
+  u32x4 xa[kLive];
+  u32x4 wv[2];
+};
+
+// The B operands of a step in the making: the eight pairs of weights of a
+// wavefront's two units go through four stages (shift, mask, selector, pick),
+// and each stage of a group of pairs is issued together, so that no
+// instruction has to wait for the one just before it.
+struct PairsInTheMaking {
+  uint32_t v[8];
+};
+template <int kStage, int kE>
+__device__ __forceinline__ void pair_stage(PairsInTheMaking &t, int p, uint32_t word0, uint32_t word1,
+                                           const uint32_t (&min_max)[2], u32x4 (&wv)[2]) {
+  const int q = 4 * kE + (p & 3);   // the pair's place in its word
+  if (kStage == 0) t.v[p] = (p >> 2 ? word1 : word0) >> (2 * q);
+  if (kStage == 1) t.v[p] &= 0x00030003u;
+  if (kStage == 2) t.v[p] = __umul24(t.v[p], 0x0202u) + 0x01000100u;
+  if (kStage == 3) wv[p >> 2][p & 3] = __builtin_amdgcn_perm(0u, min_max[p >> 2], t.v[p]);
+}
+// (keeps a stage where it was written: what it produced is not known before)
+__device__ __forceinline__ void settle(PairsInTheMaking &t, int from, int count) {
+  if (count == 8)
+    asm volatile("" : "+v"(t.v[0]), "+v"(t.v[1]), "+v"(t.v[2]), "+v"(t.v[3]), "+v"(t.v[4]), "+v"(t.v[5]),
+                 "+v"(t.v[6]), "+v"(t.v[7]));
+  else
+    asm volatile("" : "+v"(t.v[from]), "+v"(t.v[from + 1]), "+v"(t.v[from + 2]), "+v"(t.v[from + 3]));
+}
+
+// One step: 2 kLive MFMAs on `now`.  Each MFMA is followed by an equal share
+// of the work for the step after it, which the matrix core's time covers: the
+// B operands from half kE of `word0` and `word1` (the codes of the two units),
+// and whatever `extra(m)` issues.  The A operands of that step are requested
+// from `next_get` before the first MFMA and waited for after the last.  The
+// fences keep every MFMA ahead of the work that hides behind it.
+template <int kLive, int kNB, int kE, class Extra>
+__device__ __forceinline__ void tile_step(StepOperands<kLive> &now, uint32_t next_get,
+                                          uint32_t word0, uint32_t word1,
+                                          const uint32_t (&min_max)[2], f32x16 (&acc)[kNB][2],
+                                          Extra &&extra) {
+  StepOperands<kLive> next;
+  PairsInTheMaking t;
+  // (nothing that derives from the words is to be computed before this step)
+  asm volatile("" : "+v"(word0), "+v"(word1));
+  lds_request_blocks<kLive>(next_get, next.xa);
+  const bf16x8 wb0 = __builtin_bit_cast(bf16x8, now.wv[0]), wb1 = __builtin_bit_cast(bf16x8, now.wv[1]);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int m = 0; m < 2 * kLive; m++) {
+    const int i = m >> 1, j = m & 1;
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, now.xa[i]),
+                                                         j ? wb1 : wb0, acc[i][j], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (kLive == 4) {
+      // eight MFMAs: stage m % 4 of the pairs of unit m / 4
+      const int from = 4 * (m >> 2);
+#pragma unroll
+      for (int p = from; p < from + 4; p++) {
+        if ((m & 3) == 0) pair_stage<0, kE>(t, p, word0, word1, min_max, next.wv);
+        if ((m & 3) == 1) pair_stage<1, kE>(t, p, word0, word1, min_max, next.wv);
+        if ((m & 3) == 2) pair_stage<2, kE>(t, p, word0, word1, min_max, next.wv);
+        if ((m & 3) == 3) pair_stage<3, kE>(t, p, word0, word1, min_max, next.wv);
+      }
+      if ((m & 3) != 3) settle(t, from, 4);
+      else asm volatile("" : "+v"(next.wv[m >> 2]));
+    } else if constexpr (kLive == 2) {
+      // four MFMAs: stage m of all eight pairs
+#pragma unroll
+      for (int p = 0; p < 8; p++) {
+        if (m == 0) pair_stage<0, kE>(t, p, word0, word1, min_max, next.wv);
+        if (m == 1) pair_stage<1, kE>(t, p, word0, word1, min_max, next.wv);
+        if (m == 2) pair_stage<2, kE>(t, p, word0, word1, min_max, next.wv);
+        if (m == 3) pair_stage<3, kE>(t, p, word0, word1, min_max, next.wv);
+      }
+      if (m != 3) settle(t, 0, 8);
+      else asm volatile("" : "+v"(next.wv[0]), "+v"(next.wv[1]));
+    } else {
+      // two MFMAs: two stages of all eight pairs behind each
+#pragma unroll
+      for (int p = 0; p < 8; p++) {
+        if (m == 0) pair_stage<0, kE>(t, p, word0, word1, min_max, next.wv);
+        else pair_stage<2, kE>(t, p, word0, word1, min_max, next.wv);
+      }
+      settle(t, 0, 8);
+#pragma unroll
+      for (int p = 0; p < 8; p++) {
+        if (m == 0) pair_stage<1, kE>(t, p, word0, word1, min_max, next.wv);
+        else pair_stage<3, kE>(t, p, word0, word1, min_max, next.wv);
+      }
+      if (m == 0) settle(t, 0, 8);
+      else asm volatile("" : "+v"(next.wv[0]), "+v"(next.wv[1]));
+    }
+    extra(m);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  lds_arrived_blocks<kLive>(next.xa);
+  now = next;
+}
+
+template <int kRG, int kKP, int kNB>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(kNB == 2 || kRG == 4 ? 2 : 1, 4)))
+void matvec_tiles_shared_kernel(TileArgs a) {
+  static_assert(kRG * kKP == 4 && (kNB == 2 || kNB == 4), "four wavefronts");
+  constexpr int kTile = kNB * 32 * 256;        // a window of activations
+  constexpr int kLoads = 8 * kNB / kRG;        // of them this wavefront's loads
+  static_assert(kLoads % 4 == 0, "whole groups of sixteen tokens per wavefront");
+  extern __shared__ __align__(16384) unsigned char shared_tiles[];   // [part][2][kTile]
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int g = wave % kRG, k = wave / kRG;
+  const int blocks = a.units_down / 2;
+  TileLane l;
+  l.lane = threadIdx.x & 63;
+  l.half = l.lane >> 5;
+  l.block = blockIdx.x * kRG + g;
+  const bool has_rows = l.block < blocks;
+  l.t0 = blockIdx.y * (32 * kNB);
+  l.rows_here = min(32 * kNB, a.tokens - l.t0);
+  const int live = (l.rows_here + 31) / 32;
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    const int row = l.block * kRows + j * kUnitRows + (l.lane & 31);
+    l.min_max[j] = row < a.height ? a.minmax[static_cast<int64_t>(a.matrix) * a.height + row] : 0u;
+    l.unit_at[j] = static_cast<uint32_t>(j * a.windows * 1024 + l.lane * 16);
+  }
+  l.get_at = static_cast<uint32_t>((l.lane & 31) * 256 + ((l.half ^ (l.lane & 15)) << 4));
+  Fetch f = fetch_of(a, l.lane);
+#pragma unroll
+  for (int u = 0; u < 4; u++) f.at[u] += static_cast<uint32_t>(g * (kLoads / 4)) * f.step;
+  const lds_bytes part_tiles = (lds_bytes)shared_tiles + k * (2 * kTile);
+  const int last = a.windows - 1;
+  const bool ragged_edge = (a.width & (kCols - 1)) != 0;
+  if (ragged_edge) {
+    // places that no fetch writes must not hold what LDS happened to hold
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int u = 0; u < 2 * kLoads; u++)
+      *reinterpret_cast<u32x4 *>(shared_tiles + k * (2 * kTile) + ((g * 2 * kLoads + u) * 64 + l.lane) * 16) =
+          zero;
+    __syncthreads();
+  }
+
+  f32x16 acc[kNB][2];   // [32 tokens][32 rows] blocks
+#pragma unroll
+  for (int i = 0; i < kNB; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+  // Load u (0 .. kLoads - 1) of this wavefront's share of window w of the
+  // activations, into tile `buffer` of its part; and its own codes of window w.
+  auto issue_x = [&](const __amdgpu_buffer_rsrc_t &xb, int w, int buffer, int u) {
+    const bool edge = ragged_edge && w == last;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+        xb, part_tiles + buffer * kTile + g * (kLoads * 1024) + u * 1024, 16,
+        edge && f.col[u & 3] >= a.width - w * kCols ? kOutside : f.at[u & 3] + (u >> 2) * f.step,
+        w * (kCols * 2), 0, 0);
+  };
+  auto issue_codes = [&](int w, u32x4 (&codes)[2]) {
+    const __amdgpu_buffer_rsrc_t ub =
+        units_of(a, has_rows ? l.block : 0, has_rows && w < a.windows);
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+      codes[j] = __builtin_bit_cast(
+          u32x4, __builtin_amdgcn_raw_buffer_load_b128(ub, l.unit_at[j], w * 1024, 0));
+  };
+
+  // The first two windows of this part are asked for at once; from then on
+  // the window after the next is asked for during the last step of a window,
+  // into the tile and the registers that this window has just finished with.
+  const int turns = (a.windows + kKP - 1) / kKP;
+  u32x4 codes_a[2], codes_b[2];
+  {
+    const __amdgpu_buffer_rsrc_t x0 = tokens_of(a, l, k < a.windows);
+    const __amdgpu_buffer_rsrc_t x1 = tokens_of(a, l, k + kKP < a.windows);
+#pragma unroll
+    for (int u = 0; u < kLoads; u++) issue_x(x0, k, 0, u);
+    issue_codes(k, codes_a);
+#pragma unroll
+    for (int u = 0; u < kLoads; u++) issue_x(x1, k + kKP, 1, u);
+    issue_codes(k + kKP, codes_b);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  const uint32_t tile_at[2] = {
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>(part_tiles)) + l.get_at,
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>(part_tiles + kTile)) + l.get_at};
+
+  auto run = [&](auto live_c) {
+    constexpr int kLive = decltype(live_c)::value;
+    constexpr int kSlots = 2 * kLive;                          // MFMAs of a step
+    constexpr int kPerSlot = (kLoads + kSlots - 1) / kSlots;   // loads issued behind each
+    StepOperands<kLive> now;
+    lds_request_blocks<kLive>(tile_at[0], now.xa);
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) now.wv[j][q] = weight_pair(codes_a[j][0], q, l.min_max[j]);
+    lds_arrived_blocks<kLive>(now.xa);
+    auto nothing = [](int) {};
+    // one window: the tile and codes `cur`, then on to `nxt`
+    auto turn_of = [&](int turn, int cur, u32x4 (&codes_cur)[2], u32x4 (&codes_nxt)[2]) {
+      const int w = __builtin_amdgcn_readfirstlane(k + turn * kKP);
+      const int w2 = w + 2 * kKP;
+      const __amdgpu_buffer_rsrc_t x2 = tokens_of(a, l, w2 < a.windows);
+      if (has_rows && w < a.windows) {
+        const uint32_t get = tile_at[cur];
+        tile_step<kLive, kNB, 1>(now, get ^ 32u, codes_cur[0][0], codes_cur[1][0], l.min_max, acc, nothing);
+        tile_step<kLive, kNB, 0>(now, get ^ 64u, codes_cur[0][1], codes_cur[1][1], l.min_max, acc, nothing);
+        tile_step<kLive, kNB, 1>(now, get ^ 96u, codes_cur[0][1], codes_cur[1][1], l.min_max, acc, nothing);
+        tile_step<kLive, kNB, 0>(now, get ^ 128u, codes_cur[0][2], codes_cur[1][2], l.min_max, acc, nothing);
+        tile_step<kLive, kNB, 1>(now, get ^ 160u, codes_cur[0][2], codes_cur[1][2], l.min_max, acc, nothing);
+        tile_step<kLive, kNB, 0>(now, get ^ 192u, codes_cur[0][3], codes_cur[1][3], l.min_max, acc, nothing);
+        tile_step<kLive, kNB, 1>(now, get ^ 224u, codes_cur[0][3], codes_cur[1][3], l.min_max, acc, nothing);
+        // the next window is there (this wavefront's share of it, and after
+        // the barrier everyone's), and everyone has read the last of this one
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const uint32_t word0 = codes_nxt[0][0], word1 = codes_nxt[1][0];
+        tile_step<kLive, kNB, 0>(now, tile_at[cur ^ 1], word0, word1, l.min_max, acc, [&](int m) {
+#pragma unroll
+          for (int u = m * kPerSlot; u < (m + 1) * kPerSlot && u < kLoads; u++) issue_x(x2, w2, cur, u);
+          if (m == kSlots - 1) issue_codes(w2, codes_cur);
+        });
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < kLoads; u++) issue_x(x2, w2, cur, u);
+        issue_codes(w2, codes_cur);
+      }
+    };
+    for (int turn = 0; turn < turns; turn += 2) {
+      turn_of(turn, 0, codes_a, codes_b);
+      if (turn + 1 < turns) turn_of(turn + 1, 1, codes_b, codes_a);
+    }
+  };
+  if (live > kNB / 2)
+    run(std::integral_constant<int, kNB>{});
+  else
+    run(std::integral_constant<int, kNB / 2>{});
+  // nothing is on its way into LDS any more and everyone has read its last
+  // window; then the sums take the place of the activations, 32 tokens at a time
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  float *sums = reinterpret_cast<float *>(shared_tiles);   // [wavefront][32 tokens][64 rows]
+  const int pair = l.lane & 31;                            // rows 2 pair, 2 pair + 1 of the group
+  const int row = l.block * kRows + 2 * pair;
+  const __amdgpu_buffer_rsrc_t yb = buffer_over(
+      a.y + static_cast<int64_t>(l.t0) * a.ldy,
+      static_cast<uint32_t>((static_cast<int64_t>(l.rows_here - 1) * a.ldy + a.height) * 2));
+  const uint32_t y_at = has_rows && row < a.height ? static_cast<uint32_t>(row * 2) : kOutside;
+  const uint32_t y_step = static_cast<uint32_t>(a.ldy * 2);
+  constexpr int kMine = 16 / kKP;   // pairs of tokens of a block that this wavefront finishes
+#pragma unroll
+  for (int i = 0; i < kNB; i++) {
+    if (i >= live) break;
+    uint32_t before[kMine];
+#pragma unroll
+    for (int n = 0; n < kMine; n++)
+      before[n] = __builtin_amdgcn_raw_buffer_load_b32(
+          yb, y_at + (32 * i + k * (32 / kKP) + 2 * n + l.half) * y_step, 0, 0);
+    // Element (token t, row r) of an accumulator block sits in lane
+    // r + 32 * ((t / 4) % 2), register 4 * (t / 8) + t % 4.
+    float *mine = sums + wave * (32 * kRows);
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++)
+        mine[(8 * (v >> 2) + 4 * l.half + (v & 3)) * kRows + j * 32 + (l.lane & 31)] = acc[i][j][v];
+    if (kKP > 1) __syncthreads();
+#pragma unroll
+    for (int n = 0; n < kMine; n++) {
+      const int t = k * (32 / kKP) + 2 * n + l.half;
+      const float *at = sums + g * (32 * kRows) + t * kRows + 2 * pair;
+      float lo = at[0], hi = at[1];
+#pragma unroll
+      for (int part = 1; part < kKP; part++) {
+        lo += at[part * kRG * (32 * kRows)];
+        hi += at[part * kRG * (32 * kRows) + 1];
+      }
+      const uint32_t was = before[n];
+      const uint32_t now =
+          static_cast<uint32_t>(f32_to_bf16(bf16_to_f32(static_cast<uint16_t>(was & 0xffffu)) +
+                                            bf16_to_f32(f32_to_bf16(lo)))) |
+          static_cast<uint32_t>(f32_to_bf16(bf16_to_f32(static_cast<uint16_t>(was >> 16)) +
+                                            bf16_to_f32(f32_to_bf16(hi)))) << 16;
+      __builtin_amdgcn_raw_buffer_store_b32(now, yb, y_at + (32 * i + t) * y_step, 0, 0);
+    }
+    if (kKP > 1) __syncthreads();
+  }
+}
+
 // ---- any x ------------------------------------------------------------------
 //
 // The same, the activations read element by element into registers and stored
@@ -674,6 +1024,31 @@ int pick_waves(int blocks, int windows) {
     }
   }
   return best;
+}
+
+template <int kRG, int kKP, int kNB>
+int launch_shared_as(const TileArgs &a, int blocks, hipStream_t stream) {
+  constexpr int lds = kKP * 2 * kNB * 32 * 256;
+  static_assert(lds >= 4 * 32 * kRows * 4 && lds <= 160 * 1024, "tiles, then the sums of four wavefronts");
+  static bool allowed = false;   // (per process: one device kind)
+  if (!allowed) {
+    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_tiles_shared_kernel<kRG, kKP, kNB>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    allowed = true;
+  }
+  const dim3 grid((blocks + kRG - 1) / kRG, (a.tokens + 32 * kNB - 1) / (32 * kNB));
+  matvec_tiles_shared_kernel<kRG, kKP, kNB><<<grid, 256, lds, stream>>>(a);
+  HIP_TRY(hipGetLastError());
+  return SUB1_OK;
+}
+
+int launch_shared(const TileArgs &a, int parts, int token_blocks, int blocks, hipStream_t stream) {
+  sub1::note_kernel(token_blocks == 4 ? "matvec_tiles_shared_kernel<128>" : "matvec_tiles_shared_kernel<64>");
+  if (parts == 1) return token_blocks == 4 ? launch_shared_as<4, 1, 4>(a, blocks, stream)
+                                           : launch_shared_as<4, 1, 2>(a, blocks, stream);
+  if (parts == 2) return token_blocks == 4 ? launch_shared_as<2, 2, 4>(a, blocks, stream)
+                                           : launch_shared_as<2, 2, 2>(a, blocks, stream);
+  return launch_shared_as<1, 4, 2>(a, blocks, stream);
 }
 
 template <int kWaves>
@@ -816,11 +1191,28 @@ extern "C" int sub1_matvec_tiles(const sub1_tiles *t, int matrix, const void *x,
   a.windows = l.windows;
   a.matrix = matrix;
   const bool wide = !misaligned(x, 16) && ldx % 8 == 0 && t->width % 8 == 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
   if (ldx >= (1 << 24) || ldy >= (1 << 24))
     return fail(SUB1_ERR_SHAPE, "%s: token strides of 2^24 elements or more", who);
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid(l.units_down / 2, (tokens + kTokens - 1) / kTokens);
   const int waves = pick_waves(l.units_down / 2, l.windows);
+  const bool shared_ok = wide && !misaligned(y, 4) && ldy % 2 == 0 && t->height % 2 == 0 &&
+                         ldx < (1 << 22) && ldy < (1 << 22);
+  // A wavefront with tiles of its own (matvec_tiles_kernel) while all its
+  // workgroups fit the chip at once, four wavefronts per compute unit; from
+  // there on, for matrices whose windows are split two ways at most, the
+  // workgroups that share their activations (20 to 35% less time on the Switch
+  // shapes; with four parts, and below, they are no faster).  Blocks of 128
+  // tokens where blocks of 64 would make more such workgroups than the chip
+  // holds at once, three per compute unit.  The sums and their order are the
+  // same in all of these.
+  const int blocks = l.units_down / 2;
+  const int64_t tiles_of_64 = (tokens + kTokens - 1) / kTokens;
+  if (shared_ok && waves <= 2 && blocks * tiles_of_64 > 256 * (kMaxWaves / waves)) {
+    const int groups = kMaxWaves / waves;
+    const bool wide_blocks = waves == 1 && (blocks + groups - 1) / groups * tiles_of_64 > 3 * 256;
+    return launch_shared(a, waves, wide_blocks ? 4 : 2, blocks, s);
+  }
+  const dim3 grid(l.units_down / 2, (tokens + kTokens - 1) / kTokens);
   sub1::note_kernel(wide ? "matvec_tiles_kernel" : "matvec_tiles_ragged_kernel");
   if (waves == 1) launch_tiles<1>(a, wide, grid, s);
   else if (waves == 2) launch_tiles<2>(a, wide, grid, s);

@@ -94,6 +94,53 @@ def test_tiles_product(gpu, oracle, height, width, p0, tokens):
         assert torch.linalg.norm(a - b) <= REL_TOL * torch.linalg.norm(b)
 
 
+@pytest.mark.parametrize('height,width,p0,tokens,blocks_of', [
+    (3072, 768, 0.9, 700, 64),       # windows split two ways, rows in groups of 128
+    (4096, 1024, 0.88, 1100, 64),    # one part, rows in groups of 256
+    (3200, 2080, 0.9, 1500, 64),     # 50 blocks of rows (not a multiple of four), a ragged last window
+    (6272, 520, 0.9, 2100, 128)])    # blocks of 128 tokens, the last with 52
+def test_long_sequences_share_their_activations(gpu, oracle, height, width, p0, tokens, blocks_of):
+    """From the number of tokens on at which the one-wavefront workgroups no
+    longer fit the chip at once, workgroups of four wavefronts share each window
+    of activations (matvec_tiles_shared_kernel).  Every token against the
+    double-precision product; and the same bits as the same tokens in launches
+    short enough for the other kernel (same sums in the same order), which also
+    shows that a token's result does not depend on the launch."""
+    sub1, op = gpu
+    from qmoe_amd import _lib
+    c = dev_case(oracle, height, width, p0, seed=7 * height + width + tokens)
+    tm = op.TiledMatrix(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], width)
+    rng = np.random.default_rng(tokens + width)
+    xs = so.f32_to_bf16_bits(rng.standard_normal((tokens, width)).astype(np.float32))
+    pre = so.f32_to_bf16_bits(rng.standard_normal((tokens, height)).astype(np.float32))
+    xd = bf16_dev(xs)
+    y = bf16_dev(pre).clone()
+    tm.matvec_tokens(xd, y)
+    assert _lib.load().sub1_last_kernel() == b'matvec_tiles_shared_kernel<%d>' % blocks_of
+    check_all_tokens(oracle, c, xs, pre, bits_host(y))
+    check_tokens(oracle, c, xs, pre, bits_host(y), [0, tokens // 2, tokens - 1])
+    y2 = bf16_dev(pre).clone()
+    tm.matvec_tokens(xd, y2)
+    assert torch.equal(y, y2)
+    y3 = bf16_dev(pre).clone()
+    for lo in range(0, tokens, 200):
+        tm.matvec_tokens(xd[lo:lo + 200].contiguous(), y3[lo:lo + 200])
+        assert _lib.load().sub1_last_kernel() == b'matvec_tiles_kernel'
+    assert torch.equal(y, y3)
+    # rows of y and x further apart than they are long
+    xw = torch.zeros((tokens, width + 24), dtype=torch.bfloat16, device='cuda')
+    xw[:, :width] = xd
+    yw = torch.zeros((tokens, height + 6), dtype=torch.bfloat16, device='cuda')
+    yw[:, :height] = bf16_dev(pre)
+    yw[:, height:] = 7.0
+    import ctypes
+    _lib.check(_lib.load().sub1_matvec_tiles(
+        ctypes.byref(tm._c), 0, xw.data_ptr(), width + 24, yw.data_ptr(), height + 6, tokens,
+        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    assert _lib.load().sub1_last_kernel().startswith(b'matvec_tiles_shared_kernel')
+    assert torch.equal(yw[:, :height], y) and bool((yw[:, height:] == 7.0).all())
+
+
 def test_tiles_closed_forms(gpu, oracle):
     """Unit vectors pick a column exactly; zero activations leave y as it was;
     doubling the activations doubles the product exactly (y zero before)."""
@@ -165,10 +212,10 @@ def test_sub1linear_takes_the_tiles_from_64_tokens_on(gpu, oracle):
     x = torch.randn((100, 512), generator=torch.Generator().manual_seed(3)).bfloat16().cuda()
     ref = x.float() @ w.float().t()
     y = lin(x)
-    assert _lib.load().sub1_last_kernel() .startswith(b'matvec_tiles_kernel')
+    assert _lib.load().sub1_last_kernel() .startswith(b'matvec_tiles_')
     assert torch.linalg.norm(y.float() - ref) <= REL_TOL * torch.linalg.norm(ref)
     y_few = lin(x[:10])
-    assert _lib.load().sub1_last_kernel() != b'matvec_tiles_kernel'
+    assert not _lib.load().sub1_last_kernel().startswith(b'matvec_tiles_')
     assert torch.linalg.norm(y_few.float() - ref[:10]) <= REL_TOL * torch.linalg.norm(ref[:10])
     # below the tile form a token's bits do not depend on the tokens it comes with
     for n in (1, 2, 3, 63):
@@ -181,7 +228,7 @@ def test_sub1linear_takes_the_tiles_from_64_tokens_on(gpu, oracle):
     # and long sequences stay on the prepared stream, to the bit, where the tile form is switched off
     lin.packed_tokens, lin.tile_tokens = 0, None
     assert torch.equal(lin(x)[:63], lin(x[:63]))
-    assert not _lib.load().sub1_last_kernel().startswith(b'matvec_tiles_kernel')
+    assert not _lib.load().sub1_last_kernel().startswith(b'matvec_tiles_')
     lin.tile_tokens = 64
     lin.ter_minmax = (lin.ter_minmax.float() * 2).bfloat16()
     assert torch.equal(lin(x).float(), 2 * y.float())
