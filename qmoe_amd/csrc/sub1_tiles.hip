@@ -60,6 +60,8 @@
 // not to the bit.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+#include <cmath>
 #include <cstring>
 #include <type_traits>
 
@@ -638,13 +640,13 @@ template <int kOff>
 __device__ __forceinline__ void lds_request_at(uint32_t at, u32x4 &v) {
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(v) : "v"(at), "n"(kOff) : "memory");
 }
-// The operands of kN blocks of 32 tokens (8 KB apart), requested only.
-template <int kN>
+// The operands of kN blocks of 32 tokens (kStride bytes apart), requested only.
+template <int kN, int kStride = 8192>
 __device__ __forceinline__ void lds_request_blocks(uint32_t at, u32x4 (&v)[kN]) {
   lds_request_at<0>(at, v[0]);
-  if constexpr (kN > 1) lds_request_at<8192>(at, v[1]);
-  if constexpr (kN > 2) lds_request_at<16384>(at, v[2]);
-  if constexpr (kN > 3) lds_request_at<24576>(at, v[3]);
+  if constexpr (kN > 1) lds_request_at<kStride>(at, v[1]);
+  if constexpr (kN > 2) lds_request_at<2 * kStride>(at, v[2]);
+  if constexpr (kN > 3) lds_request_at<3 * kStride>(at, v[3]);
 }
 template <int kN>
 __device__ __forceinline__ void lds_arrived_blocks(u32x4 (&v)[kN]) {
@@ -695,7 +697,7 @@ __device__ __forceinline__ void settle(PairsInTheMaking &t, int from, int count)
 // and whatever `extra(m)` issues.  The A operands of that step are requested
 // from `next_get` before the first MFMA and waited for after the last.  The
 // fences keep every MFMA ahead of the work that hides behind it.
-template <int kLive, int kNB, int kE, class Extra>
+template <int kLive, int kNB, int kE, int kStride = 8192, class Extra>
 __device__ __forceinline__ void tile_step(StepOperands<kLive> &now, uint32_t next_get,
                                           uint32_t word0, uint32_t word1,
                                           const uint32_t (&min_max)[2], f32x16 (&acc)[kNB][2],
@@ -704,7 +706,7 @@ __device__ __forceinline__ void tile_step(StepOperands<kLive> &now, uint32_t nex
   PairsInTheMaking t;
   // (nothing that derives from the words is to be computed before this step)
   asm volatile("" : "+v"(word0), "+v"(word1));
-  lds_request_blocks<kLive>(next_get, next.xa);
+  lds_request_blocks<kLive, kStride>(next_get, next.xa);
   const bf16x8 wb0 = __builtin_bit_cast(bf16x8, now.wv[0]), wb1 = __builtin_bit_cast(bf16x8, now.wv[1]);
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -1003,21 +1005,42 @@ void matvec_tiles_ragged_kernel(TileArgs a) {
   finish_tile<kTokens / kWaves>(a, l, wave, kWaves, reinterpret_cast<float *>(tile), acc);
 }
 
-// Wavefronts per workgroup for a matrix of `blocks` blocks of 64 rows and
-// `windows` windows: 1, 2 or 4, whichever is estimated fastest at nine tiles of
-// tokens (568, the longest sequence of the Switch encoders): rounds of
-// workgroups over the chip, each taking 4 us plus 1.25 us per window that a
-// wavefront walks (measured on the six Switch shapes).  A wavefront has 36 KB
-// of a compute unit's 160 KB of LDS, so a unit holds four.  The choice depends
-// on the matrix alone, never on the tokens of a launch, so a token's result is
-// the same whatever launch it is part of.
+// Estimated microseconds of a launch on `tiles` blocks of 64 tokens, for a
+// matrix of `blocks` blocks of 64 rows and `windows` windows cut into n parts
+// (fitted to measurements on the six Switch shapes at 64 to 2272 tokens).
+// matvec_tiles_kernel<n>: rounds of workgroups over the chip, four wavefronts a
+// compute unit (36 KB of LDS each), each round 4 us plus 1.25 us per window that
+// a wavefront walks.
+double cost_own_tiles(int blocks, int windows, int n, int64_t tiles) {
+  const int64_t slots = 256 * (kMaxWaves / n);
+  const int64_t rounds = (blocks * tiles + slots - 1) / slots;
+  return rounds * (4.0 + 1.25 * ((windows + n - 1) / n));
+}
+// matvec_tiles_shared_kernel<4 / n, n, 2>: 1.35 us per window of a part; a
+// compute unit holds three such workgroups with one part and two with two, and
+// each one beyond the first slows the others by 0.6 of its time; more
+// workgroups than that follow as the first ones end.
+double cost_shared_tiles(int blocks, int windows, int n, int64_t tiles) {
+  const int groups = kMaxWaves / n, cap = n == 1 ? 3 : 2;
+  const int64_t workgroups = (blocks + groups - 1) / groups * tiles;
+  const int64_t per_unit = std::min<int64_t>(cap, (workgroups + 255) / 256);
+  const double fill = static_cast<double>(workgroups) / (256.0 * cap);
+  const double rounds = fill <= 1.0 ? 1.0 : 0.5 * (std::ceil(fill) + fill);
+  return rounds * (4.0 + 1.35 * ((windows + n - 1) / n) * (1.0 + 0.6 * (per_unit - 1)));
+}
+
+// Parts that the windows of a matrix are cut into: 1, 2 or 4, whichever is
+// estimated fastest at nine blocks of tokens (568, the longest sequence of the
+// Switch encoders) by the better of the two kernels.  The choice depends on
+// the matrix alone, never on the tokens of a launch, and the parts are added in
+// the same order by both kernels: a token's result is the same whatever launch
+// it is part of.
 int pick_waves(int blocks, int windows) {
   int best = 1;
   double best_cost = 0;
   for (int n = 1; n <= kMaxWaves; n *= 2) {
-    const int64_t slots = 256 * (4 / n);
-    const int64_t rounds = (9ll * blocks + slots - 1) / slots;
-    const double cost = rounds * (4.0 + 1.25 * ((windows + n - 1) / n));
+    double cost = cost_own_tiles(blocks, windows, n, 9);
+    if (n <= 2) cost = std::min(cost, cost_shared_tiles(blocks, windows, n, 9));
     if (n == 1 || cost < best_cost - 1e-9) {
       best = n;
       best_cost = cost;
@@ -1197,17 +1220,17 @@ extern "C" int sub1_matvec_tiles(const sub1_tiles *t, int matrix, const void *x,
   const int waves = pick_waves(l.units_down / 2, l.windows);
   const bool shared_ok = wide && !misaligned(y, 4) && ldy % 2 == 0 && t->height % 2 == 0 &&
                          ldx < (1 << 22) && ldy < (1 << 22);
-  // A wavefront with tiles of its own (matvec_tiles_kernel) while all its
-  // workgroups fit the chip at once, four wavefronts per compute unit; from
-  // there on, for matrices whose windows are split two ways at most, the
-  // workgroups that share their activations (20 to 35% less time on the Switch
-  // shapes; with four parts, and below, they are no faster).  Blocks of 128
-  // tokens where blocks of 64 would make more such workgroups than the chip
-  // holds at once, three per compute unit.  The sums and their order are the
-  // same in all of these.
+  // Which kernel: the one estimated faster for this many tokens (the sums and
+  // their order are the same).  Workgroups that share their activations take
+  // over where those of one wavefront's own tiles no longer fit the chip at
+  // once (20 to 35% less time on the Switch shapes from there on); with four
+  // parts they are no faster and are not used.  Blocks of 128 tokens where
+  // blocks of 64 would make more such workgroups than the chip holds at once.
   const int blocks = l.units_down / 2;
   const int64_t tiles_of_64 = (tokens + kTokens - 1) / kTokens;
-  if (shared_ok && waves <= 2 && blocks * tiles_of_64 > 256 * (kMaxWaves / waves)) {
+  if (shared_ok && waves <= 2 &&
+      cost_shared_tiles(blocks, l.windows, waves, tiles_of_64) <
+          cost_own_tiles(blocks, l.windows, waves, tiles_of_64)) {
     const int groups = kMaxWaves / waves;
     const bool wide_blocks = waves == 1 && (blocks + groups - 1) / groups * tiles_of_64 > 3 * 256;
     return launch_shared(a, waves, wide_blocks ? 4 : 2, blocks, s);
