@@ -1950,8 +1950,8 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_tagged_kernel(Prepar
 // share is one group of chunks, which its ring holds) - while wi is still being
 // walked elsewhere.  Between the last row of h and the first row of y then lie
 // the hand-over and a walk whose chunks are in registers already (one token
-// through a c-2048 expert: 13.4 -> 12.7 us, a different expert every launch
-// 14.8 -> 13.3, two tokens 15.4 -> 13.9; the base and large shapes, whose wo rows are shorter, measured
+// through a c-2048 expert: 13.4 -> 12.4 us, a different expert every launch
+// 14.8 -> 12.9, two tokens 15.4 -> 12.8; the base and large shapes, whose wo rows are shorter, measured
 // 0.5 us slower this way and keep the kernel above).
 __global__ __launch_bounds__(kMaxThreads) void moe_prepared_tagged_split_kernel(PreparedArgs a) {
   extern __shared__ __align__(16) uint32_t lds[];
@@ -2753,6 +2753,15 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
                                     static_cast<int>(lds_shared)));
         if (own_wo) {
           a.k[1].parts = wo_parts;
+          // wi's workgroups wait for nobody, so the more of them the shorter their
+          // walks: up to a slice each, within two thirds of the compute units
+          // that wo leaves a token (one token through a c-2048 expert: 96 instead
+          // of 48 workgroups 12.7 -> 12.4 us; two tokens, 63 each instead of 24:
+          // 13.8 -> 12.8; with all units taken two tokens measured 13.4)
+          shared_parts = std::max(shared_parts,
+                                  std::min(a.k[0].slices, (cus / tokens - wo_parts) * 2 / 3));
+          a.k[0].parts = shared_parts;
+          a.wi_expect = a.k[0].parts + sub1::expect_extra();
           sub1::note_kernel("moe_prepared_tagged_split_kernel");
           moe_prepared_tagged_split_kernel<<<tokens * (shared_parts + wo_parts), 64 * waves,
                                              lds_shared, s>>>(a);

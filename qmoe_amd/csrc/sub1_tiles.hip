@@ -437,7 +437,9 @@ __device__ __forceinline__ void finish_tile(const TileArgs &a, const TileLane &l
 // in statements that take the read registers as operands, so nothing uses them
 // earlier.
 
-constexpr int kLoadsPerWindow = 18;   // 16 of activations, 2 of codes
+constexpr int kActivationLoads = 16;   // of a window: four tokens each
+constexpr int kCodeLoads = 2;          // one per unit of 32 rows
+constexpr int kLoadsPerWindow = kActivationLoads + kCodeLoads;   // what fetch_window issues, every time
 constexpr int kTileBytes = 16384;     // a tile of activations
 constexpr int kBlockBytes = 2048;     // a window's codes (two units)
 
@@ -475,18 +477,18 @@ __device__ __forceinline__ void fetch_window(__amdgpu_buffer_rsrc_t xb, __amdgpu
   if (edge) {
     const int inside = a.width - w * kCols;
 #pragma unroll
-    for (int u = 0; u < 16; u++)
+    for (int u = 0; u < kActivationLoads; u++)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           xb, tile + u * 1024, 16,
           f.col[u & 3] < inside ? f.at[u & 3] + (u >> 2) * f.step : kOutside, w * (kCols * 2), 0, 0);
   } else {
 #pragma unroll
-    for (int u = 0; u < 16; u++)
+    for (int u = 0; u < kActivationLoads; u++)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(xb, tile + u * 1024, 16,
                                                f.at[u & 3] + (u >> 2) * f.step, w * (kCols * 2), 0, 0);
   }
 #pragma unroll
-  for (int j = 0; j < 2; j++)
+  for (int j = 0; j < kCodeLoads; j++)
     __builtin_amdgcn_raw_ptr_buffer_load_lds(ub, block + j * 1024, 16, l.unit_at[j], w * 1024, 0, 0);
 }
 
