@@ -423,9 +423,14 @@ int sub1_matrix_prepared_decode(const sub1_matrix_prepared *prepared, int matrix
  *
  * meta and entries are device buffers the caller owns, 256-byte aligned; the
  * source matrices are not referenced after sub1_tiles_entries has run.  Any
- * dictionary with symbols 0..2; any height and width.  x rows are read 16 bytes
- * at a time when x is 16-byte aligned and ldx a multiple of 8 (else element by
- * element, slower).  sub1_tiles_decode writes one matrix's symbols, read back
+ * dictionary with symbols 0..2; any height and width; up to 65535 * 64 tokens
+ * a launch.  x rows are read 16 bytes at a time when x is 16-byte aligned and
+ * ldx a multiple of 8 (else element by element, slower).  The windows of 128
+ * columns of a matrix are summed in 1, 2 or 4 parts, a number that depends on
+ * the matrix's shape alone: a token's result does not depend on the launch it
+ * is part of, although long launches take another kernel (workgroups of four
+ * wavefronts that share their activations; it also wants y 4-byte aligned, ldy
+ * and the height even).  sub1_tiles_decode writes one matrix's symbols, read back
  * from the tile form, to tern_out (uint8 [height, width]): the check that the
  * copy kept every weight.
  */

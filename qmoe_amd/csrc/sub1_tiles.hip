@@ -1055,12 +1055,8 @@ template <int kRG, int kKP, int kNB>
 int launch_shared_as(const TileArgs &a, int blocks, hipStream_t stream) {
   constexpr int lds = kKP * 2 * kNB * 32 * 256;
   static_assert(lds >= 4 * 32 * kRows * 4 && lds <= 160 * 1024, "tiles, then the sums of four wavefronts");
-  static bool allowed = false;   // (per process: one device kind)
-  if (!allowed) {
-    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_tiles_shared_kernel<kRG, kKP, kNB>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    allowed = true;
-  }
+  HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_tiles_shared_kernel<kRG, kKP, kNB>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds));
   const dim3 grid((blocks + kRG - 1) / kRG, (a.tokens + 32 * kNB - 1) / (32 * kNB));
   matvec_tiles_shared_kernel<kRG, kKP, kNB><<<grid, 256, lds, stream>>>(a);
   HIP_TRY(hipGetLastError());
@@ -1195,8 +1191,8 @@ extern "C" int sub1_matvec_tiles(const sub1_tiles *t, int matrix, const void *x,
   if (rc) return rc;
   if (!x || !y) return fail(SUB1_ERR_NULL, "%s: NULL argument", who);
   if (matrix < 0 || matrix >= t->count) return fail(SUB1_ERR_SHAPE, "%s: no matrix %d", who, matrix);
-  if (tokens < 0 || tokens > (1 << 22))
-    return fail(SUB1_ERR_SHAPE, "%s: tokens %d outside 0..2^22", who, tokens);
+  if (tokens < 0 || tokens > 65535 * kTokens)   // (a grid's second dimension)
+    return fail(SUB1_ERR_SHAPE, "%s: tokens %d outside 0..%d", who, tokens, 65535 * kTokens);
   if (ldx < t->width || ldy < t->height)
     return fail(SUB1_ERR_SHAPE, "%s: token strides smaller than the rows", who);
   if (misaligned(x, 2) || misaligned(y, 2)) return fail(SUB1_ERR_ALIGN, "%s: misaligned pointer", who);
