@@ -472,6 +472,7 @@ struct PreparedArgs {
   int wi_expect;                 // workgroups of a token's wi a wait expects (k[0].parts outside tests)
   int by_ticket;                 // shared-token kernel: a workgroup's place comes from the ticket
   unsigned long long *tagged;    // shared-token kernel: h is handed over by tag (NULL: by count)
+  int lane_parts;                // one-token kernel with wo in workgroups of its own: these share a slice by lanes
   int64_t wait_ticks;            // longest wait between workgroups, ticks of wall_clock64
   int32_t *sticky;               // fault flags in pinned host memory
 };
@@ -1197,7 +1198,8 @@ __device__ __forceinline__ void publish_h(const PreparedArgs &a, int t) {
 template <class Before, class Out>
 __device__ __forceinline__ void walk_tile(const PreparedArgs &a, const KindArgs &k, int64_t first,
                                           int stride, int all, const uint32_t *act,
-                                          float *partials, Before &&before, Out &&out) {
+                                          float *partials, Before &&before, Out &&out,
+                                          bool active = true) {
   const int waves = blockDim.x >> 6;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   int split = 1;
@@ -1233,23 +1235,25 @@ __device__ __forceinline__ void walk_tile(const PreparedArgs &a, const KindArgs 
   Walk<kSplitRing> tail_ahead;
   int tail_ridx = 0xffff;   // the rows of the shared slice, in the wavefront that adds them up
   if (tail_only) {
-    if (sub == 0 && tail_sl < all) tail_ridx = k.row_idx[tail_slice * 64 + (threadIdx.x & 63)];
+    if (sub == 0 && tail_sl < all && active) tail_ridx = k.row_idx[tail_slice * 64 + (threadIdx.x & 63)];
     tail_groups();
-    if (g_lo < g_hi)
+    if (g_lo < g_hi && active)
       tail_ahead = load_slice_described<kSplitRing>(a, k, tail_slice, tail_len, tail_base, g_lo, g_hi);
   }
   int s = slice_of_pass(0, wave, waves, count);
   SliceWalk cur;
   // the first loads of the stream go out before the wait and the staging
-  if (s < count) cur = load_slice(a, k, first + static_cast<int64_t>(s) * stride);
+  if (s < count && active) cur = load_slice(a, k, first + static_cast<int64_t>(s) * stride);
   before();
   for (int pass = 0; s < count; pass++) {
     const int s_next = slice_of_pass(pass + 1, wave, waves, count);
     SliceWalk nxt;
-    if (s_next < count) nxt = load_slice(a, k, first + static_cast<int64_t>(s_next) * stride);
-    const float res = run_slice(cur, a.stream, act, nullptr, pass, passes);
-    out(cur.ridx, res, first + static_cast<int64_t>(s) * stride);
-    if (s_next < count) cur = nxt;
+    if (active) {
+      if (s_next < count) nxt = load_slice(a, k, first + static_cast<int64_t>(s_next) * stride);
+      const float res = run_slice(cur, a.stream, act, nullptr, pass, passes);
+      out(cur.ridx, res, first + static_cast<int64_t>(s) * stride);
+      if (s_next < count) cur = nxt;
+    }
     s = s_next;
   }
   if (split > 1) {
@@ -1257,17 +1261,17 @@ __device__ __forceinline__ void walk_tile(const PreparedArgs &a, const KindArgs 
     const int lane = threadIdx.x & 63;
     float *mine = partials + (wave / split) * k.groups_max * 64;
     if (tail_only) {
-      if (g_lo < g_hi) run_slice(tail_ahead, a.stream, act, mine);
+      if (g_lo < g_hi && active) run_slice(tail_ahead, a.stream, act, mine);
     } else {
-      if (sub == 0 && tail_sl < all) tail_ridx = k.row_idx[tail_slice * 64 + lane];
+      if (sub == 0 && tail_sl < all && active) tail_ridx = k.row_idx[tail_slice * 64 + lane];
       tail_groups();
-      if (g_lo < g_hi) {
+      if (g_lo < g_hi && active) {
         SliceWalk tail = load_slice_described(a, k, tail_slice, tail_len, tail_base, g_lo, g_hi);
         run_slice(tail, a.stream, act, mine);
       }
     }
     __syncthreads();
-    if (sub == 0 && tail_sl < all) {
+    if (sub == 0 && tail_sl < all && active) {
       float sum = 0.f;
       for (int g = 0; g < groups; g++) sum += mine[g * 64 + lane];
       out(tail_ridx, sum, tail_slice);
@@ -1942,24 +1946,27 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_tagged_kernel(Prepar
   if (threadIdx.x == 0) leave_tagged(a.ctrl, gridDim.x);
 }
 
-// The same for shapes whose wo rows are long (the c-2048 shapes): wo has
-// workgroups of its own.  The first k[0].parts of a token's workgroups walk wi
-// (every k[0].parts-th slice from their own) and leave; the other k[1].parts
-// belong to wo and ask for all they need of the stream - the descriptions of
-// their slices, the row indices and every chunk they will walk (a wavefront's
-// share is one group of chunks, which its ring holds) - while wi is still being
-// walked elsewhere.  Between the last row of h and the first row of y then lie
-// the hand-over and a walk whose chunks are in registers already (one token
-// through a c-2048 expert: 13.4 -> 12.4 us, a different expert every launch
-// 14.8 -> 12.9, two tokens 15.4 -> 12.8; the base and large shapes, whose wo rows are shorter, measured
-// 0.5 us slower this way and keep the kernel above).
+// The same with workgroups of its own for wo (one token; two through shapes
+// whose wo rows are long).  The first k[0].parts of a token's workgroups walk wi
+// (every k[0].parts-th slice from their own; they wait for nobody, so there is
+// one per slice where the chip has room) and leave; the others belong to wo and
+// ask for all they need of the stream - the descriptions of their slices, the
+// row indices and every chunk they will walk (a wavefront's share is one group
+// of chunks, which its ring holds) - while wi is still being walked elsewhere.
+// Between the last row of h and the first row of y then lie the hand-over and
+// a walk whose chunks are in registers already.  For one token a.lane_parts = 2
+// workgroups share each slice of wo, 32 lanes (rows) each: the 9 to 14
+// wavefronts of a slice gather from one LDS, which takes 32 lanes a pass.
+// One token through a c-2048 expert: 13.4 -> 11.9 us (a different expert every
+// launch 14.8 -> 12.2), two tokens 15.4 -> 12.8; one token through a base
+// expert 11.5 -> 10.7, a large one 11.7 -> 11.5.
 __global__ __launch_bounds__(kMaxThreads) void moe_prepared_tagged_split_kernel(PreparedArgs a) {
   extern __shared__ __align__(16) uint32_t lds[];
   uint32_t *xa = lds;
   float *partials = reinterpret_cast<float *>(xa + a.xdwords);
   const KindArgs &ki = a.k[0];
   const KindArgs &ko = a.k[1];
-  const int per_token = ki.parts + ko.parts;
+  const int per_token = ki.parts + ko.parts * a.lane_parts;
   const int t = blockIdx.x / per_token;
   const int place = blockIdx.x - t * per_token;
   const bool for_wo = place >= ki.parts;
@@ -1996,7 +2003,11 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_tagged_split_kernel(
                 write_tagged_placed(ht, ridx, where, res, tag);
               });
   } else {
-    const int part = place - ki.parts;
+    // a.lane_parts workgroups share a slice of wo, each with its part of the
+    // lanes (rows): the others do nothing in its walk
+    const int part = (place - ki.parts) / a.lane_parts;
+    const int lanes_of = (place - ki.parts) % a.lane_parts;
+    const bool active = static_cast<int>((threadIdx.x & 63) * a.lane_parts) >> 6 == lanes_of;
     uint16_t *y = a.y + static_cast<int64_t>(t) * a.ldy;
     // (a test that overstates the wait looks for a tag that nobody writes)
     const unsigned long long want = a.wi_expect == ki.parts ? tag : tag + 1;
@@ -2007,7 +2018,7 @@ __global__ __launch_bounds__(kMaxThreads) void moe_prepared_tagged_split_kernel(
                                     ki.row_idx + static_cast<int64_t>(e) * ki.slices * 64,
                                     ki.slices * 64, want, xa);
               },
-              [&](int ridx, float res, int64_t) { write_row(y, ridx, res, kStore); });
+              [&](int ridx, float res, int64_t) { write_row(y, ridx, res, kStore); }, active);
   }
   if (threadIdx.x == 0) leave_tagged(a.ctrl, gridDim.x);
 }
@@ -2484,6 +2495,7 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
   PreparedArgs a;
   a.by_ticket = 0;
   a.tagged = nullptr;
+  a.lane_parts = 1;
   a.stream = static_cast<const uint2 *>(p.codes);
   a.ckpt = reinterpret_cast<const uint16_t *>(a.stream + p.total_chunks * 64);
   a.kinds = p.kinds;
@@ -2734,16 +2746,24 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
     HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(lds_shared)));
     // A token or two: h goes from wi to wo by tag (every workgroup of wo reads
-    // all of it, eight bytes an entry: for small grids only).  Where wo's rows
-    // are long (eight groups of chunks and more: the c-2048 shapes) wo gets
-    // workgroups of its own, as many as give every wavefront at most one group
-    // of chunks, so that all of wo's stream is in registers before h is there.
+    // all of it, eight bytes an entry: for small grids only).  One token, and
+    // two where wo's rows are long (eight groups of chunks and more: the c-2048
+    // shapes), give wo workgroups of its own, as many as give every wavefront at
+    // most one group of chunks, so that all of wo's stream is in registers before
+    // h is there (two tokens through the shorter rows of the base and large
+    // shapes measured 11.4 and 12.4 us that way against 11.5 and 11.8).
     if (tokens <= sub1::kTaggedTokens && 64 * waves == kMaxThreads) {
       const KindArgs &ko = a.k[1];
       const int per_wg = std::max(1, waves / std::max(1, ko.groups_max));
       const int wo_parts = (ko.slices + per_wg - 1) / per_wg;
-      const bool own_wo = ko.groups_max >= 8 &&
-                          static_cast<int64_t>(tokens) * (shared_parts + wo_parts) <= cus;
+      // One token: two workgroups share each slice of wo by lanes, 32 rows each.
+      // The walk of a slice's 9 to 14 wavefronts is bound by the one LDS they
+      // gather from, and a gather of 32 lanes takes the LDS one pass instead of
+      // two (c-2048: 12.3 -> 11.9 us; in four parts, and for two tokens, the
+      // larger grid costs more than the walk gains: 12.6, and 12.9 -> 13.4).
+      const int lane_parts = tokens == 1 ? 2 : 1;
+      const bool own_wo = (tokens == 1 || ko.groups_max >= 8) &&
+                          static_cast<int64_t>(tokens) * (shared_parts + wo_parts * lane_parts) <= cus;
       if (own_wo || static_cast<int64_t>(tokens) * shared_parts <= 64) {
         a.tagged = reinterpret_cast<unsigned long long *>(a.ctrl + sub1::kCtrlTagged);
         const void *tagged_fn =
@@ -2758,12 +2778,13 @@ int launch_prepared(const Prepared &p, const int32_t *token_matrix, const void *
           // that wo leaves a token (one token through a c-2048 expert: 96 instead
           // of 48 workgroups 12.7 -> 12.4 us; two tokens, 63 each instead of 24:
           // 13.8 -> 12.8; with all units taken two tokens measured 13.4)
+          a.lane_parts = lane_parts;
           shared_parts = std::max(shared_parts,
-                                  std::min(a.k[0].slices, (cus / tokens - wo_parts) * 2 / 3));
+                                  std::min(a.k[0].slices, (cus / tokens - wo_parts * lane_parts) * 2 / 3));
           a.k[0].parts = shared_parts;
           a.wi_expect = a.k[0].parts + sub1::expect_extra();
           sub1::note_kernel("moe_prepared_tagged_split_kernel");
-          moe_prepared_tagged_split_kernel<<<tokens * (shared_parts + wo_parts), 64 * waves,
+          moe_prepared_tagged_split_kernel<<<tokens * (shared_parts + wo_parts * lane_parts), 64 * waves,
                                              lds_shared, s>>>(a);
         } else {
           sub1::note_kernel("moe_prepared_tagged_kernel");
