@@ -455,6 +455,15 @@ int sub1_tiles_entries(const sub1_matrix_set *set, const sub1_tiles *tiles, void
 int sub1_matvec_tiles(const sub1_tiles *tiles, int matrix, const void *x, int64_t ldx, void *y,
                       int64_t ldy, int tokens, void *stream);
 
+/*
+ * For tests (no counterpart in the reference): later sub1_matvec_tiles launches
+ * take the kernel named here instead of the one estimated faster, where the
+ * arguments allow it.  0: by estimate; 1: a wavefront with tiles of its own;
+ * 2: workgroups that share their activations, blocks of 64 tokens; 3: the
+ * same, blocks of 128 tokens.  The results must not depend on it.
+ */
+int sub1_test_tiles_kernel(int which);
+
 int sub1_tiles_decode(const sub1_tiles *tiles, int matrix, void *tern_out, void *stream);
 
 /*

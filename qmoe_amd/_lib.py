@@ -118,6 +118,7 @@ PROTOTYPES = {
     'sub1_static_scratch_pointer': (_int, [ctypes.POINTER(ctypes.c_void_p)]),
     'sub1_set_wait_limit_us': (_int, [_i64]),
     'sub1_test_overstate_wait': (_int, [_int]),
+    'sub1_test_tiles_kernel': (_int, [_int]),
     'sub1_unregister_dec': (_int, [_vp]),
 }
 

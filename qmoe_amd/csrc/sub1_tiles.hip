@@ -61,6 +61,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstring>
 #include <type_traits>
@@ -1037,6 +1038,8 @@ double cost_shared_tiles(int blocks, int windows, int n, int64_t tiles) {
 // the matrix alone, never on the tokens of a launch, and the parts are added in
 // the same order by both kernels: a token's result is the same whatever launch
 // it is part of.
+std::atomic<int> g_forced_kernel{0};   // sub1_test_tiles_kernel
+
 int pick_waves(int blocks, int windows) {
   int best = 1;
   double best_cost = 0;
@@ -1226,7 +1229,9 @@ extern "C" int sub1_matvec_tiles(const sub1_tiles *t, int matrix, const void *x,
   // blocks of 64 would make more such workgroups than the chip holds at once.
   const int blocks = l.units_down / 2;
   const int64_t tiles_of_64 = (tokens + kTokens - 1) / kTokens;
-  if (shared_ok && waves <= 2 &&
+  const int forced = g_forced_kernel.load(std::memory_order_relaxed);
+  if (shared_ok && forced >= 2) return launch_shared(a, waves, forced == 3 && waves < 4 ? 4 : 2, blocks, s);
+  if (shared_ok && !forced && waves <= 2 &&
       cost_shared_tiles(blocks, l.windows, waves, tiles_of_64) <
           cost_own_tiles(blocks, l.windows, waves, tiles_of_64)) {
     const int groups = kMaxWaves / waves;
@@ -1239,6 +1244,12 @@ extern "C" int sub1_matvec_tiles(const sub1_tiles *t, int matrix, const void *x,
   else if (waves == 2) launch_tiles<2>(a, wide, grid, s);
   else launch_tiles<4>(a, wide, grid, s);
   HIP_TRY(hipGetLastError());
+  return SUB1_OK;
+}
+
+extern "C" int sub1_test_tiles_kernel(int which) {
+  if (which < 0 || which > 3) return fail(SUB1_ERR_SHAPE, "sub1_test_tiles_kernel: no kernel %d", which);
+  g_forced_kernel.store(which, std::memory_order_relaxed);
   return SUB1_OK;
 }
 

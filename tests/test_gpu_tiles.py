@@ -141,6 +141,45 @@ def test_long_sequences_share_their_activations(gpu, oracle, height, width, p0, 
     assert torch.equal(yw[:, :height], y) and bool((yw[:, height:] == 7.0).all())
 
 
+def test_both_tile_kernels_give_the_same_bits_on_any_shape(gpu, oracle):
+    """Random shapes (blocks of rows that are no multiple of a workgroup's,
+    fewer windows than parts, ragged last windows, a last block of tokens with
+    one token or with 127): the kernel whose workgroups share their activations,
+    with blocks of 64 and of 128 tokens, against the one-wavefront kernel, bit
+    for bit, and every token against the double-precision product."""
+    sub1, op = gpu
+    from qmoe_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(2024)
+    shapes = [(2, 8, 1), (64, 128, 64), (66, 136, 65), (256, 128, 129), (258, 1032, 127), (640, 264, 200)]
+    shapes += [(2 * int(rng.integers(1, 400)), 8 * int(rng.integers(1, 200)), int(rng.integers(1, 330)))
+               for _ in range(14)]
+    try:
+        for n, (height, width, tokens) in enumerate(shapes):
+            c = dev_case(oracle, height, width, float(rng.uniform(0.3, 0.97)), seed=500 + n)
+            tm = op.TiledMatrix(sub1.DEC[0], c['w_comp'], c['row_off_d'], c['mm_d'], width)
+            xs = so.f32_to_bf16_bits(rng.standard_normal((tokens, width)).astype(np.float32))
+            pre = so.f32_to_bf16_bits(rng.standard_normal((tokens, height)).astype(np.float32))
+            xd = bf16_dev(xs)
+            outs = []
+            for which, name in ((1, b'matvec_tiles_kernel'), (2, b'matvec_tiles_shared_kernel<64>'),
+                                (3, None)):
+                _lib.check(lib.sub1_test_tiles_kernel(which))
+                y = bf16_dev(pre).clone()
+                tm.matvec_tokens(xd, y)
+                if name:
+                    assert lib.sub1_last_kernel() == name, (height, width, tokens)
+                else:
+                    assert lib.sub1_last_kernel().startswith(b'matvec_tiles_shared_kernel')
+                outs.append(y)
+            assert torch.equal(outs[0], outs[1]), (height, width, tokens)
+            assert torch.equal(outs[0], outs[2]), (height, width, tokens)
+            check_all_tokens(oracle, c, xs, pre, bits_host(outs[0]))
+    finally:
+        _lib.check(lib.sub1_test_tiles_kernel(0))
+    assert lib.sub1_test_tiles_kernel(4) != 0
+
+
 def test_tiles_closed_forms(gpu, oracle):
     """Unit vectors pick a column exactly; zero activations leave y as it was;
     doubling the activations doubles the product exactly (y zero before)."""
