@@ -565,6 +565,35 @@ def test_one_or_two_tokens_dropped_or_out_of_range(gpu):
         assert torch.equal(y[0], both[0] if e == 1 else x[0]), e
 
 
+def test_one_and_two_tokens_on_random_shapes(gpu, oracle):
+    """One token (wo in workgroups of its own, two to a slice) and two tokens
+    (the same where wo's rows are long, every workgroup in both projections
+    otherwise) through seeded random shapes, among them wo rows of one group
+    of chunks and of more than sixteen, slices that are not full and a single
+    row: every token equal to the oracle to the bit, dropped tokens passed
+    through, and the launches after one another on one workspace."""
+    from qmoe_amd import _lib
+    rng = np.random.default_rng(77)
+    shapes = [(1, 1), (64, 64), (65, 130), (96, 9000), (700, 40), (130, 4096), (2080, 6144)]
+    shapes += [(int(rng.integers(1, 900)), int(rng.integers(1, 7000))) for _ in range(8)]
+    kernels = set()
+    for n, (d_model, d_ff) in enumerate(shapes):
+        p0 = float(rng.choice([0.5, 0.9, 0.97]))
+        stack, wi, wo = small_stack(oracle, 3, d_model, d_ff, p0, seed=7000 + n)
+        prep = stack.prepare()
+        xs = so.f32_to_bf16_bits(rng.standard_normal((2, d_model)).astype(np.float32))
+        for route in ([2], [0, 1], [1], [-1, 2], [1, 1]):
+            x = bf16_dev(xs[:len(route)])
+            y = prep.forward(x, torch.tensor(route, dtype=torch.int32, device='cuda'))
+            kernels.add(_lib.load().sub1_last_kernel())
+            assert prep.launch_faults(len(route)) == (0, 0)
+            got = bits_host(y)
+            for i, e in enumerate(route):
+                want = xs[i] if e < 0 else oracle.expert_ffn(wi[e], wo[e], xs[i], order=2)[0]
+                assert np.array_equal(got[i], want), (d_model, d_ff, p0, route, i)
+    assert {b'moe_prepared_tagged_split_kernel', b'moe_prepared_tagged_kernel'} <= kernels, kernels
+
+
 def test_one_workspace_serves_batches_in_any_order(gpu):
     """A workspace made for the largest batch then serves smaller and larger
     ones in any order: a small launch's h must not land on the words a larger
