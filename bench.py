@@ -657,6 +657,13 @@ def main():
             ab = algorithmic_bytes(st, range(n_e))
             entry = {'us_per_layer': round(us_s, 2), 'algorithmic_bytes': ab,
                      'GBps_cache_resident': round(ab / us_s / 1e3, 1)}
+            # batch 1 on this shape: one token to one expert, and two tokens to two
+            for n_tok in (1, 2):
+                y_few = torch.empty_like(xs[:n_tok])
+                r_few = rt[5:5 + n_tok].contiguous()
+                _, us_few = time_launches(lambda: pr.forward(xs[:n_tok], r_few, y_few), 500, 50,
+                                          stream_ptr)
+                entry['single_token_us' if n_tok == 1 else 'two_tokens_us'] = round(us_few, 2)
             if name == 'large128' and not args.no_dense:
                 entry['dense_bf16_gemv_us_per_layer'] = round(dense_gemv_us(st, xs, n_e) * n_e, 1)
             entry.update(hbm_rate_by_rotation(name, args.seed + 40, stream_ptr))
